@@ -1,0 +1,72 @@
+"""ctypes binding of libwino_amd.so (the C ABI declared in include/wino_amd.h).
+
+The library is the product; there is no fallback: if it is missing, loading
+raises and every operator fails.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libwino_amd.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_u = ctypes.c_uint
+_l = ctypes.c_long
+
+# every symbol include/wino_amd.h declares: name -> (restype, argtypes)
+SYMBOLS = {
+    "wino_conv": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
+    "wino_conv_prepared": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
+    "wino_geometry": (_i, [_i] * 7 + [ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l),
+                                     ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l)]),
+    "wino_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
+    "wino_set_workspace": (_i, [_vp, ctypes.c_size_t]),
+    "wino_filter_transform": (_i, [_i, _i, _i, _i, _vp, _vp, _vp]),
+    "wino_input_transform": (_i, [_i] * 8 + [_vp, _vp, _vp]),
+    "wino_batched_gemm": (_i, [_i, _i, _i, _l, _vp, _vp, _vp, _vp]),
+    "wino_output_transform": (_i, [_i, _i, _i, _u, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "wino_gemm_output": (_i, [_i, _i, _i, _u, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "wino_layout_transform": (_i, [_i] * 7 + [_vp, _vp, _vp]),
+    "wino_warmup": (_i, []),
+    "wino_sync": (_i, [_vp]),
+    "wino_last_error": (ctypes.c_char_p, []),
+    "wino_version": (ctypes.c_char_p, []),
+}
+
+_lib = None
+
+
+def build():
+    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
+    subprocess.check_call(["make", "-s", "-B", "-C", CSRC])
+    return LIB_PATH
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {CSRC}` (there is no non-HIP fallback)")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+class WinoError(RuntimeError):
+    def __init__(self, code, what):
+        msg = load().wino_last_error().decode()
+        super().__init__(f"{what} failed with status {code}: {msg}")
+        self.code = code
+
+
+def check(code, what):
+    if code != 0:
+        raise WinoError(code, what)

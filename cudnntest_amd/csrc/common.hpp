@@ -1,0 +1,103 @@
+// Shared definitions of the gfx950 Winograd F(2x2,3x3) library: layouts, strides,
+// storage-type conversion, padded operand geometry.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/wino_amd.h"
+
+namespace wino {
+
+// element strides of an activation tensor in the order (n, c, h, w)
+struct ActStrides {
+    long n, c, h, w;
+};
+
+__host__ __device__ inline ActStrides act_strides(int layout, long N, long C, long H, long W) {
+    switch (layout) {
+    case WINO_NHWC: return {H * W * C, 1, W * C, C};
+    case WINO_CHWN: return {1, H * W * N, W * N, N};
+    default: return {C * H * W, H * W, W, 1};
+    }
+}
+
+// element strides of a filter bank in the order (k, c, r, s)
+struct FltStrides {
+    long k, c, r, s;
+};
+
+__host__ __device__ inline FltStrides flt_strides(int layout, long K, long C) {
+    switch (layout) {
+    case WINO_NHWC: return {9 * C, 1, 3 * C, C};
+    case WINO_CHWN: return {1, 9 * K, 3 * K, K};
+    default: return {9 * C, 9, 3, 1};
+    }
+}
+
+// ---- storage types ---------------------------------------------------------
+struct bf16_t {
+    uint16_t bits;
+};
+typedef _Float16 f16_t;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(f16_t v) { return (float)v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) { return (f16_t)f; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7f800000u) != 0x7f800000u) u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+    return bf16_t{(uint16_t)(u >> 16)};
+}
+
+__host__ inline size_t dtype_size(int dtype) { return dtype == WINO_F32 ? 4 : 2; }
+
+// ---- padded geometry ---------------------------------------------------------
+constexpr int kCPad = 16;    // reduction (channel) dimension of U and V is padded to this
+constexpr int kKPad = 128;   // filter dimension of U / Mo
+constexpr int kPPad = 128;   // tile dimension of V / Mo
+
+struct Geometry {
+    int N, C, K, H, W, pad;
+    int Ho, Wo, th, tw;
+    long P;
+    int Cp, Kp;
+    long Pp;
+};
+
+__host__ inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
+
+__host__ inline bool make_geometry(int N, int C, int K, int H, int W, int pad, Geometry* g) {
+    if (N <= 0 || C <= 0 || K <= 0 || H <= 0 || W <= 0 || pad < 0 || pad > 1) return false;
+    g->N = N; g->C = C; g->K = K; g->H = H; g->W = W; g->pad = pad;
+    g->Ho = H + 2 * pad - 2;
+    g->Wo = W + 2 * pad - 2;
+    if (g->Ho <= 0 || g->Wo <= 0) return false;
+    g->th = (g->Ho + 1) / 2;
+    g->tw = (g->Wo + 1) / 2;
+    g->P = (long)N * g->th * g->tw;
+    g->Cp = (int)round_up(C, kCPad);
+    g->Kp = (int)round_up(K, kKPad);
+    g->Pp = round_up(g->P, kPPad);
+    return true;
+}
+
+// tile index -> (n, ty, tx)
+__device__ __forceinline__ void decode_tile(long p, int order, int N, int th, int tw, int& n, int& ty, int& tx) {
+    if (order == WINO_TILES_BATCH_MAJOR) {
+        tx = (int)(p % tw);
+        long q = p / tw;
+        ty = (int)(q % th);
+        n = (int)(q / th);
+    } else {
+        n = (int)(p % N);
+        long q = p / N;
+        tx = (int)(q % tw);
+        ty = (int)(q / tw);
+    }
+}
+
+}  // namespace wino

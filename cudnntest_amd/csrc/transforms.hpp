@@ -1,0 +1,186 @@
+// Winograd F(2x2,3x3) transform kernels: U = G g G^T, V = B^T d B, y = A^T Mo A.
+// All three are HBM-bandwidth bound; arithmetic is fp32 whatever the storage type.
+//
+//   B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
+//   G   = [1 0 0; 1/2 1/2 1/2; 1/2 -1/2 1/2; 0 0 1]
+//   A^T = [1 1 1 0; 0 1 -1 -1]
+#pragma once
+#include "common.hpp"
+
+namespace wino {
+
+// ---- register-level 1-D transforms ------------------------------------------
+__device__ __forceinline__ void bt4(float d0, float d1, float d2, float d3, float& o0, float& o1, float& o2,
+                                    float& o3) {
+    o0 = d0 - d2;
+    o1 = d1 + d2;
+    o2 = d2 - d1;
+    o3 = d1 - d3;
+}
+
+// v[i][j] (4x4) = B^T d B, rows first then columns
+__device__ __forceinline__ void input_tile_transform(const float d[4][4], float v[4][4]) {
+    float t[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bt4(d[0][j], d[1][j], d[2][j], d[3][j], t[0][j], t[1][j], t[2][j], t[3][j]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bt4(t[i][0], t[i][1], t[i][2], t[i][3], v[i][0], v[i][1], v[i][2], v[i][3]);
+}
+
+// u (4x4) = G g G^T
+__device__ __forceinline__ void filter_tile_transform(const float g[3][3], float u[4][4]) {
+    float t[4][3];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+        t[0][s] = g[0][s];
+        t[1][s] = 0.5f * (g[0][s] + g[1][s] + g[2][s]);
+        t[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
+        t[3][s] = g[2][s];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        u[i][0] = t[i][0];
+        u[i][1] = 0.5f * (t[i][0] + t[i][1] + t[i][2]);
+        u[i][2] = 0.5f * (t[i][0] - t[i][1] + t[i][2]);
+        u[i][3] = t[i][2];
+    }
+}
+
+// y (2x2) = A^T m A
+__device__ __forceinline__ void output_tile_transform(const float m[16], float& y00, float& y01, float& y10,
+                                                      float& y11) {
+    float r0[4], r1[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        r0[j] = m[j] + m[4 + j] + m[8 + j];
+        r1[j] = m[4 + j] - m[8 + j] - m[12 + j];
+    }
+    y00 = r0[0] + r0[1] + r0[2];
+    y01 = r0[1] - r0[2] - r0[3];
+    y10 = r1[0] + r1[1] + r1[2];
+    y11 = r1[1] - r1[2] - r1[3];
+}
+
+// ---- filter transform ---------------------------------------------------------
+// One thread per (k, c), k fastest so the 16 stores of a wave are contiguous.
+// Grid covers the padded Cp x Kp rectangle: the padding is written as zeros,
+// which is what lets the GEMM run without masks on the reduction dimension.
+template <typename T>
+__global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restrict__ w, T* __restrict__ U,
+                                                                FltStrides s, int K, int C, int Kp, int Cp) {
+    int k = blockIdx.x * blockDim.x + threadIdx.x;
+    int c = blockIdx.y;
+    if (k >= Kp) return;
+    float u[4][4];
+    if (k < K && c < C) {
+        float g[3][3];
+        const T* wp = w + k * s.k + c * s.c;
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
+        filter_tile_transform(g, u);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) u[i / 4][i % 4] = 0.f;
+    }
+    const size_t plane = (size_t)Cp * Kp;
+    T* up = U + (size_t)c * Kp + k;
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) up[xi * plane] = from_f32<T>(u[xi / 4][xi % 4]);
+}
+
+// ---- input transform, layout-generic ---------------------------------------------
+// One thread per (tile p, channel c), p fastest: the 16 stores of a wave are
+// contiguous runs of V.  Reads go through the activation strides, so the kernel
+// is correct for every layout and tile order; it is the fast path when the
+// source's contiguous axis runs along p (CHWN with batch-minor tiles) and the
+// fallback elsewhere.
+template <typename T>
+__global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* __restrict__ x, T* __restrict__ V,
+                                                                       ActStrides s, int N, int C, int H, int W,
+                                                                       int pad, int th, int tw, long P, long Pp,
+                                                                       int Cp, int order) {
+    long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    int c = blockIdx.y;
+    if (p >= P) return;
+    float v[4][4];
+    if (c < C) {
+        int n, ty, tx;
+        decode_tile(p, order, N, th, tw, n, ty, tx);
+        const int h0 = 2 * ty - pad, w0 = 2 * tx - pad;
+        const T* xp = x + n * s.n + c * s.c;
+        float d[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int ih = h0 + i, iw = w0 + j;
+                bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
+                d[i][j] = ok ? to_f32(xp[ih * s.h + iw * s.w]) : 0.f;
+            }
+        input_tile_transform(d, v);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i / 4][i % 4] = 0.f;
+    }
+    const size_t plane = (size_t)Cp * Pp;
+    T* vp = V + (size_t)c * Pp + p;
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) vp[xi * plane] = from_f32<T>(v[xi / 4][xi % 4]);
+}
+
+// ---- output transform, layout-generic ---------------------------------------------
+// One thread per (tile p, filter k), p fastest: the 16 loads of a wave are
+// contiguous runs of Mo.  Stores go through the destination strides.
+template <typename T>
+__global__ __launch_bounds__(256) void output_transform_generic_kernel(const float* __restrict__ Mo,
+                                                                        T* __restrict__ y, ActStrides s, int N,
+                                                                        int K, int Ho, int Wo, int th, int tw,
+                                                                        long P, long Pp, int Kp, int order,
+                                                                        int relu) {
+    long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    int k = blockIdx.y;
+    if (p >= P || k >= K) return;
+    const size_t plane = (size_t)Kp * Pp;
+    const float* mp = Mo + (size_t)k * Pp + p;
+    float m[16];
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];
+    float o[2][2];
+    output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    T* yp = y + n * s.n + k * s.c;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            int oh = 2 * ty + a, ow = 2 * tx + b;
+            if (oh < Ho && ow < Wo) {
+                float val = o[a][b];
+                if (relu) val = fmaxf(val, 0.f);
+                yp[oh * s.h + ow * s.w] = from_f32<T>(val);
+            }
+        }
+}
+
+// ---- plain layout permutation -------------------------------------------------------
+// Walks the destination linearly (coalesced stores) and gathers from the source.
+template <typename T>
+__global__ __launch_bounds__(256) void permute_gather_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                                              ActStrides a, int dst_layout, int N, int C, int H,
+                                                              int W) {
+    const long total = (long)N * C * H * W;
+    long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    long n, c, h, w, r;
+    switch (dst_layout) {
+    case WINO_NHWC: c = e % C; r = e / C; w = r % W; r /= W; h = r % H; n = r / H; break;
+    case WINO_CHWN: n = e % N; r = e / N; w = r % W; r /= W; h = r % H; c = r / H; break;
+    default: w = e % W; r = e / W; h = r % H; r /= H; c = r % C; n = r / C; break;
+    }
+    out[e] = in[n * a.n + c * a.c + h * a.h + w * a.w];
+}
+
+}  // namespace wino

@@ -1,0 +1,318 @@
+// C ABI of the gfx950 Winograd F(2x2,3x3) convolution library (see include/wino_amd.h).
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+
+#include "common.hpp"
+#include "gemm.hpp"
+#include "transforms.hpp"
+
+using namespace wino;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                            \
+    do {                                                                                         \
+        hipError_t e_ = (expr);                                                                  \
+        if (e_ != hipSuccess) return fail(WINO_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+#define LAUNCH_CHECK(name)                                                                        \
+    do {                                                                                          \
+        hipError_t e_ = hipGetLastError();                                                        \
+        if (e_ != hipSuccess) return fail(WINO_ERR_HIP, "launch %s: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+bool valid_layout(int l) { return l == WINO_NCHW || l == WINO_NHWC || l == WINO_CHWN; }
+bool valid_dtype(int d) { return d == WINO_F32 || d == WINO_F16 || d == WINO_BF16; }
+bool valid_order(int o) { return o == WINO_TILES_BATCH_MAJOR || o == WINO_TILES_BATCH_MINOR; }
+
+// ---- scratch arena: one grow-only allocation per device ------------------------
+constexpr int kMaxDevices = 16;
+struct Arena {
+    void* own = nullptr;
+    size_t own_bytes = 0;
+    void* ext = nullptr;
+    size_t ext_bytes = 0;
+};
+Arena g_arena[kMaxDevices];
+std::mutex g_arena_mu;
+
+int arena_get(size_t bytes, void** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(WINO_ERR_UNSUPPORTED, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_arena_mu);
+    Arena& a = g_arena[dev];
+    if (a.ext) {
+        if (a.ext_bytes < bytes)
+            return fail(WINO_ERR_WORKSPACE, "workspace of %zu bytes installed, %zu needed", a.ext_bytes, bytes);
+        *out = a.ext;
+        return WINO_OK;
+    }
+    if (a.own_bytes < bytes) {
+        if (a.own) {
+            HIP_TRY(hipDeviceSynchronize());
+            HIP_TRY(hipFree(a.own));
+            a.own = nullptr;
+            a.own_bytes = 0;
+        }
+        HIP_TRY(hipMalloc(&a.own, bytes));
+        a.own_bytes = bytes;
+    }
+    *out = a.own;
+    return WINO_OK;
+}
+
+struct Scratch {
+    size_t u_off, v_off, m_off, total;
+};
+
+Scratch scratch_layout(const Geometry& g, int dtype) {
+    const size_t es = dtype_size(dtype);
+    auto al = [](size_t v) { return (v + 255) / 256 * 256; };
+    Scratch s;
+    s.u_off = 0;
+    s.v_off = al(16 * (size_t)g.Cp * g.Kp * es);
+    s.m_off = s.v_off + al(16 * (size_t)g.Cp * g.Pp * es);
+    s.total = s.m_off + al(16 * (size_t)g.Kp * g.Pp * sizeof(float));
+    return s;
+}
+
+// ---- stage launchers (typed) -------------------------------------------------------
+template <typename T>
+int launch_filter_transform(int layout, int K, int C, int Kp, int Cp, const void* w, void* U, hipStream_t st) {
+    dim3 grid((Kp + 255) / 256, Cp), block(256);
+    hipLaunchKernelGGL(filter_transform_kernel<T>, grid, block, 0, st, (const T*)w, (T*)U, flt_strides(layout, K, C),
+                       K, C, Kp, Cp);
+    LAUNCH_CHECK("filter_transform");
+    return WINO_OK;
+}
+
+template <typename T>
+int launch_input_transform(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st) {
+    dim3 grid((unsigned)((g.P + 255) / 256), g.Cp), block(256);
+    hipLaunchKernelGGL(input_transform_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
+                       act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
+                       g.Cp, order);
+    LAUNCH_CHECK("input_transform");
+    return WINO_OK;
+}
+
+template <typename T>
+int launch_output_transform(int layout, int order, unsigned flags, int N, int K, int Ho, int Wo, int Kp, long P,
+                            long Pp, const float* Mo, void* y, hipStream_t st) {
+    const int th = (Ho + 1) / 2, tw = (Wo + 1) / 2;
+    dim3 grid((unsigned)((P + 255) / 256), K), block(256);
+    hipLaunchKernelGGL(output_transform_generic_kernel<T>, grid, block, 0, st, Mo, (T*)y,
+                       act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order,
+                       (flags & WINO_FLAG_RELU) ? 1 : 0);
+    LAUNCH_CHECK("output_transform");
+    return WINO_OK;
+}
+
+int launch_gemm(int dtype, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
+    if (dtype != WINO_F32) return fail(WINO_ERR_UNSUPPORTED, "batched GEMM: dtype %d not built yet", dtype);
+    dim3 grid((unsigned)(Pp / GEMM_BN), Kp / GEMM_BM, 16), block(256);
+    hipLaunchKernelGGL(gemm_f32_128x128_kernel, grid, block, 0, st, (const float*)U, (const float*)V, Mo, Cp, Kp, Pp);
+    LAUNCH_CHECK("batched_gemm");
+    return WINO_OK;
+}
+
+#define DISPATCH_DTYPE(dtype, CALL)                          \
+    switch (dtype) {                                         \
+    case WINO_F32: { typedef float T; return CALL; }         \
+    case WINO_F16: { typedef f16_t T; return CALL; }         \
+    case WINO_BF16: { typedef bf16_t T; return CALL; }       \
+    default: return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype); \
+    }
+
+int tile_order_for(int src, int dst) {
+    // batch-minor tiles keep both the CHWN reads and the CHWN writes contiguous
+    if (src == WINO_CHWN) return WINO_TILES_BATCH_MINOR;
+    if (dst == WINO_CHWN && src != WINO_NHWC) return WINO_TILES_BATCH_MAJOR;
+    return WINO_TILES_BATCH_MAJOR;
+}
+
+int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
+              const void* x, const void* w, const void* Upre, void* y, void* stream) {
+    if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_FUSED) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
+    if (!x || (!w && !Upre) || !y) return fail(WINO_ERR_INVALID, "null tensor pointer");
+    Geometry g;
+    if (!make_geometry(N, C, K, H, W, pad, &g))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
+    if (algo == WINO_ALGO_AUTO) algo = WINO_ALGO_STAGED;
+    if (algo != WINO_ALGO_STAGED) return fail(WINO_ERR_UNSUPPORTED, "algo %d not built yet", algo);
+
+    hipStream_t st = (hipStream_t)stream;
+    const Scratch sc = scratch_layout(g, dtype);
+    void* base = nullptr;
+    int rc = arena_get(sc.total, &base);
+    if (rc) return rc;
+    char* b = (char*)base;
+    void* U = b + sc.u_off;
+    void* V = b + sc.v_off;
+    float* Mo = (float*)(b + sc.m_off);
+    const int order = tile_order_for(src, dst);
+
+    if (Upre) {
+        U = const_cast<void*>(Upre);
+    } else {
+        rc = wino_filter_transform(src, dtype, K, C, w, U, stream);
+        if (rc) return rc;
+    }
+    rc = wino_input_transform(src, dtype, order, N, C, H, W, pad, x, V, stream);
+    if (rc) return rc;
+    rc = launch_gemm(dtype, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
+    if (rc) return rc;
+    return wino_output_transform(dst, dtype, order, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
+}
+
+__global__ void warmup_kernel() {}
+
+}  // namespace
+
+extern "C" {
+
+int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
+              const void* x, const void* w, void* y, void* stream) {
+    if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
+    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, y, stream);
+}
+
+int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W,
+                       int pad, const void* x, const void* U, void* y, void* stream) {
+    if (!U) return fail(WINO_ERR_INVALID, "null transformed-filter pointer");
+    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, y, stream);
+}
+
+int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp, int* Kp,
+                  long* Pp) {
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    Geometry g;
+    if (!make_geometry(N, C, K, H, W, pad, &g))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
+    if (th) *th = g.th;
+    if (tw) *tw = g.tw;
+    if (P) *P = g.P;
+    if (Cp) *Cp = g.Cp;
+    if (Kp) *Kp = g.Kp;
+    if (Pp) *Pp = g.Pp;
+    return WINO_OK;
+}
+
+size_t wino_workspace_bytes(int dtype, int N, int C, int K, int H, int W, int pad) {
+    Geometry g;
+    if (!valid_dtype(dtype) || !make_geometry(N, C, K, H, W, pad, &g)) {
+        fail(WINO_ERR_INVALID, "bad shape or dtype");
+        return 0;
+    }
+    return scratch_layout(g, dtype).total;
+}
+
+int wino_set_workspace(void* ptr, size_t bytes) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(WINO_ERR_UNSUPPORTED, "device index %d out of range", dev);
+    if (ptr && bytes == 0) return fail(WINO_ERR_INVALID, "workspace pointer with zero size");
+    std::lock_guard<std::mutex> lk(g_arena_mu);
+    g_arena[dev].ext = ptr;
+    g_arena[dev].ext_bytes = ptr ? bytes : 0;
+    return WINO_OK;
+}
+
+int wino_filter_transform(int layout, int dtype, int K, int C, const void* w, void* U, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!w || !U) return fail(WINO_ERR_INVALID, "null pointer");
+    if (K <= 0 || C <= 0) return fail(WINO_ERR_INVALID, "bad filter bank K=%d C=%d", K, C);
+    const int Kp = (int)round_up(K, kKPad), Cp = (int)round_up(C, kCPad);
+    DISPATCH_DTYPE(dtype, launch_filter_transform<T>(layout, K, C, Kp, Cp, w, U, (hipStream_t)stream));
+}
+
+int wino_input_transform(int layout, int dtype, int tile_order, int N, int C, int H, int W, int pad, const void* x,
+                         void* V, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
+    if (!x || !V) return fail(WINO_ERR_INVALID, "null pointer");
+    Geometry g;
+    if (!make_geometry(N, C, 1, H, W, pad, &g))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d H=%d W=%d pad=%d", N, C, H, W, pad);
+    DISPATCH_DTYPE(dtype, launch_input_transform<T>(layout, tile_order, g, x, V, (hipStream_t)stream));
+}
+
+int wino_batched_gemm(int dtype, int C, int K, long P, const void* U, const void* V, float* Mo, void* stream) {
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
+    if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
+    return launch_gemm(dtype, (int)round_up(C, kCPad), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
+                       (hipStream_t)stream);
+}
+
+int wino_output_transform(int layout, int dtype, int tile_order, unsigned flags, int N, int K, int Ho, int Wo,
+                          const float* Mo, void* y, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
+    if (!Mo || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    if (N <= 0 || K <= 0 || Ho <= 0 || Wo <= 0)
+        return fail(WINO_ERR_INVALID, "bad shape N=%d K=%d Ho=%d Wo=%d", N, K, Ho, Wo);
+    const long P = (long)N * ((Ho + 1) / 2) * ((Wo + 1) / 2);
+    const int Kp = (int)round_up(K, kKPad);
+    const long Pp = round_up(P, kPPad);
+    DISPATCH_DTYPE(dtype, launch_output_transform<T>(layout, tile_order, flags, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
+                                                     (hipStream_t)stream));
+}
+
+int wino_gemm_output(int, int, int, unsigned, int, int, int, int, int, const void*, const void*, void*, void*) {
+    return fail(WINO_ERR_UNSUPPORTED, "epilogue-fused GEMM not built yet");
+}
+
+int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void* in, void* out,
+                          void* stream) {
+    if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!in || !out) return fail(WINO_ERR_INVALID, "null pointer");
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0) return fail(WINO_ERR_INVALID, "bad shape");
+    const long total = (long)N * C * H * W;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    const ActStrides a = act_strides(src, N, C, H, W);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == WINO_F32)
+        hipLaunchKernelGGL(permute_gather_kernel<float>, grid, block, 0, st, (const float*)in, (float*)out, a, dst, N,
+                           C, H, W);
+    else
+        hipLaunchKernelGGL(permute_gather_kernel<uint16_t>, grid, block, 0, st, (const uint16_t*)in, (uint16_t*)out,
+                           a, dst, N, C, H, W);
+    LAUNCH_CHECK("layout_transform");
+    return WINO_OK;
+}
+
+int wino_warmup(void) {
+    hipLaunchKernelGGL(warmup_kernel, dim3(1), dim3(1), 0, 0);
+    LAUNCH_CHECK("warmup");
+    return WINO_OK;
+}
+
+int wino_sync(void* stream) {
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return WINO_OK;
+}
+
+const char* wino_last_error(void) { return g_err; }
+
+const char* wino_version(void) { return "wino_amd 0.1 (gfx950, F(2x2,3x3))"; }
+
+}  // extern "C"

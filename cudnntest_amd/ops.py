@@ -1,0 +1,220 @@
+"""Operators over libwino_amd.so.
+
+Two levels:
+  * the reference's names -- wrapedConv_NCHW / _NHWC / _CHWN
+    (comparison/wrapedConv_NCHW.cuh:335, wrapedConv_NHWC.cuh:24,
+    wrapedConv_CHWN.cuh:16), the six convLayoutTrans_X_to_Y and layoutManager
+    with DataLayout (comparison/DataLayoutTrans.cuh:9-651) -- same argument
+    order and meaning: (bat4Conv, inside, chn, numOfFilter, padding, m1, m2,
+    inputTran_gpu, filterTran_gpu, gemmOutput_gpu, output).  They are blocking,
+    like the reference's (each ends in a device sync).  `chn` is a C++ int&
+    there, overwritten with numOfFilter; here the new value is returned.  The
+    three scratch arguments are accepted and ignored: the library owns its
+    scratch, because F(2x2) intermediates are larger than the F(4x4) buffers a
+    reference caller allocates.
+  * stage-level and whole-layer functions that take torch tensors and derive
+    sizes from them.
+"""
+import enum
+
+import torch
+
+from . import _lib
+
+NCHW, NHWC, CHWN = 0, 1, 2
+F32, F16, BF16 = 0, 1, 2
+ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED = 0, 1, 2, 3
+TILES_BATCH_MAJOR, TILES_BATCH_MINOR = 0, 1
+FLAG_RELU = 1
+
+
+class DataLayout(enum.IntEnum):
+    NCHW = 0
+    NHWC = 1
+    CHWN = 2
+
+
+_DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+_TORCH_DTYPES = {v: k for k, v in _DTYPES.items()}
+
+
+def _dt(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}") from None
+
+
+def _ptr(t):
+    if not t.is_cuda:
+        raise ValueError("tensor must live on the GPU")
+    if not t.is_contiguous():
+        raise ValueError("tensor must be contiguous in its layout's memory order")
+    return t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def act_shape(layout, N, C, H, W):
+    return {NCHW: (N, C, H, W), NHWC: (N, H, W, C), CHWN: (C, H, W, N)}[int(layout)]
+
+
+def act_dims(layout, t):
+    s = t.shape
+    return {NCHW: (s[0], s[1], s[2], s[3]), NHWC: (s[0], s[3], s[1], s[2]),
+            CHWN: (s[3], s[0], s[1], s[2])}[int(layout)]
+
+
+def flt_dims(layout, w):
+    s = w.shape
+    return {NCHW: (s[0], s[1]), NHWC: (s[0], s[3]), CHWN: (s[3], s[0])}[int(layout)]
+
+
+def geometry(dtype, N, C, K, H, W, pad):
+    import ctypes
+    th, tw, Cp, Kp = (ctypes.c_int() for _ in range(4))
+    P, Pp = ctypes.c_long(), ctypes.c_long()
+    _lib.check(_lib.load().wino_geometry(dtype, N, C, K, H, W, pad, th, tw, P, Cp, Kp, Pp), "wino_geometry")
+    return dict(th=th.value, tw=tw.value, P=P.value, Cp=Cp.value, Kp=Kp.value, Pp=Pp.value)
+
+
+def workspace_bytes(dtype, N, C, K, H, W, pad):
+    return int(_lib.load().wino_workspace_bytes(dtype, N, C, K, H, W, pad))
+
+
+def warmup():
+    _lib.check(_lib.load().wino_warmup(), "wino_warmup")
+
+
+# ---- whole layer -------------------------------------------------------------
+
+def conv(x, w, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None):
+    """y = conv3x3(x, w); x, w in `src`'s conventions, y in `dst`'s.  Asynchronous."""
+    dst = src if dst is None else dst
+    N, C, H, W = act_dims(src, x)
+    K, C2 = flt_dims(src, w)
+    if C2 != C:
+        raise ValueError(f"filter bank has {C2} channels, input has {C}")
+    if w.dtype != x.dtype:
+        raise TypeError("x and w must share a dtype")
+    if out is None:
+        out = torch.empty(act_shape(dst, N, K, H + 2 * pad - 2, W + 2 * pad - 2), dtype=x.dtype, device=x.device)
+    rc = _lib.load().wino_conv(int(src), int(dst), _dt(x), algo, FLAG_RELU if relu else 0, N, C, K, H, W, pad,
+                               _ptr(x), _ptr(w), _ptr(out), _stream())
+    _lib.check(rc, "wino_conv")
+    return out
+
+
+def conv_prepared(x, U, K, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None):
+    """Same with the filter bank already transformed by filter_transform()."""
+    dst = src if dst is None else dst
+    N, C, H, W = act_dims(src, x)
+    if out is None:
+        out = torch.empty(act_shape(dst, N, K, H + 2 * pad - 2, W + 2 * pad - 2), dtype=x.dtype, device=x.device)
+    rc = _lib.load().wino_conv_prepared(int(src), int(dst), _dt(x), algo, FLAG_RELU if relu else 0, N, C, K, H, W,
+                                        pad, _ptr(x), _ptr(U), _ptr(out), _stream())
+    _lib.check(rc, "wino_conv_prepared")
+    return out
+
+
+# ---- stages ------------------------------------------------------------------------
+
+def filter_transform(w, layout=NCHW):
+    """U[16][Cp][Kp] = G g G^T (padding zero-filled)."""
+    K, C = flt_dims(layout, w)
+    g = geometry(_dt(w), 1, C, K, 4, 4, 1)
+    U = torch.empty((16, g["Cp"], g["Kp"]), dtype=w.dtype, device=w.device)
+    _lib.check(_lib.load().wino_filter_transform(int(layout), _dt(w), K, C, _ptr(w), _ptr(U), _stream()),
+               "wino_filter_transform")
+    return U
+
+
+def input_transform(x, pad=1, layout=NCHW, tile_order=TILES_BATCH_MAJOR):
+    """V[16][Cp][Pp] = B^T d B; columns p >= P are left as allocated (zeros here)."""
+    N, C, H, W = act_dims(layout, x)
+    g = geometry(_dt(x), N, C, 1, H, W, pad)
+    V = torch.zeros((16, g["Cp"], g["Pp"]), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().wino_input_transform(int(layout), _dt(x), tile_order, N, C, H, W, pad, _ptr(x), _ptr(V),
+                                                _stream()), "wino_input_transform")
+    return V
+
+
+def batched_gemm(U, V, C, K, P):
+    """Mo[16][Kp][Pp] (fp32) = sum_c U[xi][c][k] V[xi][c][p]."""
+    Mo = torch.empty((16, U.shape[2], V.shape[2]), dtype=torch.float32, device=U.device)
+    _lib.check(_lib.load().wino_batched_gemm(_dt(U), C, K, P, _ptr(U), _ptr(V), _ptr(Mo), _stream()),
+               "wino_batched_gemm")
+    return Mo
+
+
+def output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False, dtype=torch.float32):
+    y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=dtype, device=Mo.device)
+    _lib.check(_lib.load().wino_output_transform(int(layout), _DTYPES[dtype], tile_order, FLAG_RELU if relu else 0,
+                                                 N, K, Ho, Wo, _ptr(Mo), _ptr(y), _stream()),
+               "wino_output_transform")
+    return y
+
+
+def gemm_output(U, V, N, C, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False):
+    y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=U.dtype, device=U.device)
+    _lib.check(_lib.load().wino_gemm_output(int(layout), _dt(U), tile_order, FLAG_RELU if relu else 0, N, C, K, Ho,
+                                            Wo, _ptr(U), _ptr(V), _ptr(y), _stream()), "wino_gemm_output")
+    return y
+
+
+def layout_transform(t, src, dst):
+    N, C, H, W = act_dims(src, t)
+    out = torch.empty(act_shape(dst, N, C, H, W), dtype=t.dtype, device=t.device)
+    _lib.check(_lib.load().wino_layout_transform(int(src), int(dst), _dt(t), N, C, H, W, _ptr(t), _ptr(out),
+                                                 _stream()), "wino_layout_transform")
+    return out
+
+
+# ---- the reference's call surface --------------------------------------------------------
+
+def _wrapped(src, dst, bat4Conv, inside, chn, numOfFilter, padding, m1, m2, output):
+    L = _lib.load()
+    rc = L.wino_conv(int(src), int(dst), _dt(m1), ALGO_AUTO, 0, bat4Conv, chn, numOfFilter, inside, inside, padding,
+                     _ptr(m1), _ptr(m2), _ptr(output), _stream())
+    _lib.check(rc, "wino_conv")
+    _lib.check(L.wino_sync(_stream()), "wino_sync")
+    return numOfFilter
+
+
+def wrapedConv_NCHW(bat4Conv, inside, chn, numOfFilter, padding, m1, m2, inputTran_gpu, filterTran_gpu,
+                    gemmOutput_gpu, output):
+    return _wrapped(NCHW, NCHW, bat4Conv, inside, chn, numOfFilter, padding, m1, m2, output)
+
+
+def wrapedConv_NHWC(bat4Conv, inside, chn, numOfFilter, padding, m1, m2, inputTran_gpu, filterTran_gpu,
+                    gemmOutput_gpu, output):
+    return _wrapped(NHWC, NHWC, bat4Conv, inside, chn, numOfFilter, padding, m1, m2, output)
+
+
+def wrapedConv_CHWN(bat4Conv, inside, chn, numOfFilter, padding, m1, m2, inputTran_gpu, filterTran_gpu,
+                    gemmOutput_gpu, output):
+    return _wrapped(CHWN, CHWN, bat4Conv, inside, chn, numOfFilter, padding, m1, m2, output)
+
+
+def _make_cross(src, dst):
+    def f(bat4Conv, inside, chn, numOfFilter, padding, m1, m2, inputTran_gpu, filterTran_gpu, gemmOutput_gpu,
+          output):
+        return _wrapped(src, dst, bat4Conv, inside, chn, numOfFilter, padding, m1, m2, output)
+    return f
+
+
+convLayoutTrans_CHWN_to_NCHW = _make_cross(CHWN, NCHW)
+convLayoutTrans_CHWN_to_NHWC = _make_cross(CHWN, NHWC)
+convLayoutTrans_NHWC_to_NCHW = _make_cross(NHWC, NCHW)
+convLayoutTrans_NHWC_to_CHWN = _make_cross(NHWC, CHWN)
+convLayoutTrans_NCHW_to_NHWC = _make_cross(NCHW, NHWC)
+convLayoutTrans_NCHW_to_CHWN = _make_cross(NCHW, CHWN)
+
+
+def layoutManager(srcLayout, dstLayout, bat4Conv, inside, chn, numOfFilter, padding, input, weights, inputTran_gpu,
+                  filterTran_gpu, gemmOutput_gpu, output):
+    """Dispatch on (src, dst) as comparison/DataLayoutTrans.cuh:594-651 does."""
+    return _wrapped(DataLayout(srcLayout), DataLayout(dstLayout), bat4Conv, inside, chn, numOfFilter, padding,
+                    input, weights, output)

@@ -1,0 +1,133 @@
+/*
+ * wino_amd.h -- C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) convolution library.
+ *
+ * Every entry point takes plain device pointers and sizes; `stream` is a
+ * hipStream_t passed as void* (NULL = the null stream).  Calls are asynchronous
+ * on that stream unless stated otherwise.  Return value: 0 on success, a
+ * negative wino_status_t otherwise; wino_last_error() gives the text of the
+ * calling thread's last failure.
+ *
+ * Tensor conventions (those of the reference's three wrappers):
+ *   layout   activations x / y           3x3 filter bank w
+ *   NCHW     [N][C][H][W]                [K][C][3][3]   comparison/wrapedConv_NCHW.cuh:869
+ *   NHWC     [N][H][W][C]                [K][3][3][C]   comparison/wrapedConv_NHWC.cuh:341
+ *   CHWN     [C][H][W][N]                [C][3][3][K]   comparison/wrapedConv_CHWN.cuh:288
+ * The convolution is a stride-1 cross-correlation with `pad` rows/columns of
+ * zeros on every side; the output is Ho x Wo = (H+2*pad-2) x (W+2*pad-2).
+ */
+#ifndef WINO_AMD_H
+#define WINO_AMD_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* same order as `enum class DataLayout` (comparison/DataLayoutTrans.cuh:587-591) */
+typedef enum { WINO_NCHW = 0, WINO_NHWC = 1, WINO_CHWN = 2 } wino_layout_t;
+
+/* storage type of x, w, y and of the transformed operands; accumulation is always fp32 */
+typedef enum { WINO_F32 = 0, WINO_F16 = 1, WINO_BF16 = 2 } wino_dtype_t;
+
+typedef enum {
+    WINO_ALGO_AUTO = 0,     /* library picks per shape */
+    WINO_ALGO_STAGED = 1,   /* four kernels: input/filter transform, 16-way GEMM, output transform
+                               (the pipeline of comparison/wrapedConv_NCHW.cuh:408-452) */
+    WINO_ALGO_EPILOGUE = 2, /* output transform applied in the GEMM epilogue (no product tensor in HBM) */
+    WINO_ALGO_FUSED = 3     /* one kernel: input transform, multiply-accumulate and output transform
+                               (the structure of fusedTest/winotrans.cuh:1452 Winofuse4433) */
+} wino_algo_t;
+
+/* order of the tile index p inside the transformed operands */
+typedef enum {
+    WINO_TILES_BATCH_MAJOR = 0, /* p = (n*th + ty)*tw + tx */
+    WINO_TILES_BATCH_MINOR = 1  /* p = (ty*tw + tx)*N + n  */
+} wino_tile_order_t;
+
+typedef enum {
+    WINO_OK = 0,
+    WINO_ERR_INVALID = -1,     /* null pointer, non-positive size, unknown enum */
+    WINO_ERR_UNSUPPORTED = -2, /* valid request this build does not implement */
+    WINO_ERR_HIP = -3,         /* a HIP runtime call failed */
+    WINO_ERR_WORKSPACE = -4    /* caller-provided workspace too small */
+} wino_status_t;
+
+/* flags for wino_conv */
+#define WINO_FLAG_RELU 1u /* clamp negatives in the output transform */
+
+/*
+ * Whole layer: y = conv3x3(x, w).  x and w are in `src`'s conventions, y in
+ * `dst`'s.  Replaces the body of
+ *   wrapedConv_NCHW  comparison/wrapedConv_NCHW.cuh:335-492
+ *   wrapedConv_NHWC  comparison/wrapedConv_NHWC.cuh:24-112
+ *   wrapedConv_CHWN  comparison/wrapedConv_CHWN.cuh:16-82
+ * and, for src != dst, the six convLayoutTrans_X_to_Y of
+ * comparison/DataLayoutTrans.cuh:9,101,192,309,418,502 (dispatch :594-651).
+ * Scratch comes from the library's per-device arena (grown on demand) unless
+ * wino_set_workspace() installed a caller buffer.
+ */
+int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
+              int W, int pad, const void *x, const void *w, void *y, void *stream);
+
+/*
+ * Same, with the filter bank already transformed by wino_filter_transform()
+ * (the reference recomputes it on every call: wrapedConv_NCHW.cuh:423).
+ */
+int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K,
+                       int H, int W, int pad, const void *x, const void *U, void *y, void *stream);
+
+/* ---- padded operand geometry ------------------------------------------------
+ * U is [16][Cp][Kp], V is [16][Cp][Pp], the GEMM product Mo is [16][Kp][Pp]
+ * (fp32), with th = ceil(Ho/2), tw = ceil(Wo/2), P = N*th*tw.  The counterpart
+ * of MSize/NSize/KSize at comparison/wrapedConv_NCHW.cuh:346-362. */
+int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int *th, int *tw,
+                  long *P, int *Cp, int *Kp, long *Pp);
+
+/* bytes of scratch wino_conv needs for this problem (upper bound over algos) */
+size_t wino_workspace_bytes(int dtype, int N, int C, int K, int H, int W, int pad);
+
+/* install (ptr != NULL) or remove (ptr == NULL) a caller-owned workspace for the current device */
+int wino_set_workspace(void *ptr, size_t bytes);
+
+/* ---- the four stages on their own (stage parity tests, per-stage timing) -- */
+
+/* U = G g G^T.  Replaces wino_kernel_trans_{nchw,nhwc,chwn}_suitFor128
+ * (wrapedConv_NCHW.cuh:861, wrapedConv_NHWC.cuh:333, wrapedConv_CHWN.cuh:279).
+ * Rows c >= C and columns k >= K of U are written as zeros. */
+int wino_filter_transform(int layout, int dtype, int K, int C, const void *w, void *U, void *stream);
+
+/* V = B^T d B.  Replaces wino_input_trans_{nchw,nhwc,chwn}_suitFor128*
+ * (wrapedConv_NCHW.cuh:683,760, wrapedConv_NHWC.cuh:266, wrapedConv_CHWN.cuh:225).
+ * Rows c >= C are written as zeros; columns p >= P are left untouched. */
+int wino_input_transform(int layout, int dtype, int tile_order, int N, int C, int H, int W, int pad,
+                         const void *x, void *V, void *stream);
+
+/* Mo[xi][k][p] = sum_c U[xi][c][k] V[xi][c][p], xi = 0..15, fp32 accumulate on MFMA.
+ * Replaces GEMM_batch_256_128x128_{KMKN,MKNK} (comparison/GEMM.cuh:124,4). */
+int wino_batched_gemm(int dtype, int C, int K, long P, const void *U, const void *V, float *Mo,
+                      void *stream);
+
+/* y = A^T Mo A.  Replaces wino_invers_{nchw,nhwc,chwn}_suitFor128*
+ * (wrapedConv_NCHW.cuh:905,1034, wrapedConv_NHWC.cuh:376, wrapedConv_CHWN.cuh:379). */
+int wino_output_transform(int layout, int dtype, int tile_order, unsigned flags, int N, int K, int Ho,
+                          int Wo, const float *Mo, void *y, void *stream);
+
+/* GEMM with the output transform in its epilogue: y directly from U and V. */
+int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int N, int C, int K,
+                     int Ho, int Wo, const void *U, const void *V, void *y, void *stream);
+
+/* ---- plain layout permutation (bench harness; the reference has no such kernel) */
+int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void *in,
+                          void *out, void *stream);
+
+/* ---- housekeeping ----------------------------------------------------------- */
+int wino_warmup(void);                 /* empty kernel; replaces warmup<<<1,1>>> (wrapedConv_NCHW.cuh:4-7) */
+int wino_sync(void *stream);           /* hipStreamSynchronize; the reference ends each wrapper with a device sync (:482) */
+const char *wino_last_error(void);
+const char *wino_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WINO_AMD_H */

@@ -1,0 +1,91 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every function that
+include/wino_amd.h declares, validates arguments before touching a GPU, and its
+geometry matches the oracle's tile arithmetic."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from cudnntest_amd import _lib, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "wino_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(wino_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    names = header_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in wino_amd.h but not exported"
+    assert sorted(_lib.SYMBOLS) == names, "ctypes table and header disagree"
+
+
+def test_version_string():
+    assert b"gfx950" in _lib.load().wino_version()
+
+
+@pytest.mark.parametrize("shape,want", [
+    ((32, 256, 256, 56, 56, 1), dict(th=28, tw=28, P=25088, Cp=256, Kp=256, Pp=25088)),
+    ((1, 64, 64, 56, 56, 1), dict(th=28, tw=28, P=784, Cp=64, Kp=128, Pp=896)),
+    ((32, 3, 64, 224, 224, 1), dict(th=112, tw=112, P=401408, Cp=16, Kp=128, Pp=401408)),
+    ((2, 5, 7, 9, 6, 1), dict(th=5, tw=3, P=30, Cp=16, Kp=128, Pp=128)),
+    ((1, 1, 1, 5, 5, 0), dict(th=2, tw=2, P=4, Cp=16, Kp=128, Pp=128)),
+])
+def test_geometry(oracle, shape, want):
+    N, C, K, H, W, pad = shape
+    g = ops.geometry(ops.F32, N, C, K, H, W, pad)
+    assert g == want
+    assert (g["th"], g["tw"]) == oracle.wino_tiles(2, H, W, pad)
+
+
+def test_workspace_bytes_covers_operands():
+    N, C, K, H, W = 32, 256, 256, 56, 56
+    g = ops.geometry(ops.F32, N, C, K, H, W, 1)
+    need = 4 * 16 * (g["Cp"] * g["Kp"] + g["Cp"] * g["Pp"] + g["Kp"] * g["Pp"])
+    assert ops.workspace_bytes(ops.F32, N, C, K, H, W, 1) >= need
+    assert ops.workspace_bytes(ops.F16, N, C, K, H, W, 1) < ops.workspace_bytes(ops.F32, N, C, K, H, W, 1)
+
+
+def test_invalid_arguments_are_rejected_without_a_gpu():
+    L = _lib.load()
+    one = ctypes.c_void_p(16)   # never dereferenced: validation fails first
+    # null tensors
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1, None, one, one, None) == -1
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1, one, None, one, None) == -1
+    assert b"null" in L.wino_last_error()
+    # bad enums
+    assert L.wino_conv(7, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1, one, one, one, None) == -1
+    assert L.wino_conv(0, 0, 9, 0, 0, 1, 1, 1, 4, 4, 1, one, one, one, None) == -1
+    assert L.wino_conv(0, 0, 0, 12, 0, 1, 1, 1, 4, 4, 1, one, one, one, None) == -1
+    # bad shapes: zero batch, image too small for pad 0, unsupported pad
+    assert L.wino_conv(0, 0, 0, 0, 0, 0, 1, 1, 4, 4, 1, one, one, one, None) == -1
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 2, 2, 0, one, one, one, None) == -1
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 2, one, one, one, None) == -1
+    assert b"bad shape" in L.wino_last_error()
+    assert L.wino_filter_transform(0, 0, 0, 4, one, one, None) == -1
+    assert L.wino_input_transform(0, 0, 5, 1, 1, 4, 4, 1, one, one, None) == -1
+    assert L.wino_batched_gemm(0, 0, 1, 1, one, one, one, None) == -1
+    assert L.wino_output_transform(3, 0, 0, 0, 1, 1, 4, 4, one, one, None) == -1
+    assert L.wino_layout_transform(0, 1, 0, 1, 1, 0, 4, one, one, None) == -1
+    assert L.wino_workspace_bytes(0, 0, 1, 1, 4, 4, 1) == 0
+
+
+def test_operator_layer_refuses_cpu_tensors():
+    import torch
+    x = torch.zeros(1, 1, 4, 4)
+    w = torch.zeros(1, 1, 3, 3)
+    with pytest.raises(ValueError):
+        ops.conv(x, w)
+
+
+def test_datalayout_enum_order_matches_reference():
+    # enum class DataLayout { NCHW, NHWC, CHWN }  comparison/DataLayoutTrans.cuh:587-591
+    assert [int(v) for v in ops.DataLayout] == [0, 1, 2]
+    assert [v.name for v in ops.DataLayout] == ["NCHW", "NHWC", "CHWN"]

@@ -1,0 +1,109 @@
+"""Stage-by-stage parity of the HIP kernels against the CPU oracle, through the
+C ABI -- the reference's Module1/2/3.bin idea (layoutTest/NCHW/data/
+ConvTest_V3_NCHW-Mar18.ipynb cells 10-11), seeded and asserted.
+
+Integer-valued inputs make every F(2x2) intermediate exact in fp32, so the
+transform stages must match the oracle bit-for-bit; the GEMM is checked
+bit-for-bit on integers too (sums stay far below 2^24)."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from cudnntest_amd import ops, synth
+from gpu_util import batch_minor_perm, dev, host
+
+pytestmark = pytest.mark.gpu
+LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("K,C", [(4, 3), (64, 64), (130, 17), (7, 40)])
+def test_filter_transform(oracle, layout, K, C):
+    w = synth.small_ints(K * C * 9, 31 + K + C, -4, 4).reshape(K, C, 3, 3)
+    wl = synth.flt_to_layout(w, layout)
+    U = host(ops.filter_transform(dev(wl), layout))
+    want = oracle.wino_filter_transform(wl, layout)
+    assert np.array_equal(U[:, :C, :K], want)
+    assert not U[:, C:, :].any() and not U[:, :, K:].any(), "padding must be zero"
+    # float data: same arithmetic order is not promised, closeness is
+    wf = synth.normal(K * C * 9, 5, 0.1).reshape(K, C, 3, 3)
+    wfl = synth.flt_to_layout(wf, layout)
+    Uf = host(ops.filter_transform(dev(wfl), layout))[:, :C, :K]
+    np.testing.assert_allclose(Uf, oracle.wino_filter_transform(wfl, layout), rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("order", [ops.TILES_BATCH_MAJOR, ops.TILES_BATCH_MINOR])
+@pytest.mark.parametrize("shape,pad", [((2, 3, 5, 5), 1), ((3, 17, 9, 6), 1), ((1, 64, 14, 14), 1),
+                                       ((2, 5, 8, 7), 0), ((4, 16, 28, 28), 1), ((1, 2, 3, 3), 1)])
+def test_input_transform(oracle, layout, order, shape, pad):
+    N, C, H, W = shape
+    x = synth.small_ints(N * C * H * W, 77 + sum(shape), -8, 8).reshape(N, C, H, W)
+    xl = synth.act_to_layout(x, layout)
+    V = host(ops.input_transform(dev(xl), pad, layout, order))
+    want = oracle.wino_input_transform(xl, pad, layout)          # batch-major columns
+    th, tw = oracle.wino_tiles(2, H, W, pad)
+    P = N * th * tw
+    got = V[:, :C, :P]
+    if order == ops.TILES_BATCH_MINOR:
+        got = got[:, :, np.argsort(batch_minor_perm(N, th, tw))]
+    assert np.array_equal(got, want)
+    assert not V[:, C:, :P].any(), "channel padding must be zero"
+
+
+@pytest.mark.parametrize("C,K,P", [(16, 128, 128), (3, 5, 30), (64, 64, 784), (40, 130, 300), (256, 256, 512)])
+def test_batched_gemm(oracle, C, K, P):
+    g = ops.geometry(ops.F32, 1, C, K, 4, 4, 1)
+    Cp, Kp = g["Cp"], g["Kp"]
+    Pp = (P + 127) // 128 * 128
+    U = np.zeros((16, Cp, Kp), np.float32)
+    V = np.zeros((16, Cp, Pp), np.float32)
+    U[:, :C, :K] = synth.small_ints(16 * C * K, 3, -3, 3).reshape(16, C, K)
+    V[:, :C, :P] = synth.small_ints(16 * C * P, 4, -5, 5).reshape(16, C, P)
+    Mo = host(ops.batched_gemm(dev(U), dev(V), C, K, P))
+    want = oracle.wino_gemm(np.ascontiguousarray(U[:, :C, :K]), np.ascontiguousarray(V[:, :C, :P]))
+    assert np.array_equal(Mo[:, :K, :P], want)
+
+
+def test_batched_gemm_floats(oracle):
+    C, K, P = 64, 128, 256
+    U = synth.normal(16 * C * K, 8, 0.2).reshape(16, C, K)
+    V = synth.uniform_pm1(16 * C * P, 9).reshape(16, C, P)
+    Mo = host(ops.batched_gemm(dev(U), dev(V), C, K, P))
+    assert oracle.rel_l2(Mo, oracle.wino_gemm(U, V)) < 1e-6
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("order", [ops.TILES_BATCH_MAJOR, ops.TILES_BATCH_MINOR])
+@pytest.mark.parametrize("N,K,Ho,Wo", [(2, 4, 5, 5), (3, 7, 9, 6), (1, 130, 14, 14), (4, 16, 28, 28), (2, 3, 1, 1)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_output_transform(oracle, layout, order, N, K, Ho, Wo, relu):
+    th, tw = (Ho + 1) // 2, (Wo + 1) // 2
+    P = N * th * tw
+    g = ops.geometry(ops.F32, 1, 1, K, 4, 4, 1)
+    Kp, Pp = g["Kp"], (P + 127) // 128 * 128
+    M = synth.small_ints(16 * K * P, 13 + K, -6, 6).reshape(16, K, P)     # batch-major columns
+    Mo = np.full((16, Kp, Pp), 1e30, np.float32)                         # poison the padding
+    if order == ops.TILES_BATCH_MINOR:
+        Mo[:, :K, :P] = M[:, :, batch_minor_perm(N, th, tw)]
+    else:
+        Mo[:, :K, :P] = M
+    y = host(ops.output_transform(dev(Mo), N, K, Ho, Wo, layout, order, relu))
+    want = oracle.wino_output_transform(M, N, Ho, Wo, layout)
+    if relu:
+        want = np.maximum(want, 0)
+    assert np.array_equal(y, want)
+
+
+@pytest.mark.parametrize("src,dst", list(itertools.permutations(LAYOUTS, 2)))
+def test_layout_transform(oracle, src, dst):
+    N, C, H, W = 3, 5, 7, 6
+    x = synth.uniform_pm1(N * C * H * W, 2).reshape(N, C, H, W)
+    xs = synth.act_to_layout(x, src)
+    got = host(ops.layout_transform(dev(xs), src, dst))
+    assert np.array_equal(got, synth.act_to_layout(x, dst))
+    xh = dev(xs, ops.F16)
+    assert torch.equal(ops.layout_transform(xh, src, dst).cpu(),
+                       torch.from_numpy(synth.act_to_layout(x, dst)).half())
