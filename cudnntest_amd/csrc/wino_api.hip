@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
+#include <vector>
 
 #include "common.hpp"
 #include "gemm.hpp"
@@ -75,6 +76,34 @@ int arena_get(size_t bytes, void** out) {
     *out = a.own;
     return WINO_OK;
 }
+
+// ---- optional per-stage timing: HIP events recorded on the launch stream ---------
+struct StageSpan {
+    int stage;
+    hipEvent_t a, b;
+};
+bool g_timing = false;
+std::vector<StageSpan> g_spans;
+std::mutex g_spans_mu;
+
+struct StageScope {
+    bool on;
+    int stage;
+    hipStream_t st;
+    hipEvent_t a = nullptr, b = nullptr;
+    StageScope(int stage_, hipStream_t st_) : on(g_timing), stage(stage_), st(st_) {
+        if (on) {
+            on = hipEventCreate(&a) == hipSuccess && hipEventCreate(&b) == hipSuccess &&
+                 hipEventRecord(a, st) == hipSuccess;
+        }
+    }
+    ~StageScope() {
+        if (on && hipEventRecord(b, st) == hipSuccess) {
+            std::lock_guard<std::mutex> lk(g_spans_mu);
+            g_spans.push_back({stage, a, b});
+        }
+    }
+};
 
 struct Scratch {
     size_t u_off, v_off, m_off, total;
@@ -172,13 +201,21 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     if (Upre) {
         U = const_cast<void*>(Upre);
     } else {
+        StageScope t(WINO_STAGE_FILTER, st);
         rc = wino_filter_transform(src, dtype, K, C, w, U, stream);
         if (rc) return rc;
     }
-    rc = wino_input_transform(src, dtype, order, N, C, H, W, pad, x, V, stream);
-    if (rc) return rc;
-    rc = launch_gemm(dtype, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
-    if (rc) return rc;
+    {
+        StageScope t(WINO_STAGE_INPUT, st);
+        rc = wino_input_transform(src, dtype, order, N, C, H, W, pad, x, V, stream);
+        if (rc) return rc;
+    }
+    {
+        StageScope t(WINO_STAGE_GEMM, st);
+        rc = launch_gemm(dtype, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
+        if (rc) return rc;
+    }
+    StageScope t(WINO_STAGE_OUTPUT, st);
     return wino_output_transform(dst, dtype, order, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
 }
 
@@ -298,6 +335,33 @@ int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int 
                            a, dst, N, C, H, W);
     LAUNCH_CHECK("layout_transform");
     return WINO_OK;
+}
+
+int wino_stage_timing(int enable) {
+    std::lock_guard<std::mutex> lk(g_spans_mu);
+    g_timing = enable != 0;
+    return WINO_OK;
+}
+
+int wino_stage_times(float* ms, long* calls) {
+    if (!ms || !calls) return fail(WINO_ERR_INVALID, "null pointer");
+    std::vector<StageSpan> spans;
+    {
+        std::lock_guard<std::mutex> lk(g_spans_mu);
+        spans.swap(g_spans);
+    }
+    for (int i = 0; i < WINO_NUM_STAGES; ++i) { ms[i] = 0.f; calls[i] = 0; }
+    int rc = WINO_OK;
+    for (auto& sp : spans) {
+        float t = 0.f;
+        hipError_t e = hipEventSynchronize(sp.b);
+        if (e == hipSuccess) e = hipEventElapsedTime(&t, sp.a, sp.b);
+        if (e != hipSuccess) rc = fail(WINO_ERR_HIP, "stage timing: %s", hipGetErrorString(e));
+        else { ms[sp.stage] += t; calls[sp.stage] += 1; }
+        (void)hipEventDestroy(sp.a);
+        (void)hipEventDestroy(sp.b);
+    }
+    return rc;
 }
 
 int wino_warmup(void) {

@@ -88,6 +88,22 @@ def warmup():
     _lib.check(_lib.load().wino_warmup(), "wino_warmup")
 
 
+STAGES = ("filter", "input", "gemm", "output")
+
+
+def stage_timing(enable):
+    _lib.check(_lib.load().wino_stage_timing(int(bool(enable))), "wino_stage_timing")
+
+
+def stage_times():
+    """{stage: (total_ms, spans)} accumulated since the last call; blocks on the recorded events."""
+    import ctypes
+    ms = (ctypes.c_float * 4)()
+    calls = (ctypes.c_long * 4)()
+    _lib.check(_lib.load().wino_stage_times(ms, calls), "wino_stage_times")
+    return {name: (float(ms[i]), int(calls[i])) for i, name in enumerate(STAGES)}
+
+
 # ---- whole layer -------------------------------------------------------------
 
 def conv(x, w, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None):

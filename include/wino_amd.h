@@ -121,6 +121,21 @@ int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int 
 int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void *in,
                           void *out, void *stream);
 
+/* ---- per-stage timing (the commented-out event pairs of wrapedConv_NCHW.cuh:88-138, made usable)
+ * While enabled, wino_conv / wino_conv_prepared bracket every stage they launch
+ * with a pair of HIP events on the launch stream.  wino_stage_times() waits for
+ * the recorded events, returns the accumulated milliseconds and number of spans
+ * per stage (arrays of WINO_NUM_STAGES) and forgets them. */
+typedef enum {
+    WINO_STAGE_FILTER = 0,
+    WINO_STAGE_INPUT = 1,
+    WINO_STAGE_GEMM = 2,   /* the batched GEMM, or the kernel that contains it (epilogue-fused / fused) */
+    WINO_STAGE_OUTPUT = 3,
+    WINO_NUM_STAGES = 4
+} wino_stage_t;
+int wino_stage_timing(int enable);
+int wino_stage_times(float *ms, long *calls);
+
 /* ---- housekeeping ----------------------------------------------------------- */
 int wino_warmup(void);                 /* empty kernel; replaces warmup<<<1,1>>> (wrapedConv_NCHW.cuh:4-7) */
 int wino_sync(void *stream);           /* hipStreamSynchronize; the reference ends each wrapper with a device sync (:482) */
