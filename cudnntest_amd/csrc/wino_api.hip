@@ -160,6 +160,35 @@ int launch_gemm(int dtype, int Cp, int Kp, long Pp, const void* U, const void* V
     return WINO_OK;
 }
 
+template <typename OutT, bool SWAP>
+int launch_gemm_out_t(int order, unsigned flags, const Geometry& g, const float* U, const float* V, void* y,
+                      int dst, hipStream_t st) {
+    auto kern = gemm_out_f32_kernel<OutT, SWAP>;
+    static bool attr_set = false;   // per instantiation
+    if (!attr_set) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)GO_LDS_BYTES));
+        attr_set = true;
+    }
+    const int kTiles = (g.K + GO_T - 1) / GO_T;
+    const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
+    const int pGroups = (pTiles + 7) / 8;
+    dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
+    hipLaunchKernelGGL(kern, grid, block, GO_LDS_BYTES, st, U, V, (OutT*)y, act_strides(dst, g.N, g.K, g.Ho, g.Wo),
+                       g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, g.Pp, order,
+                       (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
+    LAUNCH_CHECK("gemm_output");
+    return WINO_OK;
+}
+
+int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* U, const void* V,
+                    void* y, hipStream_t st) {
+    if (dtype != WINO_F32) return fail(WINO_ERR_UNSUPPORTED, "epilogue-fused GEMM: dtype %d not built yet", dtype);
+    if (dst == WINO_NHWC)
+        return launch_gemm_out_t<float, true>(order, flags, g, (const float*)U, (const float*)V, y, dst, st);
+    return launch_gemm_out_t<float, false>(order, flags, g, (const float*)U, (const float*)V, y, dst, st);
+}
+
 #define DISPATCH_DTYPE(dtype, CALL)                          \
     switch (dtype) {                                         \
     case WINO_F32: { typedef float T; return CALL; }         \
@@ -185,7 +214,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     if (!make_geometry(N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     if (algo == WINO_ALGO_AUTO) algo = WINO_ALGO_STAGED;
-    if (algo != WINO_ALGO_STAGED) return fail(WINO_ERR_UNSUPPORTED, "algo %d not built yet", algo);
+    if (algo == WINO_ALGO_FUSED) return fail(WINO_ERR_UNSUPPORTED, "algo %d not built yet", algo);
 
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype);
@@ -209,6 +238,10 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         StageScope t(WINO_STAGE_INPUT, st);
         rc = wino_input_transform(src, dtype, order, N, C, H, W, pad, x, V, stream);
         if (rc) return rc;
+    }
+    if (algo == WINO_ALGO_EPILOGUE) {
+        StageScope t(WINO_STAGE_GEMM, st);
+        return launch_gemm_out(dst, dtype, order, flags, g, U, V, y, st);
     }
     {
         StageScope t(WINO_STAGE_GEMM, st);
@@ -313,8 +346,17 @@ int wino_output_transform(int layout, int dtype, int tile_order, unsigned flags,
                                                      (hipStream_t)stream));
 }
 
-int wino_gemm_output(int, int, int, unsigned, int, int, int, int, int, const void*, const void*, void*, void*) {
-    return fail(WINO_ERR_UNSUPPORTED, "epilogue-fused GEMM not built yet");
+int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int N, int C, int K, int Ho, int Wo,
+                     const void* U, const void* V, void* y, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
+    if (!U || !V || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    Geometry g;
+    // geometry from the output size: pad 1 keeps H == Ho
+    if (!make_geometry(N, C, K, Ho, Wo, 1, &g))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d Ho=%d Wo=%d", N, C, K, Ho, Wo);
+    return launch_gemm_out(layout, dtype, tile_order, flags, g, U, V, y, (hipStream_t)stream);
 }
 
 int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void* in, void* out,

@@ -15,7 +15,7 @@ from gpu_util import TOL, dev, host
 
 pytestmark = pytest.mark.gpu
 LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
-ALGOS = [ops.ALGO_STAGED]
+ALGOS = [ops.ALGO_STAGED, ops.ALGO_EPILOGUE]
 
 SMALL = [(2, 3, 4, 5, 5), (1, 8, 8, 6, 6), (3, 5, 7, 9, 9), (2, 16, 130, 7, 10), (1, 1, 1, 3, 3), (5, 40, 24, 14, 14)]
 
@@ -93,6 +93,9 @@ def test_properties_at_full_size():
     x2 = torch.rand((N, C, H, H), device="cuda", generator=g) * 2 - 1
     w = torch.randn((K, C, 3, 3), device="cuda", generator=g) * (2.0 / (9 * C)) ** 0.5
     y1, y2 = ops.conv(x1, w), ops.conv(x2, w)
+    for algo in ALGOS[1:]:
+        ya = ops.conv(x1, w, algo=algo)
+        assert ((ya - y1).norm() / y1.norm()).item() < 1e-6, algo
     y12 = ops.conv(x1 + x2, w)
     rel = ((y12 - (y1 + y2)).norm() / y12.norm()).item()
     assert rel < 1e-5, rel

@@ -97,6 +97,29 @@ def test_output_transform(oracle, layout, order, N, K, Ho, Wo, relu):
     assert np.array_equal(y, want)
 
 
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("order", [ops.TILES_BATCH_MAJOR, ops.TILES_BATCH_MINOR])
+@pytest.mark.parametrize("N,C,K,Ho,Wo", [(2, 3, 4, 5, 5), (3, 20, 70, 9, 6), (1, 64, 130, 14, 14), (4, 16, 64, 28, 28)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_gemm_with_output_epilogue(oracle, layout, order, N, C, K, Ho, Wo, relu):
+    """y straight from U and V: must equal oracle GEMM followed by oracle output transform."""
+    th, tw = (Ho + 1) // 2, (Wo + 1) // 2
+    P = N * th * tw
+    g = ops.geometry(ops.F32, N, C, K, Ho, Wo, 1)
+    Cp, Kp, Pp = g["Cp"], g["Kp"], g["Pp"]
+    Uc = synth.small_ints(16 * C * K, 3 + K, -3, 3).reshape(16, C, K)
+    Vc = synth.small_ints(16 * C * P, 4 + C, -5, 5).reshape(16, C, P)       # batch-major columns
+    U = np.zeros((16, Cp, Kp), np.float32)
+    V = np.zeros((16, Cp, Pp), np.float32)
+    U[:, :C, :K] = Uc
+    V[:, :C, :P] = Vc[:, :, batch_minor_perm(N, th, tw)] if order == ops.TILES_BATCH_MINOR else Vc
+    y = host(ops.gemm_output(dev(U), dev(V), N, C, K, Ho, Wo, layout, order, relu))
+    want = oracle.wino_output_transform(oracle.wino_gemm(Uc, Vc), N, Ho, Wo, layout)
+    if relu:
+        want = np.maximum(want, 0)
+    assert np.array_equal(y, want)
+
+
 @pytest.mark.parametrize("src,dst", list(itertools.permutations(LAYOUTS, 2)))
 def test_layout_transform(oracle, src, dst):
     N, C, H, W = 3, 5, 7, 6
