@@ -55,6 +55,29 @@ template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
 
 __host__ inline size_t dtype_size(int dtype) { return dtype == WINO_F32 ? 4 : 2; }
 
+// ---- channel vectors ------------------------------------------------------------
+// The transformed operands keep CV consecutive channels of one (coordinate, tile)
+// or (coordinate, filter) together in a 16-byte vector:
+//     U[xi][Cp/CV][Kp][CV]     V[xi][Cp/CV][Pp][CV]      CV = 16 / sizeof(T)
+// so every HBM and LDS access of the GEMM side is a 16-byte access, and a lane
+// of an MFMA fetches the channels it multiplies with one LDS read.
+template <typename T> struct ChanVec {
+    static constexpr int n = 16 / (int)sizeof(T);
+};
+__host__ inline int chan_vec(int dtype) { return dtype == WINO_F32 ? 4 : 8; }
+
+template <typename T> struct alignas(16) Pack16 {
+    T e[16 / sizeof(T)];
+};
+
+// dst[0..CV) = v[0..CV) as one 16-byte store
+template <typename T> __device__ __forceinline__ void store_chan_vec(T* dst, const float* v) {
+    Pack16<T> pk;
+#pragma unroll
+    for (int i = 0; i < ChanVec<T>::n; ++i) pk.e[i] = from_f32<T>(v[i]);
+    *reinterpret_cast<Pack16<T>*>(dst) = pk;
+}
+
 // ---- padded geometry ---------------------------------------------------------
 constexpr int kCPad = 16;    // reduction (channel) dimension of U and V is padded to this
 constexpr int kKPad = 128;   // filter dimension of U / Mo

@@ -2,11 +2,18 @@
 //
 //   Mo[xi][k][p] = sum_c U[xi][c][k] * V[xi][c][p]          xi = 0..15
 //
-// fp32 path: v_mfma_f32_32x32x2_f32.  Operand registers of that instruction for
-// lane l:  a = A[i = l%32][kk = l/32],  b = B[kk = l/32][j = l%32];  the 16
-// accumulator registers r hold D[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32].
-// With A = U^T (i = filter) and B = V (j = tile) a wave store of one register
-// is a contiguous run of tiles.
+// Operands arrive as 16-byte channel vectors, U[xi][Cp/CV][Kp][CV] and
+// V[xi][Cp/CV][Pp][CV]; HBM -> LDS copies and LDS -> register fetches are all
+// 16-byte accesses in the same arrangement.
+//
+// MFMA register conventions (32x32 family), lane l, l32 = l%32, lh = l/32:
+//   fp32  v_mfma_f32_32x32x2_f32 :  a = A[i=l32][kk=lh]        b = B[kk=lh][j=l32]
+//   16bit v_mfma_f32_32x32x16_*  :  a = A[i=l32][8*lh .. +7]   b = B[8*lh .. +7][j=l32]
+//   accumulator register r holds D[i = 8*(r/4) + 4*lh + r%4][j = l32].
+// A "k-group" is the pair of channel vectors (2g, 2g+1) taken by the lane halves
+// lh = 0 and 1: 8 channels for fp32 (4 MFMAs, one per vector element), 16
+// channels for f16/bf16 (one MFMA).  The sum over channels does not care which
+// channel a lane half takes as long as both operands agree.
 #pragma once
 #include "common.hpp"
 #include "transforms.hpp"
@@ -15,32 +22,61 @@ namespace wino {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
+template <typename T> struct Mma;
+template <> struct Mma<float> {
+    typedef floatx4 vec;
+    static __device__ __forceinline__ void run(const vec& a, const vec& b, floatx16& acc) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+    }
+};
+template <> struct Mma<f16_t> {
+    typedef halfx8 vec;
+    static __device__ __forceinline__ void run(const vec& a, const vec& b, floatx16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+    }
+};
+template <> struct Mma<bf16_t> {
+    typedef bf16x8 vec;
+    static __device__ __forceinline__ void run(const vec& a, const vec& b, floatx16& acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+    }
+};
+
+// =============================================================================
+// Plain batched GEMM, product written to HBM as Mo[xi][Kp][Pp] (fp32).
+//
 // Block tile 128 filters x 128 tiles, 4 waves in a 2x2 arrangement, each wave
-// 64x64 = 2x2 MFMA tiles.  Reduction is consumed 16 channels at a time from LDS,
-// double-buffered: the next slab travels HBM -> registers while the current one
-// feeds the MFMAs, then registers -> the other LDS buffer, one barrier per slab.
-constexpr int GEMM_BM = 128, GEMM_BN = 128, GEMM_KC = 16;
+// 64x64 = 2x2 MFMA tiles.  The reduction is consumed NV channel vectors at a
+// time from LDS, double-buffered: the next slab travels HBM -> registers while
+// the current one feeds the MFMAs, then registers -> the other LDS buffer, one
+// barrier per slab.
+// =============================================================================
+constexpr int GEMM_BM = 128, GEMM_BN = 128;
 
-__global__ __launch_bounds__(256) void gemm_f32_128x128_kernel(const float* __restrict__ U,
-                                                                const float* __restrict__ V,
-                                                                float* __restrict__ Mo, int Cp, int Kp, long Pp) {
-    __shared__ float As[2][GEMM_KC][GEMM_BM];
-    __shared__ float Bs[2][GEMM_KC][GEMM_BN];
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                            float* __restrict__ Mo, int Cp, int Kp, long Pp) {
+    typedef typename Mma<T>::vec vec;
+    constexpr int CV = ChanVec<T>::n;
+    __shared__ vec As[2][NV][GEMM_BM];
+    __shared__ vec Bs[2][NV][GEMM_BN];
 
     const int xi = blockIdx.z;
     const long p0 = (long)blockIdx.x * GEMM_BN;
     const int k0 = blockIdx.y * GEMM_BM;
-    const float* Ub = U + (size_t)xi * Cp * Kp + k0;
-    const float* Vb = V + (size_t)xi * Cp * Pp + p0;
+    const int CQ = Cp / CV;
+    const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
+    const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
-
-    // global -> LDS mapping: thread moves rows (tid/32) and (tid/32 + 8), 4 floats at column 4*(tid%32)
-    const int lrow = tid >> 5, lcol = (tid & 31) * 4;
+    const int lrow = tid >> 7, lcol = tid & 127;   // rows lrow + 2*h
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -50,24 +86,24 @@ __global__ __launch_bounds__(256) void gemm_f32_128x128_kernel(const float* __re
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    floatx4 ra[2], rb[2];
+    vec ra[NV / 2], rb[NV / 2];
     auto gload = [&](int ch) {
-        const int c0 = ch * GEMM_KC;
+        const int q0 = ch * NV;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            ra[h] = *reinterpret_cast<const floatx4*>(Ub + (size_t)(c0 + lrow + 8 * h) * Kp + lcol);
-            rb[h] = *reinterpret_cast<const floatx4*>(Vb + (size_t)(c0 + lrow + 8 * h) * Pp + lcol);
+        for (int h = 0; h < NV / 2; ++h) {
+            ra[h] = Ub[(size_t)(q0 + lrow + 2 * h) * Kp + lcol];
+            rb[h] = Vb[(size_t)(q0 + lrow + 2 * h) * Pp + lcol];
         }
     };
     auto lstore = [&](int buf) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            *reinterpret_cast<floatx4*>(&As[buf][lrow + 8 * h][lcol]) = ra[h];
-            *reinterpret_cast<floatx4*>(&Bs[buf][lrow + 8 * h][lcol]) = rb[h];
+        for (int h = 0; h < NV / 2; ++h) {
+            As[buf][lrow + 2 * h][lcol] = ra[h];
+            Bs[buf][lrow + 2 * h][lcol] = rb[h];
         }
     };
 
-    const int nch = Cp / GEMM_KC;
+    const int nch = CQ / NV;
     gload(0);
     lstore(0);
     __syncthreads();
@@ -76,18 +112,17 @@ __global__ __launch_bounds__(256) void gemm_f32_128x128_kernel(const float* __re
         const int buf = ch & 1;
         if (ch + 1 < nch) gload(ch + 1);
 #pragma unroll
-        for (int kk = 0; kk < GEMM_KC / 2; ++kk) {
-            float a[2], b[2];
+        for (int g = 0; g < NV / 2; ++g) {
+            vec a[2], b[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                a[t] = As[buf][kk * 2 + lh][wm * 64 + t * 32 + l32];
-                b[t] = Bs[buf][kk * 2 + lh][wn * 64 + t * 32 + l32];
+                a[t] = As[buf][2 * g + lh][wm * 64 + t * 32 + l32];
+                b[t] = Bs[buf][2 * g + lh][wn * 64 + t * 32 + l32];
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < 2; ++j) Mma<T>::run(a[i], b[j], acc[i][j]);
         }
         if (ch + 1 < nch) lstore(buf ^ 1);
         __syncthreads();
@@ -115,8 +150,8 @@ __global__ __launch_bounds__(256) void gemm_f32_128x128_kernel(const float* __re
 // channels ends every lane holds the 16 coordinates of its (filter, tile) pairs
 // and applies A^T(.)A in registers; the product tensor never reaches HBM.
 //
-// Reduction runs KC channels at a time through LDS ([xi][KC][64] for U and for
-// V), double-buffered through registers as in the plain GEMM.
+// The reduction runs one k-group at a time through LDS ([xi][2][64] channel
+// vectors for U and for V), double-buffered through registers.
 //
 // SWAP = false: MFMA rows = filters, lanes = tiles  (stores contiguous along the
 //               tile axis: NCHW, or CHWN with batch-minor tiles)
@@ -126,9 +161,8 @@ __global__ __launch_bounds__(256) void gemm_f32_128x128_kernel(const float* __re
 // 8 XCDs round-robin, so the ids that land on one XCD walk the filter tiles of
 // one tile patch first; the V slab they share then stays in that XCD's L2.
 // =============================================================================
-constexpr int GO_KC = 8;
 constexpr int GO_T = 64;   // patch edge (filters and tiles)
-constexpr size_t GO_LDS_BYTES = 2ull * 2 * 16 * GO_KC * GO_T * sizeof(float);
+constexpr size_t GO_LDS_BYTES = 2ull * 2 * 16 * 2 * GO_T * 16;   // stages x operands x xi x 2 vectors x 64 x 16 B
 
 template <typename OutT>
 __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const ActStrides& ys, int n, int k, int ty,
@@ -148,16 +182,17 @@ __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const A
     }
 }
 
-template <typename OutT, bool SWAP>
-__global__ __launch_bounds__(256) void gemm_out_f32_kernel(const float* __restrict__ U, const float* __restrict__ V,
-                                                           OutT* __restrict__ y, ActStrides ys, int N, int K, int Ho,
-                                                           int Wo, int th, int tw, long P, int Cp, int Kp, long Pp,
-                                                           int order, int relu, int kTiles, int pTiles) {
-    // 2 stages x (U slab + V slab) x 16 x KC x 64 floats = 128 KB: dynamic LDS
-    extern __shared__ float go_smem[];
-    typedef float (*slab_t)[16][GO_KC][GO_T];
+template <typename T, bool SWAP>
+__global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                       T* __restrict__ y, ActStrides ys, int N, int K, int Ho, int Wo,
+                                                       int th, int tw, long P, int Cp, int Kp, long Pp, int order,
+                                                       int relu, int kTiles, int pTiles) {
+    typedef typename Mma<T>::vec vec;
+    constexpr int CV = ChanVec<T>::n;
+    extern __shared__ __attribute__((aligned(16))) unsigned char go_smem[];
+    typedef vec (*slab_t)[16][2][GO_T];
     slab_t Us = reinterpret_cast<slab_t>(go_smem);
-    slab_t Vs = reinterpret_cast<slab_t>(go_smem + 2 * 16 * GO_KC * GO_T);
+    slab_t Vs = reinterpret_cast<slab_t>(go_smem + GO_LDS_BYTES / 2);
 
     const int b = blockIdx.x;
     const int xcd = b & 7, j = b >> 3;
@@ -166,6 +201,9 @@ __global__ __launch_bounds__(256) void gemm_out_f32_kernel(const float* __restri
     if (ptile >= pTiles) return;
     const int k0 = ktile * GO_T;
     const long p0 = (long)ptile * GO_T;
+    const int CQ = Cp / CV;
+    const vec* Ug = reinterpret_cast<const vec*>(U);
+    const vec* Vg = reinterpret_cast<const vec*>(V);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -178,48 +216,44 @@ __global__ __launch_bounds__(256) void gemm_out_f32_kernel(const float* __restri
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[xi][r] = 0.f;
 
-    // global -> LDS: 128 rows (xi, c) of 64 floats per operand = 2048 float4, 8 per thread per operand
-    floatx4 ru[8], rv[8];
-    const int q4 = (tid & 15) * 4;      // column inside the 64-wide row
-    const int rbase = tid >> 4;         // 0..15, rows rbase + 16*i
-    auto gload = [&](int ch) {
-        const int c0 = ch * GO_KC;
+    // HBM -> LDS: per operand 32 rows (xi, half) of 64 vectors = 2048 vectors, 8 per thread
+    vec ru[8], rv[8];
+    const int col = tid & 63;
+    const int rbase = tid >> 6;          // 0..3, rows rbase + 4*i
+    auto gload = [&](int g) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int row = rbase + 16 * i;            // 0..127
-            const int xi = row / GO_KC, c = row % GO_KC;
-            ru[i] = *reinterpret_cast<const floatx4*>(U + ((size_t)xi * Cp + c0 + c) * Kp + k0 + q4);
-            rv[i] = *reinterpret_cast<const floatx4*>(V + ((size_t)xi * Cp + c0 + c) * Pp + p0 + q4);
+            const int row = rbase + 4 * i;     // 0..31
+            const int xi = row >> 1, h = row & 1;
+            ru[i] = Ug[((size_t)xi * CQ + 2 * g + h) * Kp + k0 + col];
+            rv[i] = Vg[((size_t)xi * CQ + 2 * g + h) * Pp + p0 + col];
         }
     };
     auto lstore = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int row = rbase + 16 * i;
-            const int xi = row / GO_KC, c = row % GO_KC;
-            *reinterpret_cast<floatx4*>(&Us[buf][xi][c][q4]) = ru[i];
-            *reinterpret_cast<floatx4*>(&Vs[buf][xi][c][q4]) = rv[i];
+            const int row = rbase + 4 * i;
+            Us[buf][row >> 1][row & 1][col] = ru[i];
+            Vs[buf][row >> 1][row & 1][col] = rv[i];
         }
     };
 
-    const int nch = Cp / GO_KC;
+    const int ngrp = CQ / 2;
     gload(0);
     lstore(0);
     __syncthreads();
 
-    for (int ch = 0; ch < nch; ++ch) {
-        const int buf = ch & 1;
-        if (ch + 1 < nch) gload(ch + 1);
+    for (int g = 0; g < ngrp; ++g) {
+        const int buf = g & 1;
+        if (g + 1 < ngrp) gload(g + 1);
 #pragma unroll
         for (int xi = 0; xi < 16; ++xi) {
-#pragma unroll
-            for (int kk = 0; kk < GO_KC / 2; ++kk) {
-                const float fu = Us[buf][xi][kk * 2 + lh][(SWAP ? wn : wm) * 32 + l32];
-                const float fv = Vs[buf][xi][kk * 2 + lh][(SWAP ? wm : wn) * 32 + l32];
-                acc[xi] = __builtin_amdgcn_mfma_f32_32x32x2f32(SWAP ? fv : fu, SWAP ? fu : fv, acc[xi], 0, 0, 0);
-            }
+            const vec fu = Us[buf][xi][lh][(SWAP ? wn : wm) * 32 + l32];
+            const vec fv = Vs[buf][xi][lh][(SWAP ? wm : wn) * 32 + l32];
+            if (SWAP) Mma<T>::run(fv, fu, acc[xi]);
+            else Mma<T>::run(fu, fv, acc[xi]);
         }
-        if (ch + 1 < nch) lstore(buf ^ 1);
+        if (g + 1 < ngrp) lstore(buf ^ 1);
         __syncthreads();
     }
 
@@ -238,7 +272,7 @@ __global__ __launch_bounds__(256) void gemm_out_f32_kernel(const float* __restri
             for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
             float y00, y01, y10, y11;
             output_tile_transform(m, y00, y01, y10, y11);
-            store_tile_outputs<OutT>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
         }
     } else {
         const int k = k0 + wn * 32 + l32;
@@ -254,7 +288,7 @@ __global__ __launch_bounds__(256) void gemm_out_f32_kernel(const float* __restri
             for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
             float y00, y01, y10, y11;
             output_tile_transform(m, y00, y01, y10, y11);
-            store_tile_outputs<OutT>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
         }
     }
 }

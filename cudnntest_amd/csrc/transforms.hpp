@@ -4,6 +4,9 @@
 //   B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
 //   G   = [1 0 0; 1/2 1/2 1/2; 1/2 -1/2 1/2; 0 0 1]
 //   A^T = [1 1 1 0; 0 1 -1 -1]
+//
+// Operand layouts written here (CV = 16 / sizeof(T) channels per 16-byte vector):
+//   U[xi][Cp/CV][Kp][CV]     V[xi][Cp/CV][Pp][CV]
 #pragma once
 #include "common.hpp"
 
@@ -18,17 +21,17 @@ __device__ __forceinline__ void bt4(float d0, float d1, float d2, float d3, floa
     o3 = d1 - d3;
 }
 
-// v[i][j] (4x4) = B^T d B, rows first then columns
-__device__ __forceinline__ void input_tile_transform(const float d[4][4], float v[4][4]) {
+// v (16, row-major 4x4) = B^T d B, rows first then columns
+__device__ __forceinline__ void input_tile_transform(const float d[4][4], float* v) {
     float t[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) bt4(d[0][j], d[1][j], d[2][j], d[3][j], t[0][j], t[1][j], t[2][j], t[3][j]);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) bt4(t[i][0], t[i][1], t[i][2], t[i][3], v[i][0], v[i][1], v[i][2], v[i][3]);
+    for (int i = 0; i < 4; ++i) bt4(t[i][0], t[i][1], t[i][2], t[i][3], v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
 }
 
-// u (4x4) = G g G^T
-__device__ __forceinline__ void filter_tile_transform(const float g[3][3], float u[4][4]) {
+// u (16, row-major 4x4) = G g G^T
+__device__ __forceinline__ void filter_tile_transform(const float g[3][3], float* u) {
     float t[4][3];
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
@@ -39,10 +42,10 @@ __device__ __forceinline__ void filter_tile_transform(const float g[3][3], float
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        u[i][0] = t[i][0];
-        u[i][1] = 0.5f * (t[i][0] + t[i][1] + t[i][2]);
-        u[i][2] = 0.5f * (t[i][0] - t[i][1] + t[i][2]);
-        u[i][3] = t[i][2];
+        u[4 * i + 0] = t[i][0];
+        u[4 * i + 1] = 0.5f * (t[i][0] + t[i][1] + t[i][2]);
+        u[4 * i + 2] = 0.5f * (t[i][0] - t[i][1] + t[i][2]);
+        u[4 * i + 3] = t[i][2];
     }
 }
 
@@ -62,85 +65,106 @@ __device__ __forceinline__ void output_tile_transform(const float m[16], float& 
 }
 
 // ---- filter transform ---------------------------------------------------------
-// One thread per (k, c), k fastest so the 16 stores of a wave are contiguous.
-// Grid covers the padded Cp x Kp rectangle: the padding is written as zeros,
-// which is what lets the GEMM run without masks on the reduction dimension.
+// One thread per (filter k, channel vector cq), k fastest: each of its 16 stores
+// is a 16-byte vector and a wave's stores are contiguous.  The grid covers the
+// padded (Cp/CV) x Kp rectangle and the padding is written as zeros, which is
+// what lets the GEMM run without masks on the reduction dimension.
 template <typename T>
 __global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restrict__ w, T* __restrict__ U,
                                                                 FltStrides s, int K, int C, int Kp, int Cp) {
-    int k = blockIdx.x * blockDim.x + threadIdx.x;
-    int c = blockIdx.y;
+    constexpr int CV = ChanVec<T>::n;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    const int cq = blockIdx.y;
     if (k >= Kp) return;
-    float u[4][4];
-    if (k < K && c < C) {
-        float g[3][3];
-        const T* wp = w + k * s.k + c * s.c;
+    float u[CV][16];
 #pragma unroll
-        for (int r = 0; r < 3; ++r)
+    for (int e = 0; e < CV; ++e) {
+        const int c = cq * CV + e;
+        if (k < K && c < C) {
+            float g[3][3];
+            const T* wp = w + k * s.k + c * s.c;
 #pragma unroll
-            for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
-        filter_tile_transform(g, u);
-    } else {
+            for (int r = 0; r < 3; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) u[i / 4][i % 4] = 0.f;
+                for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
+            filter_tile_transform(g, u[e]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) u[e][i] = 0.f;
+        }
     }
-    const size_t plane = (size_t)Cp * Kp;
-    T* up = U + (size_t)c * Kp + k;
+    const size_t plane = (size_t)Cp * Kp;   // elements per coordinate
+    T* up = U + ((size_t)cq * Kp + k) * CV;
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi) up[xi * plane] = from_f32<T>(u[xi / 4][xi % 4]);
+    for (int xi = 0; xi < 16; ++xi) {
+        float v[CV];
+#pragma unroll
+        for (int e = 0; e < CV; ++e) v[e] = u[e][xi];
+        store_chan_vec<T>(up + xi * plane, v);
+    }
 }
 
 // ---- input transform, layout-generic ---------------------------------------------
-// One thread per (tile p, channel c), p fastest: the 16 stores of a wave are
-// contiguous runs of V.  Reads go through the activation strides, so the kernel
-// is correct for every layout and tile order; it is the fast path when the
-// source's contiguous axis runs along p (CHWN with batch-minor tiles) and the
-// fallback elsewhere.
+// One thread per (tile p, channel vector cq), p fastest: every store is a
+// 16-byte vector and a wave's stores form a contiguous 1 KB run of V.  Reads go
+// through the activation strides, so the kernel is correct for every layout and
+// tile order; it is the fast path when the source's contiguous axis runs along
+// p (NCHW rows, CHWN with batch-minor tiles).
 template <typename T>
 __global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* __restrict__ x, T* __restrict__ V,
                                                                        ActStrides s, int N, int C, int H, int W,
                                                                        int pad, int th, int tw, long P, long Pp,
                                                                        int Cp, int order) {
-    long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    int c = blockIdx.y;
+    constexpr int CV = ChanVec<T>::n;
+    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int cq = blockIdx.y;
     if (p >= P) return;
-    float v[4][4];
-    if (c < C) {
-        int n, ty, tx;
-        decode_tile(p, order, N, th, tw, n, ty, tx);
-        const int h0 = 2 * ty - pad, w0 = 2 * tx - pad;
-        const T* xp = x + n * s.n + c * s.c;
-        float d[4][4];
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    const int h0 = 2 * ty - pad, w0 = 2 * tx - pad;
+    float v[CV][16];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+    for (int e = 0; e < CV; ++e) {
+        const int c = cq * CV + e;
+        if (c < C) {
+            const T* xp = x + n * s.n + c * s.c;
+            float d[4][4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                int ih = h0 + i, iw = w0 + j;
-                bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
-                d[i][j] = ok ? to_f32(xp[ih * s.h + iw * s.w]) : 0.f;
-            }
-        input_tile_transform(d, v);
-    } else {
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i / 4][i % 4] = 0.f;
+                for (int j = 0; j < 4; ++j) {
+                    const int ih = h0 + i, iw = w0 + j;
+                    const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
+                    d[i][j] = ok ? to_f32(xp[ih * s.h + iw * s.w]) : 0.f;
+                }
+            input_tile_transform(d, v[e]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[e][i] = 0.f;
+        }
     }
     const size_t plane = (size_t)Cp * Pp;
-    T* vp = V + (size_t)c * Pp + p;
+    T* vp = V + ((size_t)cq * Pp + p) * CV;
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi) vp[xi * plane] = from_f32<T>(v[xi / 4][xi % 4]);
+    for (int xi = 0; xi < 16; ++xi) {
+        float o[CV];
+#pragma unroll
+        for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
+        store_chan_vec<T>(vp + xi * plane, o);
+    }
 }
 
 // ---- output transform, layout-generic ---------------------------------------------
 // One thread per (tile p, filter k), p fastest: the 16 loads of a wave are
-// contiguous runs of Mo.  Stores go through the destination strides.
+// contiguous runs of Mo[xi][k][.].  Stores go through the destination strides.
 template <typename T>
 __global__ __launch_bounds__(256) void output_transform_generic_kernel(const float* __restrict__ Mo,
                                                                         T* __restrict__ y, ActStrides s, int N,
                                                                         int K, int Ho, int Wo, int th, int tw,
                                                                         long P, long Pp, int Kp, int order,
                                                                         int relu) {
-    long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    int k = blockIdx.y;
+    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int k = blockIdx.y;
     if (p >= P || k >= K) return;
     const size_t plane = (size_t)Kp * Pp;
     const float* mp = Mo + (size_t)k * Pp + p;
@@ -156,7 +180,7 @@ __global__ __launch_bounds__(256) void output_transform_generic_kernel(const flo
     for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
-            int oh = 2 * ty + a, ow = 2 * tx + b;
+            const int oh = 2 * ty + a, ow = 2 * tx + b;
             if (oh < Ho && ow < Wo) {
                 float val = o[a][b];
                 if (relu) val = fmaxf(val, 0.f);

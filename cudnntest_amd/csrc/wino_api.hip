@@ -123,7 +123,7 @@ Scratch scratch_layout(const Geometry& g, int dtype) {
 // ---- stage launchers (typed) -------------------------------------------------------
 template <typename T>
 int launch_filter_transform(int layout, int K, int C, int Kp, int Cp, const void* w, void* U, hipStream_t st) {
-    dim3 grid((Kp + 255) / 256, Cp), block(256);
+    dim3 grid((Kp + 255) / 256, Cp / ChanVec<T>::n), block(256);
     hipLaunchKernelGGL(filter_transform_kernel<T>, grid, block, 0, st, (const T*)w, (T*)U, flt_strides(layout, K, C),
                        K, C, Kp, Cp);
     LAUNCH_CHECK("filter_transform");
@@ -132,7 +132,7 @@ int launch_filter_transform(int layout, int K, int C, int Kp, int Cp, const void
 
 template <typename T>
 int launch_input_transform(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st) {
-    dim3 grid((unsigned)((g.P + 255) / 256), g.Cp), block(256);
+    dim3 grid((unsigned)((g.P + 255) / 256), g.Cp / ChanVec<T>::n), block(256);
     hipLaunchKernelGGL(input_transform_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
                        act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
                        g.Cp, order);
@@ -152,18 +152,32 @@ int launch_output_transform(int layout, int order, unsigned flags, int N, int K,
     return WINO_OK;
 }
 
-int launch_gemm(int dtype, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
-    if (dtype != WINO_F32) return fail(WINO_ERR_UNSUPPORTED, "batched GEMM: dtype %d not built yet", dtype);
+template <typename T, int NV>
+int launch_gemm_t(int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
     dim3 grid((unsigned)(Pp / GEMM_BN), Kp / GEMM_BM, 16), block(256);
-    hipLaunchKernelGGL(gemm_f32_128x128_kernel, grid, block, 0, st, (const float*)U, (const float*)V, Mo, Cp, Kp, Pp);
+    hipLaunchKernelGGL((gemm_128x128_kernel<T, NV>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp, Kp, Pp);
     LAUNCH_CHECK("batched_gemm");
     return WINO_OK;
 }
 
-template <typename OutT, bool SWAP>
-int launch_gemm_out_t(int order, unsigned flags, const Geometry& g, const float* U, const float* V, void* y,
-                      int dst, hipStream_t st) {
-    auto kern = gemm_out_f32_kernel<OutT, SWAP>;
+int launch_gemm(int dtype, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
+    // slab per barrier: 16 channels (fp32, 4 vectors) or 32 channels (16-bit, 4 vectors); Cp is a multiple of 16
+    switch (dtype) {
+    case WINO_F32: return launch_gemm_t<float, 4>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_F16:
+        return Cp % 32 == 0 ? launch_gemm_t<f16_t, 4>(Cp, Kp, Pp, U, V, Mo, st)
+                            : launch_gemm_t<f16_t, 2>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_BF16:
+        return Cp % 32 == 0 ? launch_gemm_t<bf16_t, 4>(Cp, Kp, Pp, U, V, Mo, st)
+                            : launch_gemm_t<bf16_t, 2>(Cp, Kp, Pp, U, V, Mo, st);
+    }
+    return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+template <typename T, bool SWAP>
+int launch_gemm_out_t(int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y, int dst,
+                      hipStream_t st) {
+    auto kern = gemm_out_kernel<T, SWAP>;
     static bool attr_set = false;   // per instantiation
     if (!attr_set) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -174,19 +188,28 @@ int launch_gemm_out_t(int order, unsigned flags, const Geometry& g, const float*
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
-    hipLaunchKernelGGL(kern, grid, block, GO_LDS_BYTES, st, U, V, (OutT*)y, act_strides(dst, g.N, g.K, g.Ho, g.Wo),
-                       g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, g.Pp, order,
-                       (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
+    hipLaunchKernelGGL(kern, grid, block, GO_LDS_BYTES, st, (const T*)U, (const T*)V, (T*)y,
+                       act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
+                       g.Pp, order, (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
     LAUNCH_CHECK("gemm_output");
     return WINO_OK;
 }
 
+template <typename T>
+int launch_gemm_out_d(int dst, int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y,
+                      hipStream_t st) {
+    if (dst == WINO_NHWC) return launch_gemm_out_t<T, true>(order, flags, g, U, V, y, dst, st);
+    return launch_gemm_out_t<T, false>(order, flags, g, U, V, y, dst, st);
+}
+
 int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* U, const void* V,
                     void* y, hipStream_t st) {
-    if (dtype != WINO_F32) return fail(WINO_ERR_UNSUPPORTED, "epilogue-fused GEMM: dtype %d not built yet", dtype);
-    if (dst == WINO_NHWC)
-        return launch_gemm_out_t<float, true>(order, flags, g, (const float*)U, (const float*)V, y, dst, st);
-    return launch_gemm_out_t<float, false>(order, flags, g, (const float*)U, (const float*)V, y, dst, st);
+    switch (dtype) {
+    case WINO_F32: return launch_gemm_out_d<float>(dst, order, flags, g, U, V, y, st);
+    case WINO_F16: return launch_gemm_out_d<f16_t>(dst, order, flags, g, U, V, y, st);
+    case WINO_BF16: return launch_gemm_out_d<bf16_t>(dst, order, flags, g, U, V, y, st);
+    }
+    return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
 #define DISPATCH_DTYPE(dtype, CALL)                          \
@@ -197,11 +220,10 @@ int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometr
     default: return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype); \
     }
 
-int tile_order_for(int src, int dst) {
-    // batch-minor tiles keep both the CHWN reads and the CHWN writes contiguous
-    if (src == WINO_CHWN) return WINO_TILES_BATCH_MINOR;
-    if (dst == WINO_CHWN && src != WINO_NHWC) return WINO_TILES_BATCH_MAJOR;
-    return WINO_TILES_BATCH_MAJOR;
+int tile_order_for(int src, int /*dst*/) {
+    // The tile order follows the source: batch-minor keeps CHWN reads (and CHWN
+    // writes, when the destination is CHWN too) contiguous along n.
+    return src == WINO_CHWN ? WINO_TILES_BATCH_MINOR : WINO_TILES_BATCH_MAJOR;
 }
 
 int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,

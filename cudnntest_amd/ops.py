@@ -138,27 +138,29 @@ def conv_prepared(x, U, K, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False
 # ---- stages ------------------------------------------------------------------------
 
 def filter_transform(w, layout=NCHW):
-    """U[16][Cp][Kp] = G g G^T (padding zero-filled)."""
+    """U[16][Cp/CV][Kp][CV] = G g G^T (padding zero-filled); CV = 4 (fp32) or 8 (f16/bf16)."""
     K, C = flt_dims(layout, w)
     g = geometry(_dt(w), 1, C, K, 4, 4, 1)
-    U = torch.empty((16, g["Cp"], g["Kp"]), dtype=w.dtype, device=w.device)
+    cv = 16 // w.element_size()
+    U = torch.empty((16, g["Cp"] // cv, g["Kp"], cv), dtype=w.dtype, device=w.device)
     _lib.check(_lib.load().wino_filter_transform(int(layout), _dt(w), K, C, _ptr(w), _ptr(U), _stream()),
                "wino_filter_transform")
     return U
 
 
 def input_transform(x, pad=1, layout=NCHW, tile_order=TILES_BATCH_MAJOR):
-    """V[16][Cp][Pp] = B^T d B; columns p >= P are left as allocated (zeros here)."""
+    """V[16][Cp/CV][Pp][CV] = B^T d B; columns p >= P are left as allocated (zeros here)."""
     N, C, H, W = act_dims(layout, x)
     g = geometry(_dt(x), N, C, 1, H, W, pad)
-    V = torch.zeros((16, g["Cp"], g["Pp"]), dtype=x.dtype, device=x.device)
+    cv = 16 // x.element_size()
+    V = torch.zeros((16, g["Cp"] // cv, g["Pp"], cv), dtype=x.dtype, device=x.device)
     _lib.check(_lib.load().wino_input_transform(int(layout), _dt(x), tile_order, N, C, H, W, pad, _ptr(x), _ptr(V),
                                                 _stream()), "wino_input_transform")
     return V
 
 
 def batched_gemm(U, V, C, K, P):
-    """Mo[16][Kp][Pp] (fp32) = sum_c U[xi][c][k] V[xi][c][p]."""
+    """Mo[16][Kp][Pp] (fp32) = sum_c U[xi][c][k] V[xi][c][p]; U, V in channel-vector layout."""
     Mo = torch.empty((16, U.shape[2], V.shape[2]), dtype=torch.float32, device=U.device)
     _lib.check(_lib.load().wino_batched_gemm(_dt(U), C, K, P, _ptr(U), _ptr(V), _ptr(Mo), _stream()),
                "wino_batched_gemm")

@@ -78,9 +78,13 @@ int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, in
                        int H, int W, int pad, const void *x, const void *U, void *y, void *stream);
 
 /* ---- padded operand geometry ------------------------------------------------
- * U is [16][Cp][Kp], V is [16][Cp][Pp], the GEMM product Mo is [16][Kp][Pp]
- * (fp32), with th = ceil(Ho/2), tw = ceil(Wo/2), P = N*th*tw.  The counterpart
- * of MSize/NSize/KSize at comparison/wrapedConv_NCHW.cuh:346-362. */
+ * With th = ceil(Ho/2), tw = ceil(Wo/2), P = N*th*tw and CV = 16/sizeof(element)
+ * (4 channels per 16-byte vector for fp32, 8 for f16/bf16):
+ *   U   [16][Cp/CV][Kp][CV]   transformed filters, channel vectors innermost
+ *   V   [16][Cp/CV][Pp][CV]   transformed input tiles
+ *   Mo  [16][Kp][Pp]          GEMM product, always fp32
+ * Cp, Kp, Pp are C, K, P rounded up to 16, 128, 128.  The counterpart of
+ * MSize/NSize/KSize at comparison/wrapedConv_NCHW.cuh:346-362. */
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int *th, int *tw,
                   long *P, int *Cp, int *Kp, long *Pp);
 

@@ -34,3 +34,18 @@ def batch_minor_perm(N, th, tw):
     perm = np.empty(N * th * tw, np.int64)
     perm[p_minor] = p_major
     return perm
+
+
+def unpack_operand(t, dtype=ops.F32):
+    """[16][Cp/CV][X][CV] (channel vectors innermost) -> numpy [16][Cp][X]."""
+    a = host(t)
+    xi, cq, X, cv = a.shape
+    return np.ascontiguousarray(a.transpose(0, 1, 3, 2).reshape(xi, cq * cv, X))
+
+
+def pack_operand(a, dtype=ops.F32):
+    """numpy [16][Cp][X] -> device [16][Cp/CV][X][CV]."""
+    cv = 4 if dtype == ops.F32 else 8
+    xi, Cp, X = a.shape
+    assert Cp % cv == 0
+    return dev(np.ascontiguousarray(a.reshape(xi, Cp // cv, cv, X).transpose(0, 1, 3, 2)), dtype)

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from cudnntest_amd import ops, synth
-from gpu_util import batch_minor_perm, dev, host
+from gpu_util import batch_minor_perm, dev, host, pack_operand, unpack_operand
 
 pytestmark = pytest.mark.gpu
 LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
@@ -23,14 +23,14 @@ LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
 def test_filter_transform(oracle, layout, K, C):
     w = synth.small_ints(K * C * 9, 31 + K + C, -4, 4).reshape(K, C, 3, 3)
     wl = synth.flt_to_layout(w, layout)
-    U = host(ops.filter_transform(dev(wl), layout))
+    U = unpack_operand(ops.filter_transform(dev(wl), layout))
     want = oracle.wino_filter_transform(wl, layout)
     assert np.array_equal(U[:, :C, :K], want)
     assert not U[:, C:, :].any() and not U[:, :, K:].any(), "padding must be zero"
     # float data: same arithmetic order is not promised, closeness is
     wf = synth.normal(K * C * 9, 5, 0.1).reshape(K, C, 3, 3)
     wfl = synth.flt_to_layout(wf, layout)
-    Uf = host(ops.filter_transform(dev(wfl), layout))[:, :C, :K]
+    Uf = unpack_operand(ops.filter_transform(dev(wfl), layout))[:, :C, :K]
     np.testing.assert_allclose(Uf, oracle.wino_filter_transform(wfl, layout), rtol=1e-6, atol=1e-7)
 
 
@@ -42,7 +42,7 @@ def test_input_transform(oracle, layout, order, shape, pad):
     N, C, H, W = shape
     x = synth.small_ints(N * C * H * W, 77 + sum(shape), -8, 8).reshape(N, C, H, W)
     xl = synth.act_to_layout(x, layout)
-    V = host(ops.input_transform(dev(xl), pad, layout, order))
+    V = unpack_operand(ops.input_transform(dev(xl), pad, layout, order))
     want = oracle.wino_input_transform(xl, pad, layout)          # batch-major columns
     th, tw = oracle.wino_tiles(2, H, W, pad)
     P = N * th * tw
@@ -62,7 +62,7 @@ def test_batched_gemm(oracle, C, K, P):
     V = np.zeros((16, Cp, Pp), np.float32)
     U[:, :C, :K] = synth.small_ints(16 * C * K, 3, -3, 3).reshape(16, C, K)
     V[:, :C, :P] = synth.small_ints(16 * C * P, 4, -5, 5).reshape(16, C, P)
-    Mo = host(ops.batched_gemm(dev(U), dev(V), C, K, P))
+    Mo = host(ops.batched_gemm(pack_operand(U), pack_operand(V), C, K, P))
     want = oracle.wino_gemm(np.ascontiguousarray(U[:, :C, :K]), np.ascontiguousarray(V[:, :C, :P]))
     assert np.array_equal(Mo[:, :K, :P], want)
 
@@ -71,7 +71,7 @@ def test_batched_gemm_floats(oracle):
     C, K, P = 64, 128, 256
     U = synth.normal(16 * C * K, 8, 0.2).reshape(16, C, K)
     V = synth.uniform_pm1(16 * C * P, 9).reshape(16, C, P)
-    Mo = host(ops.batched_gemm(dev(U), dev(V), C, K, P))
+    Mo = host(ops.batched_gemm(pack_operand(U), pack_operand(V), C, K, P))
     assert oracle.rel_l2(Mo, oracle.wino_gemm(U, V)) < 1e-6
 
 
@@ -113,7 +113,7 @@ def test_gemm_with_output_epilogue(oracle, layout, order, N, C, K, Ho, Wo, relu)
     V = np.zeros((16, Cp, Pp), np.float32)
     U[:, :C, :K] = Uc
     V[:, :C, :P] = Vc[:, :, batch_minor_perm(N, th, tw)] if order == ops.TILES_BATCH_MINOR else Vc
-    y = host(ops.gemm_output(dev(U), dev(V), N, C, K, Ho, Wo, layout, order, relu))
+    y = host(ops.gemm_output(pack_operand(U), pack_operand(V), N, C, K, Ho, Wo, layout, order, relu))
     want = oracle.wino_output_transform(oracle.wino_gemm(Uc, Vc), N, Ho, Wo, layout)
     if relu:
         want = np.maximum(want, 0)
