@@ -8,7 +8,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libwino_amd.so")
+# WINO_AMD_LIB selects another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("WINO_AMD_LIB") or os.path.join(_HERE, "libwino_amd.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 _vp = ctypes.c_void_p

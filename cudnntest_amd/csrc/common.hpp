@@ -79,7 +79,8 @@ template <typename T> __device__ __forceinline__ void store_chan_vec(T* dst, con
 }
 
 // ---- padded geometry ---------------------------------------------------------
-constexpr int kCPad = 16;    // reduction (channel) dimension of U and V is padded to this
+// the reduction (channel) dimension of U and V is padded to 4 channel vectors (two k-groups)
+__host__ inline int c_pad(int dtype) { return 4 * chan_vec(dtype); }   // 16 (fp32) or 32 (f16/bf16)
 constexpr int kKPad = 128;   // filter dimension of U / Mo
 constexpr int kPPad = 128;   // tile dimension of V / Mo
 
@@ -93,7 +94,7 @@ struct Geometry {
 
 __host__ inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
 
-__host__ inline bool make_geometry(int N, int C, int K, int H, int W, int pad, Geometry* g) {
+__host__ inline bool make_geometry(int dtype, int N, int C, int K, int H, int W, int pad, Geometry* g) {
     if (N <= 0 || C <= 0 || K <= 0 || H <= 0 || W <= 0 || pad < 0 || pad > 1) return false;
     g->N = N; g->C = C; g->K = K; g->H = H; g->W = W; g->pad = pad;
     g->Ho = H + 2 * pad - 2;
@@ -102,7 +103,7 @@ __host__ inline bool make_geometry(int N, int C, int K, int H, int W, int pad, G
     g->th = (g->Ho + 1) / 2;
     g->tw = (g->Wo + 1) / 2;
     g->P = (long)N * g->th * g->tw;
-    g->Cp = (int)round_up(C, kCPad);
+    g->Cp = (int)round_up(C, c_pad(dtype));
     g->Kp = (int)round_up(K, kKPad);
     g->Pp = round_up(g->P, kPPad);
     return true;

@@ -15,6 +15,8 @@
 // channels for f16/bf16 (one MFMA).  The sum over channels does not care which
 // channel a lane half takes as long as both operands agree.
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 #include "transforms.hpp"
 
@@ -162,7 +164,6 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
 // one tile patch first; the V slab they share then stays in that XCD's L2.
 // =============================================================================
 constexpr int GO_T = 64;   // patch edge (filters and tiles)
-constexpr size_t GO_LDS_BYTES = 2ull * 2 * 16 * 2 * GO_T * 16;   // stages x operands x xi x 2 vectors x 64 x 16 B
 
 template <typename OutT>
 __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const ActStrides& ys, int n, int k, int ty,
@@ -189,10 +190,10 @@ __global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, 
                                                        int relu, int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
-    extern __shared__ __attribute__((aligned(16))) unsigned char go_smem[];
-    typedef vec (*slab_t)[16][2][GO_T];
-    slab_t Us = reinterpret_cast<slab_t>(go_smem);
-    slab_t Vs = reinterpret_cast<slab_t>(go_smem + GO_LDS_BYTES / 2);
+    // two stages, each a U slab and a V slab of [xi][lane half][64] channel vectors (4 x 32 KB);
+    // separate arrays so the compiler can tell the stage being filled from the stage being read
+    __shared__ vec Us0[16][2][GO_T], Us1[16][2][GO_T];
+    __shared__ vec Vs0[16][2][GO_T], Vs1[16][2][GO_T];
 
     const int b = blockIdx.x;
     const int xcd = b & 7, j = b >> 3;
@@ -216,45 +217,59 @@ __global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, 
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[xi][r] = 0.f;
 
-    // HBM -> LDS: per operand 32 rows (xi, half) of 64 vectors = 2048 vectors, 8 per thread
-    vec ru[8], rv[8];
-    const int col = tid & 63;
-    const int rbase = tid >> 6;          // 0..3, rows rbase + 4*i
-    auto gload = [&](int g) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = rbase + 4 * i;     // 0..31
-            const int xi = row >> 1, h = row & 1;
-            ru[i] = Ug[((size_t)xi * CQ + 2 * g + h) * Kp + k0 + col];
-            rv[i] = Vg[((size_t)xi * CQ + 2 * g + h) * Pp + p0 + col];
-        }
-    };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = rbase + 4 * i;
-            Us[buf][row >> 1][row & 1][col] = ru[i];
-            Vs[buf][row >> 1][row & 1][col] = rv[i];
-        }
-    };
-
+    // HBM -> LDS without passing through registers: one global_load_lds_dwordx4 moves a
+    // whole (xi, lane-half) row of 64 channel vectors (lane l -> LDS row base + 16*l).
+    // A stage is 64 such rows (32 of U, 32 of V); wave w issues rows w, w+4, ...
     const int ngrp = CQ / 2;
-    gload(0);
-    lstore(0);
-    __syncthreads();
-
-    for (int g = 0; g < ngrp; ++g) {
-        const int buf = g & 1;
-        if (g + 1 < ngrp) gload(g + 1);
+    typedef std::integral_constant<int, 0> par0_t;
+    typedef std::integral_constant<int, 1> par1_t;
+    auto stage_load = [&](auto par, int g) {
+        constexpr int S = decltype(par)::value;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = wave + 4 * i;            // 0..31, wave-uniform
+            const int xi = row >> 1, h = row & 1;
+            const vec* usrc = Ug + ((size_t)xi * CQ + 2 * g + h) * Kp + k0 + lane;
+            const vec* vsrc = Vg + ((size_t)xi * CQ + 2 * g + h) * Pp + p0 + lane;
+            vec* udst = S ? &Us1[xi][h][0] : &Us0[xi][h][0];
+            vec* vdst = S ? &Vs1[xi][h][0] : &Vs0[xi][h][0];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)usrc,
+                                             (__attribute__((address_space(3))) void*)udst, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc,
+                                             (__attribute__((address_space(3))) void*)vdst, 16, 0, 0);
+        }
+    };
+    // One k-group per iteration: start the next stage's loads, multiply the
+    // current stage (fragments fetched two coordinates ahead of their MFMAs),
+    // then wait for the loads and meet the other waves.
+    vec fu[3], fv[3];
+    auto iteration = [&](auto par, int g) {
+        constexpr int S = decltype(par)::value;
+        auto frag_load = [&](int xi) {
+            fu[xi % 3] = S ? Us1[xi][lh][(SWAP ? wn : wm) * 32 + l32] : Us0[xi][lh][(SWAP ? wn : wm) * 32 + l32];
+            fv[xi % 3] = S ? Vs1[xi][lh][(SWAP ? wm : wn) * 32 + l32] : Vs0[xi][lh][(SWAP ? wm : wn) * 32 + l32];
+        };
+        stage_load(std::integral_constant<int, 1 - S>{}, g + 1 < ngrp ? g + 1 : g);   // surplus load never read
+        frag_load(0);
+        frag_load(1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int xi = 0; xi < 16; ++xi) {
-            const vec fu = Us[buf][xi][lh][(SWAP ? wn : wm) * 32 + l32];
-            const vec fv = Vs[buf][xi][lh][(SWAP ? wm : wn) * 32 + l32];
-            if (SWAP) Mma<T>::run(fv, fu, acc[xi]);
-            else Mma<T>::run(fu, fv, acc[xi]);
+            if (xi + 2 < 16) frag_load(xi + 2);
+            if (SWAP) Mma<T>::run(fv[xi % 3], fu[xi % 3], acc[xi]);
+            else Mma<T>::run(fu[xi % 3], fv[xi % 3], acc[xi]);
         }
-        if (g + 1 < ngrp) lstore(buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's rows of the next stage are in LDS
         __syncthreads();
+    };
+
+    stage_load(par0_t{}, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    for (int g = 0; g < ngrp; g += 2) {   // ngrp is even: Cp is a multiple of 4 channel vectors
+        iteration(par0_t{}, g);
+        iteration(par1_t{}, g + 1);
     }
 
     // ---- epilogue: A^T (.) A on the 16 accumulators, then store ----------------------

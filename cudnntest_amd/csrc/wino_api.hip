@@ -161,15 +161,11 @@ int launch_gemm_t(int Cp, int Kp, long Pp, const void* U, const void* V, float* 
 }
 
 int launch_gemm(int dtype, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
-    // slab per barrier: 16 channels (fp32, 4 vectors) or 32 channels (16-bit, 4 vectors); Cp is a multiple of 16
+    // slab per barrier: 4 channel vectors = 16 channels (fp32) or 32 (16-bit); Cp is a multiple of that
     switch (dtype) {
     case WINO_F32: return launch_gemm_t<float, 4>(Cp, Kp, Pp, U, V, Mo, st);
-    case WINO_F16:
-        return Cp % 32 == 0 ? launch_gemm_t<f16_t, 4>(Cp, Kp, Pp, U, V, Mo, st)
-                            : launch_gemm_t<f16_t, 2>(Cp, Kp, Pp, U, V, Mo, st);
-    case WINO_BF16:
-        return Cp % 32 == 0 ? launch_gemm_t<bf16_t, 4>(Cp, Kp, Pp, U, V, Mo, st)
-                            : launch_gemm_t<bf16_t, 2>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_F16: return launch_gemm_t<f16_t, 4>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_BF16: return launch_gemm_t<bf16_t, 4>(Cp, Kp, Pp, U, V, Mo, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -178,17 +174,11 @@ template <typename T, bool SWAP>
 int launch_gemm_out_t(int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y, int dst,
                       hipStream_t st) {
     auto kern = gemm_out_kernel<T, SWAP>;
-    static bool attr_set = false;   // per instantiation
-    if (!attr_set) {
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)GO_LDS_BYTES));
-        attr_set = true;
-    }
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
-    hipLaunchKernelGGL(kern, grid, block, GO_LDS_BYTES, st, (const T*)U, (const T*)V, (T*)y,
+    hipLaunchKernelGGL(kern, grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
                        act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
                        g.Pp, order, (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
     LAUNCH_CHECK("gemm_output");
@@ -233,7 +223,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_FUSED) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
     if (!x || (!w && !Upre) || !y) return fail(WINO_ERR_INVALID, "null tensor pointer");
     Geometry g;
-    if (!make_geometry(N, C, K, H, W, pad, &g))
+    if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     if (algo == WINO_ALGO_AUTO) algo = WINO_ALGO_STAGED;
     if (algo == WINO_ALGO_FUSED) return fail(WINO_ERR_UNSUPPORTED, "algo %d not built yet", algo);
@@ -296,7 +286,7 @@ int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th
                   long* Pp) {
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     Geometry g;
-    if (!make_geometry(N, C, K, H, W, pad, &g))
+    if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     if (th) *th = g.th;
     if (tw) *tw = g.tw;
@@ -309,7 +299,7 @@ int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th
 
 size_t wino_workspace_bytes(int dtype, int N, int C, int K, int H, int W, int pad) {
     Geometry g;
-    if (!valid_dtype(dtype) || !make_geometry(N, C, K, H, W, pad, &g)) {
+    if (!valid_dtype(dtype) || !make_geometry(dtype, N, C, K, H, W, pad, &g)) {
         fail(WINO_ERR_INVALID, "bad shape or dtype");
         return 0;
     }
@@ -331,7 +321,8 @@ int wino_filter_transform(int layout, int dtype, int K, int C, const void* w, vo
     if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
     if (!w || !U) return fail(WINO_ERR_INVALID, "null pointer");
     if (K <= 0 || C <= 0) return fail(WINO_ERR_INVALID, "bad filter bank K=%d C=%d", K, C);
-    const int Kp = (int)round_up(K, kKPad), Cp = (int)round_up(C, kCPad);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    const int Kp = (int)round_up(K, kKPad), Cp = (int)round_up(C, c_pad(dtype));
     DISPATCH_DTYPE(dtype, launch_filter_transform<T>(layout, K, C, Kp, Cp, w, U, (hipStream_t)stream));
 }
 
@@ -341,7 +332,7 @@ int wino_input_transform(int layout, int dtype, int tile_order, int N, int C, in
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!x || !V) return fail(WINO_ERR_INVALID, "null pointer");
     Geometry g;
-    if (!make_geometry(N, C, 1, H, W, pad, &g))
+    if (!make_geometry(dtype, N, C, 1, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d H=%d W=%d pad=%d", N, C, H, W, pad);
     DISPATCH_DTYPE(dtype, launch_input_transform<T>(layout, tile_order, g, x, V, (hipStream_t)stream));
 }
@@ -350,7 +341,7 @@ int wino_batched_gemm(int dtype, int C, int K, long P, const void* U, const void
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
     if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
-    return launch_gemm(dtype, (int)round_up(C, kCPad), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
+    return launch_gemm(dtype, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
                        (hipStream_t)stream);
 }
 
@@ -376,7 +367,7 @@ int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int 
     if (!U || !V || !y) return fail(WINO_ERR_INVALID, "null pointer");
     Geometry g;
     // geometry from the output size: pad 1 keeps H == Ho
-    if (!make_geometry(N, C, K, Ho, Wo, 1, &g))
+    if (!make_geometry(dtype, N, C, K, Ho, Wo, 1, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d Ho=%d Wo=%d", N, C, K, Ho, Wo);
     return launch_gemm_out(layout, dtype, tile_order, flags, g, U, V, y, (hipStream_t)stream);
 }

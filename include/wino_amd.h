@@ -83,7 +83,8 @@ int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, in
  *   U   [16][Cp/CV][Kp][CV]   transformed filters, channel vectors innermost
  *   V   [16][Cp/CV][Pp][CV]   transformed input tiles
  *   Mo  [16][Kp][Pp]          GEMM product, always fp32
- * Cp, Kp, Pp are C, K, P rounded up to 16, 128, 128.  The counterpart of
+ * Cp is C rounded up to 4 channel vectors (16 for fp32, 32 for f16/bf16); Kp and Pp are K
+ * and P rounded up to 128.  The counterpart of
  * MSize/NSize/KSize at comparison/wrapedConv_NCHW.cuh:346-362. */
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int *th, int *tw,
                   long *P, int *Cp, int *Kp, long *Pp);
