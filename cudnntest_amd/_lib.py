@@ -27,8 +27,8 @@ SYMBOLS = {
     "wino_set_workspace": (_i, [_vp, ctypes.c_size_t]),
     "wino_filter_transform": (_i, [_i, _i, _i, _i, _vp, _vp, _vp]),
     "wino_input_transform": (_i, [_i] * 8 + [_vp, _vp, _vp]),
-    "wino_batched_gemm": (_i, [_i, _i, _i, _l, _vp, _vp, _vp, _vp]),
-    "wino_output_transform": (_i, [_i, _i, _i, _u, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "wino_batched_gemm": (_i, [_i, _i, _i, _i, _l, _vp, _vp, _vp, _vp]),
+    "wino_output_transform": (_i, [_i, _i, _i, _i, _u, _i, _i, _i, _i, _vp, _vp, _vp]),
     "wino_gemm_output": (_i, [_i, _i, _i, _u, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "wino_layout_transform": (_i, [_i] * 7 + [_vp, _vp, _vp]),
     "wino_stage_timing": (_i, [_i]),

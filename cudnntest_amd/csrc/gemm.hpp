@@ -59,7 +59,10 @@ template <> struct Mma<bf16_t> {
 // =============================================================================
 constexpr int GEMM_BM = 128, GEMM_BN = 128;
 
-template <typename T, int NV>
+// PK = false: product stored as Mo[xi][Kp][Pp] (MFMA rows = filters, lanes = tiles)
+// PK = true : product stored as Mo[xi][Pp][Kp] (MFMA rows = tiles, lanes = filters), for
+//             destinations whose contiguous axis is K (NHWC)
+template <typename T, int NV, bool PK>
 __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__ U, const T* __restrict__ V,
                                                             float* __restrict__ Mo, int Cp, int Kp, long Pp) {
     typedef typename Mma<T>::vec vec;
@@ -118,8 +121,13 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
             vec a[2], b[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                a[t] = As[buf][2 * g + lh][wm * 64 + t * 32 + l32];
-                b[t] = Bs[buf][2 * g + lh][wn * 64 + t * 32 + l32];
+                if (PK) {
+                    a[t] = Bs[buf][2 * g + lh][wm * 64 + t * 32 + l32];
+                    b[t] = As[buf][2 * g + lh][wn * 64 + t * 32 + l32];
+                } else {
+                    a[t] = As[buf][2 * g + lh][wm * 64 + t * 32 + l32];
+                    b[t] = Bs[buf][2 * g + lh][wn * 64 + t * 32 + l32];
+                }
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
@@ -137,9 +145,10 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = k0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                const long col = p0 + wn * 64 + j * 32 + l32;
-                Mb[(size_t)row * Pp + col] = acc[i][j][r];
+                const int ri = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);   // MFMA row
+                const int ci = wn * 64 + j * 32 + l32;                               // MFMA column (lane)
+                if (PK) Mb[(size_t)(p0 + ri) * Kp + k0 + ci] = acc[i][j][r];
+                else Mb[(size_t)(k0 + ri) * Pp + p0 + ci] = acc[i][j][r];
             }
 }
 

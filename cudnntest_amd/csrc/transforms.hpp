@@ -154,6 +154,161 @@ __global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* _
     }
 }
 
+// ---- input transform, NCHW source, LDS-staged ----------------------------------------
+// A workgroup takes one image n, one channel vector cq and a TR x TC block of
+// tiles.  The (2*TR+2) x (2*TC+2) input halo of each of its CV channels is read
+// once, along W (contiguous), into LDS with the zero padding materialised; each
+// thread then builds its tile from LDS with 8-byte reads (conflict-free: lanes
+// walk tx, two columns apart) and issues 16 coalesced 16-byte stores.
+template <typename T>
+__global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __restrict__ x, T* __restrict__ V, int N,
+                                                                   int C, int H, int W, int pad, int th, int tw,
+                                                                   long Pp, int Cp, int TR, int TC, int colBlocks,
+                                                                   int chunkLog2) {
+    constexpr int CV = ChanVec<T>::n;
+    extern __shared__ float in_smem[];   // [CV][rows][ldsW]
+    const int cq = blockIdx.y, n = blockIdx.z;
+    const int rb = blockIdx.x / colBlocks, cb = blockIdx.x % colBlocks;
+    const int ty0 = rb * TR, tx0 = cb * TC;
+    const int rows = 2 * TR + 2;
+    const int ldsW = 2 * TC + 2;          // even
+    const int h0 = 2 * ty0 - pad, w0 = 2 * tx0 - pad;
+    const int tid = threadIdx.x;
+
+    const int per_ch = rows * ldsW;
+    // Halo copy.  A unit is 64 consecutive columns of one halo row; wave w takes
+    // units w, w+4, ...  Loads are issued in batches of CV x MAXU before any of
+    // them is written to LDS, so a wave keeps that many HBM requests in flight.
+    const int lane = tid & 63, wv = tid >> 6;
+    constexpr int MAXU = 6;
+    const int nunits = rows << chunkLog2;
+    const int cmask = (1 << chunkLog2) - 1;
+    for (int u0 = 0; u0 < nunits; u0 += 4 * MAXU) {
+        float buf[CV][MAXU];
+#pragma unroll
+        for (int i = 0; i < MAXU; ++i) {
+            const int u = u0 + wv + 4 * i;
+            const int r = u >> chunkLog2, q = ((u & cmask) << 6) + lane;
+            const int ih = h0 + r, iw = w0 + q;
+            const bool ok = u < nunits && q < ldsW && ih >= 0 && ih < H && iw >= 0 && iw < W;
+#pragma unroll
+            for (int ch = 0; ch < CV; ++ch) {
+                const int c = cq * CV + ch;
+                buf[ch][i] = (ok && c < C) ? to_f32(x[(((size_t)n * C + c) * H + ih) * W + iw]) : 0.f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MAXU; ++i) {
+            const int u = u0 + wv + 4 * i;
+            const int r = u >> chunkLog2, q = ((u & cmask) << 6) + lane;
+            if (u < nunits && q < ldsW) {
+#pragma unroll
+                for (int ch = 0; ch < CV; ++ch) in_smem[ch * per_ch + r * ldsW + q] = buf[ch][i];
+            }
+        }
+    }
+    __syncthreads();
+
+    const int tr = tid / TC, tc = tid % TC;
+    const int ty = ty0 + tr, tx = tx0 + tc;
+    if (tr >= TR || ty >= th || tx >= tw) return;
+    float v[CV][16];
+#pragma unroll
+    for (int ch = 0; ch < CV; ++ch) {
+        float d[4][4];
+        const float* base = in_smem + ch * per_ch + (2 * tr) * ldsW + 2 * tc;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float2 a = *reinterpret_cast<const float2*>(base + i * ldsW);
+            const float2 b = *reinterpret_cast<const float2*>(base + i * ldsW + 2);
+            d[i][0] = a.x; d[i][1] = a.y; d[i][2] = b.x; d[i][3] = b.y;
+        }
+        input_tile_transform(d, v[ch]);
+    }
+    const long p = ((long)n * th + ty) * tw + tx;
+    const size_t plane = (size_t)Cp * Pp;
+    T* vp = V + ((size_t)cq * Pp + p) * CV;
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) {
+        float o[CV];
+#pragma unroll
+        for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
+        store_chan_vec<T>(vp + xi * plane, o);
+    }
+}
+
+// ---- input transform, NHWC source, LDS-transposed ---------------------------------------
+// Reads run along C (contiguous in NHWC), stores along p, so the block
+// transposes through LDS.  A workgroup takes one (n, ty), TC consecutive tx and
+// NQ channel vectors: phase 1 copies the 4 x (2*TC+2) pixel halo, 16 bytes per
+// (pixel, cq) with cq fastest across lanes; phase 2 gives thread (tile, cq) its
+// 16 pixels as 16-byte LDS reads (even/odd columns kept apart so lanes walking
+// tx read consecutive vectors) and stores 16 coalesced vectors of V.
+template <typename T, int TC, int NQ>
+__global__ __launch_bounds__(TC * NQ) void input_transform_nhwc_kernel(const T* __restrict__ x, T* __restrict__ V,
+                                                                       int N, int C, int H, int W, int pad, int th,
+                                                                       int tw, long Pp, int Cp, int colBlocks) {
+    constexpr int CV = ChanVec<T>::n;
+    constexpr int HALF = TC + 1;                       // columns of one parity
+    __shared__ Pack16<T> sm[NQ][4][2][HALF];           // [cq][row][col parity][col/2]
+    const int cq0 = blockIdx.y * NQ;
+    const int cb = blockIdx.x % colBlocks, rowid = blockIdx.x / colBlocks;
+    const int ty = rowid % th, n = rowid / th;
+    const int tx0 = cb * TC;
+    const int h0 = 2 * ty - pad, w0 = 2 * tx0 - pad;
+    const int tid = threadIdx.x;
+    const int CQ = Cp / CV;
+
+    constexpr int COLS = 2 * TC + 2;
+    for (int e = tid; e < 4 * COLS * NQ; e += TC * NQ) {
+        const int q = e % NQ, col = (e / NQ) % COLS, r = e / (NQ * COLS);
+        const int ih = h0 + r, iw = w0 + col, cq = cq0 + q;
+        Pack16<T> v;
+#pragma unroll
+        for (int i = 0; i < CV; ++i) v.e[i] = from_f32<T>(0.f);
+        if (ih >= 0 && ih < H && iw >= 0 && iw < W && cq < CQ) {
+            const T* src = x + (((size_t)n * H + ih) * W + iw) * C + cq * CV;
+            if ((cq + 1) * CV <= C && (C % CV) == 0) {
+                v = *reinterpret_cast<const Pack16<T>*>(src);
+            } else {
+#pragma unroll
+                for (int i = 0; i < CV; ++i)
+                    if (cq * CV + i < C) v.e[i] = src[i];
+            }
+        }
+        sm[q][r][col & 1][col >> 1] = v;
+    }
+    __syncthreads();
+
+    const int tc = tid % TC, q = tid / TC;
+    const int tx = tx0 + tc, cq = cq0 + q;
+    if (tx >= tw || cq >= CQ) return;
+    float v[CV][16];
+    {
+        float d[CV][4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const Pack16<T> pk = sm[q][i][j & 1][tc + (j >> 1)];
+#pragma unroll
+                for (int e = 0; e < CV; ++e) d[e][i][j] = to_f32(pk.e[e]);
+            }
+#pragma unroll
+        for (int e = 0; e < CV; ++e) input_tile_transform(d[e], v[e]);
+    }
+    const long p = ((long)n * th + ty) * tw + tx;
+    const size_t plane = (size_t)Cp * Pp;
+    T* vp = V + ((size_t)cq * Pp + p) * CV;
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) {
+        float o[CV];
+#pragma unroll
+        for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
+        store_chan_vec<T>(vp + xi * plane, o);
+    }
+}
+
 // ---- output transform, layout-generic ---------------------------------------------
 // One thread per (tile p, filter k), p fastest: the 16 loads of a wave are
 // contiguous runs of Mo[xi][k][.].  Stores go through the destination strides.
@@ -168,6 +323,55 @@ __global__ __launch_bounds__(256) void output_transform_generic_kernel(const flo
     if (p >= P || k >= K) return;
     const size_t plane = (size_t)Kp * Pp;
     const float* mp = Mo + (size_t)k * Pp + p;
+    float m[16];
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];
+    float o[2][2];
+    output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    T* yp = y + n * s.n + k * s.c;
+    if (relu) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) o[a][b] = fmaxf(o[a][b], 0.f);
+    }
+    if (s.w == 1 && (Wo & 1) == 0 && (s.h & 1) == 0 && (s.c & 1) == 0 && (s.n & 1) == 0) {
+        // W-contiguous destination with even rows: the two outputs of a tile row go out as one store
+        struct alignas(2 * sizeof(T)) Pair { T a, b; };
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            const int oh = 2 * ty + a;
+            if (oh < Ho) {
+                Pair pr{from_f32<T>(o[a][0]), from_f32<T>(o[a][1])};
+                *reinterpret_cast<Pair*>(yp + oh * s.h + 2 * tx) = pr;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int oh = 2 * ty + a, ow = 2 * tx + b;
+            if (oh < Ho && ow < Wo) yp[oh * s.h + ow * s.w] = from_f32<T>(o[a][b]);
+        }
+}
+
+// ---- output transform from the K-contiguous product Mo[xi][Pp][Kp] ------------------------
+// One thread per (filter k, tile p), k fastest: loads are contiguous along K and
+// so are the stores of a K-contiguous destination (NHWC).
+template <typename T>
+__global__ __launch_bounds__(256) void output_transform_pk_kernel(const float* __restrict__ Mo, T* __restrict__ y,
+                                                                   ActStrides s, int N, int K, int Ho, int Wo, int th,
+                                                                   int tw, long P, long Pp, int Kp, int order,
+                                                                   int relu) {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    const long p = (long)blockIdx.y * blockDim.y + threadIdx.y;
+    if (k >= K || p >= P) return;
+    const size_t plane = (size_t)Kp * Pp;
+    const float* mp = Mo + (size_t)p * Kp + k;
     float m[16];
 #pragma unroll
     for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];

@@ -3,6 +3,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <vector>
 
@@ -38,6 +39,7 @@ int fail(int code, const char* fmt, ...) {
 
 bool valid_layout(int l) { return l == WINO_NCHW || l == WINO_NHWC || l == WINO_CHWN; }
 bool valid_dtype(int d) { return d == WINO_F32 || d == WINO_F16 || d == WINO_BF16; }
+bool valid_porder(int o) { return o == WINO_PRODUCT_KP || o == WINO_PRODUCT_PK; }
 bool valid_order(int o) { return o == WINO_TILES_BATCH_MAJOR || o == WINO_TILES_BATCH_MINOR; }
 
 // ---- scratch arena: one grow-only allocation per device ------------------------
@@ -132,7 +134,37 @@ int launch_filter_transform(int layout, int K, int C, int Kp, int Cp, const void
 
 template <typename T>
 int launch_input_transform(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st) {
-    dim3 grid((unsigned)((g.P + 255) / 256), g.Cp / ChanVec<T>::n), block(256);
+    constexpr int CV = ChanVec<T>::n;
+    const int CQ = g.Cp / CV;
+    if (layout == WINO_NCHW && order == WINO_TILES_BATCH_MAJOR && g.th * g.tw >= 64) {
+        // TR x TC tiles per workgroup, TR*TC <= 256, halo of CV channels in LDS (<= 44 KB).
+        // TR is kept a multiple of 8 when it can be, so a workgroup's run of V (TR*tw
+        // 16-byte vectors per coordinate) starts and ends on a 128-byte boundary.
+        const int TC = g.tw < 128 ? g.tw : 128;
+        int TR = 256 / TC;
+        if (TR > 8) TR = 8;
+        if (TR > g.th) TR = g.th;
+        const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
+        const int ldsW = 2 * TC + 2;
+        int chunkLog2 = 0;
+        while ((64 << chunkLog2) < ldsW) ++chunkLog2;
+        const size_t lds = (size_t)CV * (2 * TR + 2) * ldsW * sizeof(float);
+        dim3 grid(rowBlocks * colBlocks, CQ, g.N), block(256);
+        hipLaunchKernelGGL(input_transform_nchw_kernel<T>, grid, block, lds, st, (const T*)x, (T*)V, g.N, g.C, g.H,
+                           g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, TR, TC, colBlocks, chunkLog2);
+        LAUNCH_CHECK("input_transform_nchw");
+        return WINO_OK;
+    }
+    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR) {
+        constexpr int TC = 32, NQ = 8;
+        const int colBlocks = (g.tw + TC - 1) / TC;
+        dim3 grid((unsigned)((long)g.N * g.th * colBlocks), (CQ + NQ - 1) / NQ), block(TC * NQ);
+        hipLaunchKernelGGL((input_transform_nhwc_kernel<T, TC, NQ>), grid, block, 0, st, (const T*)x, (T*)V, g.N, g.C,
+                           g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks);
+        LAUNCH_CHECK("input_transform_nhwc");
+        return WINO_OK;
+    }
+    dim3 grid((unsigned)((g.P + 255) / 256), CQ), block(256);
     hipLaunchKernelGGL(input_transform_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
                        act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
                        g.Cp, order);
@@ -141,31 +173,51 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
 }
 
 template <typename T>
-int launch_output_transform(int layout, int order, unsigned flags, int N, int K, int Ho, int Wo, int Kp, long P,
-                            long Pp, const float* Mo, void* y, hipStream_t st) {
+int launch_output_transform(int layout, int order, int porder, unsigned flags, int N, int K, int Ho, int Wo, int Kp,
+                            long P, long Pp, const float* Mo, void* y, hipStream_t st) {
     const int th = (Ho + 1) / 2, tw = (Wo + 1) / 2;
-    dim3 grid((unsigned)((P + 255) / 256), K), block(256);
-    hipLaunchKernelGGL(output_transform_generic_kernel<T>, grid, block, 0, st, Mo, (T*)y,
-                       act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order,
-                       (flags & WINO_FLAG_RELU) ? 1 : 0);
+    const int relu = (flags & WINO_FLAG_RELU) ? 1 : 0;
+    if (porder == WINO_PRODUCT_PK) {
+        int bx = 64;
+        while (bx < K && bx < 256) bx *= 2;
+        dim3 block(bx, 256 / bx), grid((K + bx - 1) / bx, (unsigned)((P + block.y - 1) / block.y));
+        hipLaunchKernelGGL(output_transform_pk_kernel<T>, grid, block, 0, st, Mo, (T*)y,
+                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+    } else {
+        dim3 grid((unsigned)((P + 255) / 256), K), block(256);
+        hipLaunchKernelGGL(output_transform_generic_kernel<T>, grid, block, 0, st, Mo, (T*)y,
+                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+    }
     LAUNCH_CHECK("output_transform");
     return WINO_OK;
 }
 
-template <typename T, int NV>
+template <typename T, int NV, bool PK>
 int launch_gemm_t(int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
     dim3 grid((unsigned)(Pp / GEMM_BN), Kp / GEMM_BM, 16), block(256);
-    hipLaunchKernelGGL((gemm_128x128_kernel<T, NV>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp, Kp, Pp);
+    hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp, Kp,
+                       Pp);
     LAUNCH_CHECK("batched_gemm");
     return WINO_OK;
 }
 
-int launch_gemm(int dtype, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
+int launch_gemm(int dtype, int porder, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo,
+                hipStream_t st) {
     // slab per barrier: 4 channel vectors = 16 channels (fp32) or 32 (16-bit); Cp is a multiple of that
+    const bool pk = porder == WINO_PRODUCT_PK;
     switch (dtype) {
-    case WINO_F32: return launch_gemm_t<float, 4>(Cp, Kp, Pp, U, V, Mo, st);
-    case WINO_F16: return launch_gemm_t<f16_t, 4>(Cp, Kp, Pp, U, V, Mo, st);
-    case WINO_BF16: return launch_gemm_t<bf16_t, 4>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_F32:
+        if (Cp % 32 == 0 && getenv("WINO_NV8"))
+            return pk ? launch_gemm_t<float, 8, true>(Cp, Kp, Pp, U, V, Mo, st)
+                      : launch_gemm_t<float, 8, false>(Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<float, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
+                  : launch_gemm_t<float, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_F16:
+        return pk ? launch_gemm_t<f16_t, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
+                  : launch_gemm_t<f16_t, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
+    case WINO_BF16:
+        return pk ? launch_gemm_t<bf16_t, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
+                  : launch_gemm_t<bf16_t, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -255,13 +307,14 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         StageScope t(WINO_STAGE_GEMM, st);
         return launch_gemm_out(dst, dtype, order, flags, g, U, V, y, st);
     }
+    const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
     {
         StageScope t(WINO_STAGE_GEMM, st);
-        rc = launch_gemm(dtype, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
+        rc = launch_gemm(dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
         if (rc) return rc;
     }
     StageScope t(WINO_STAGE_OUTPUT, st);
-    return wino_output_transform(dst, dtype, order, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
+    return wino_output_transform(dst, dtype, order, porder, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
 }
 
 __global__ void warmup_kernel() {}
@@ -337,17 +390,20 @@ int wino_input_transform(int layout, int dtype, int tile_order, int N, int C, in
     DISPATCH_DTYPE(dtype, launch_input_transform<T>(layout, tile_order, g, x, V, (hipStream_t)stream));
 }
 
-int wino_batched_gemm(int dtype, int C, int K, long P, const void* U, const void* V, float* Mo, void* stream) {
+int wino_batched_gemm(int dtype, int product_order, int C, int K, long P, const void* U, const void* V, float* Mo,
+                      void* stream) {
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
     if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
-    return launch_gemm(dtype, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
+    return launch_gemm(dtype, product_order, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
                        (hipStream_t)stream);
 }
 
-int wino_output_transform(int layout, int dtype, int tile_order, unsigned flags, int N, int K, int Ho, int Wo,
-                          const float* Mo, void* y, void* stream) {
+int wino_output_transform(int layout, int dtype, int tile_order, int product_order, unsigned flags, int N, int K,
+                          int Ho, int Wo, const float* Mo, void* y, void* stream) {
     if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!Mo || !y) return fail(WINO_ERR_INVALID, "null pointer");
     if (N <= 0 || K <= 0 || Ho <= 0 || Wo <= 0)
@@ -355,7 +411,7 @@ int wino_output_transform(int layout, int dtype, int tile_order, unsigned flags,
     const long P = (long)N * ((Ho + 1) / 2) * ((Wo + 1) / 2);
     const int Kp = (int)round_up(K, kKPad);
     const long Pp = round_up(P, kPPad);
-    DISPATCH_DTYPE(dtype, launch_output_transform<T>(layout, tile_order, flags, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
+    DISPATCH_DTYPE(dtype, launch_output_transform<T>(layout, tile_order, product_order, flags, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
                                                      (hipStream_t)stream));
 }
 

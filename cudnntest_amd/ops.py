@@ -25,6 +25,7 @@ NCHW, NHWC, CHWN = 0, 1, 2
 F32, F16, BF16 = 0, 1, 2
 ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED = 0, 1, 2, 3
 TILES_BATCH_MAJOR, TILES_BATCH_MINOR = 0, 1
+PRODUCT_KP, PRODUCT_PK = 0, 1
 FLAG_RELU = 1
 
 
@@ -159,17 +160,21 @@ def input_transform(x, pad=1, layout=NCHW, tile_order=TILES_BATCH_MAJOR):
     return V
 
 
-def batched_gemm(U, V, C, K, P):
-    """Mo[16][Kp][Pp] (fp32) = sum_c U[xi][c][k] V[xi][c][p]; U, V in channel-vector layout."""
-    Mo = torch.empty((16, U.shape[2], V.shape[2]), dtype=torch.float32, device=U.device)
-    _lib.check(_lib.load().wino_batched_gemm(_dt(U), C, K, P, _ptr(U), _ptr(V), _ptr(Mo), _stream()),
+def batched_gemm(U, V, C, K, P, product_order=PRODUCT_KP):
+    """Mo (fp32) = sum_c U[xi][c][k] V[xi][c][p]; U, V in channel-vector layout.
+    Shape [16][Kp][Pp], or [16][Pp][Kp] with PRODUCT_PK."""
+    shape = (16, U.shape[2], V.shape[2]) if product_order == PRODUCT_KP else (16, V.shape[2], U.shape[2])
+    Mo = torch.empty(shape, dtype=torch.float32, device=U.device)
+    _lib.check(_lib.load().wino_batched_gemm(_dt(U), product_order, C, K, P, _ptr(U), _ptr(V), _ptr(Mo), _stream()),
                "wino_batched_gemm")
     return Mo
 
 
-def output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False, dtype=torch.float32):
+def output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False, dtype=torch.float32,
+                     product_order=PRODUCT_KP):
     y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=dtype, device=Mo.device)
-    _lib.check(_lib.load().wino_output_transform(int(layout), _DTYPES[dtype], tile_order, FLAG_RELU if relu else 0,
+    _lib.check(_lib.load().wino_output_transform(int(layout), _DTYPES[dtype], tile_order, product_order,
+                                                 FLAG_RELU if relu else 0,
                                                  N, K, Ho, Wo, _ptr(Mo), _ptr(y), _stream()),
                "wino_output_transform")
     return y

@@ -45,6 +45,12 @@ typedef enum {
     WINO_TILES_BATCH_MINOR = 1  /* p = (ty*tw + tx)*N + n  */
 } wino_tile_order_t;
 
+/* orientation of the GEMM product in HBM (staged algorithm only) */
+typedef enum {
+    WINO_PRODUCT_KP = 0, /* Mo[16][Kp][Pp]: tiles contiguous -- for NCHW / CHWN destinations */
+    WINO_PRODUCT_PK = 1  /* Mo[16][Pp][Kp]: filters contiguous -- for NHWC destinations      */
+} wino_product_order_t;
+
 typedef enum {
     WINO_OK = 0,
     WINO_ERR_INVALID = -1,     /* null pointer, non-positive size, unknown enum */
@@ -82,7 +88,7 @@ int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, in
  * (4 channels per 16-byte vector for fp32, 8 for f16/bf16):
  *   U   [16][Cp/CV][Kp][CV]   transformed filters, channel vectors innermost
  *   V   [16][Cp/CV][Pp][CV]   transformed input tiles
- *   Mo  [16][Kp][Pp]          GEMM product, always fp32
+ *   Mo  [16][Kp][Pp]          GEMM product, always fp32 ([16][Pp][Kp] with WINO_PRODUCT_PK)
  * Cp is C rounded up to 4 channel vectors (16 for fp32, 32 for f16/bf16); Kp and Pp are K
  * and P rounded up to 128.  The counterpart of
  * MSize/NSize/KSize at comparison/wrapedConv_NCHW.cuh:346-362. */
@@ -110,13 +116,13 @@ int wino_input_transform(int layout, int dtype, int tile_order, int N, int C, in
 
 /* Mo[xi][k][p] = sum_c U[xi][c][k] V[xi][c][p], xi = 0..15, fp32 accumulate on MFMA.
  * Replaces GEMM_batch_256_128x128_{KMKN,MKNK} (comparison/GEMM.cuh:124,4). */
-int wino_batched_gemm(int dtype, int C, int K, long P, const void *U, const void *V, float *Mo,
-                      void *stream);
+int wino_batched_gemm(int dtype, int product_order, int C, int K, long P, const void *U, const void *V,
+                      float *Mo, void *stream);
 
 /* y = A^T Mo A.  Replaces wino_invers_{nchw,nhwc,chwn}_suitFor128*
  * (wrapedConv_NCHW.cuh:905,1034, wrapedConv_NHWC.cuh:376, wrapedConv_CHWN.cuh:379). */
-int wino_output_transform(int layout, int dtype, int tile_order, unsigned flags, int N, int K, int Ho,
-                          int Wo, const float *Mo, void *y, void *stream);
+int wino_output_transform(int layout, int dtype, int tile_order, int product_order, unsigned flags, int N,
+                          int K, int Ho, int Wo, const float *Mo, void *y, void *stream);
 
 /* GEMM with the output transform in its epilogue: y directly from U and V. */
 int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int N, int C, int K,

@@ -71,8 +71,9 @@ def test_invalid_arguments_are_rejected_without_a_gpu():
     assert b"bad shape" in L.wino_last_error()
     assert L.wino_filter_transform(0, 0, 0, 4, one, one, None) == -1
     assert L.wino_input_transform(0, 0, 5, 1, 1, 4, 4, 1, one, one, None) == -1
-    assert L.wino_batched_gemm(0, 0, 1, 1, one, one, one, None) == -1
-    assert L.wino_output_transform(3, 0, 0, 0, 1, 1, 4, 4, one, one, None) == -1
+    assert L.wino_batched_gemm(0, 0, 0, 1, 1, one, one, one, None) == -1
+    assert L.wino_batched_gemm(0, 5, 1, 1, 1, one, one, one, None) == -1
+    assert L.wino_output_transform(3, 0, 0, 0, 0, 1, 1, 4, 4, one, one, None) == -1
     assert L.wino_layout_transform(0, 1, 0, 1, 1, 0, 4, one, one, None) == -1
     assert L.wino_workspace_bytes(0, 0, 1, 1, 4, 4, 1) == 0
 

@@ -53,8 +53,9 @@ def test_input_transform(oracle, layout, order, shape, pad):
     assert not V[:, C:, :P].any(), "channel padding must be zero"
 
 
+@pytest.mark.parametrize("porder", [ops.PRODUCT_KP, ops.PRODUCT_PK])
 @pytest.mark.parametrize("C,K,P", [(16, 128, 128), (3, 5, 30), (64, 64, 784), (40, 130, 300), (256, 256, 512)])
-def test_batched_gemm(oracle, C, K, P):
+def test_batched_gemm(oracle, C, K, P, porder):
     g = ops.geometry(ops.F32, 1, C, K, 4, 4, 1)
     Cp, Kp = g["Cp"], g["Kp"]
     Pp = (P + 127) // 128 * 128
@@ -62,7 +63,9 @@ def test_batched_gemm(oracle, C, K, P):
     V = np.zeros((16, Cp, Pp), np.float32)
     U[:, :C, :K] = synth.small_ints(16 * C * K, 3, -3, 3).reshape(16, C, K)
     V[:, :C, :P] = synth.small_ints(16 * C * P, 4, -5, 5).reshape(16, C, P)
-    Mo = host(ops.batched_gemm(pack_operand(U), pack_operand(V), C, K, P))
+    Mo = host(ops.batched_gemm(pack_operand(U), pack_operand(V), C, K, P, porder))
+    if porder == ops.PRODUCT_PK:
+        Mo = Mo.transpose(0, 2, 1)
     want = oracle.wino_gemm(np.ascontiguousarray(U[:, :C, :K]), np.ascontiguousarray(V[:, :C, :P]))
     assert np.array_equal(Mo[:, :K, :P], want)
 
@@ -79,7 +82,8 @@ def test_batched_gemm_floats(oracle):
 @pytest.mark.parametrize("order", [ops.TILES_BATCH_MAJOR, ops.TILES_BATCH_MINOR])
 @pytest.mark.parametrize("N,K,Ho,Wo", [(2, 4, 5, 5), (3, 7, 9, 6), (1, 130, 14, 14), (4, 16, 28, 28), (2, 3, 1, 1)])
 @pytest.mark.parametrize("relu", [False, True])
-def test_output_transform(oracle, layout, order, N, K, Ho, Wo, relu):
+@pytest.mark.parametrize("porder", [ops.PRODUCT_KP, ops.PRODUCT_PK])
+def test_output_transform(oracle, layout, order, N, K, Ho, Wo, relu, porder):
     th, tw = (Ho + 1) // 2, (Wo + 1) // 2
     P = N * th * tw
     g = ops.geometry(ops.F32, 1, 1, K, 4, 4, 1)
@@ -90,7 +94,8 @@ def test_output_transform(oracle, layout, order, N, K, Ho, Wo, relu):
         Mo[:, :K, :P] = M[:, :, batch_minor_perm(N, th, tw)]
     else:
         Mo[:, :K, :P] = M
-    y = host(ops.output_transform(dev(Mo), N, K, Ho, Wo, layout, order, relu))
+    Md = dev(np.ascontiguousarray(Mo.transpose(0, 2, 1))) if porder == ops.PRODUCT_PK else dev(Mo)
+    y = host(ops.output_transform(Md, N, K, Ho, Wo, layout, order, relu, product_order=porder))
     want = oracle.wino_output_transform(M, N, Ho, Wo, layout)
     if relu:
         want = np.maximum(want, 0)
