@@ -192,6 +192,47 @@ __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const A
     }
 }
 
+// A^T (.) A on a wave's sixteen 32x32 accumulators, then the stores.  Register r of
+// an accumulator is MFMA row 8*(r/4) + 4*lh + r%4, the lane's l32 is the MFMA column.
+template <typename T, bool SWAP>
+__device__ __forceinline__ void winograd_epilogue(const floatx16 (&acc)[16], T* __restrict__ y, const ActStrides& ys,
+                                                  int N, int K, int Ho, int Wo, int th, int tw, long P, int order,
+                                                  int relu, int k0, long p0, int wm, int wn, int l32, int lh) {
+    if (!SWAP) {
+        const long p = p0 + wn * 32 + l32;
+        if (p >= P) return;
+        int n, ty, tx;
+        decode_tile(p, order, N, th, tw, n, ty, tx);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (k >= K) continue;
+            float m[16];
+#pragma unroll
+            for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
+            float y00, y01, y10, y11;
+            output_tile_transform(m, y00, y01, y10, y11);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
+        }
+    } else {
+        const int k = k0 + wn * 32 + l32;
+        if (k >= K) return;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const long p = p0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (p >= P) continue;
+            int n, ty, tx;
+            decode_tile(p, order, N, th, tw, n, ty, tx);
+            float m[16];
+#pragma unroll
+            for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
+            float y00, y01, y10, y11;
+            output_tile_transform(m, y00, y01, y10, y11);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
+        }
+    }
+}
+
 template <typename T, bool SWAP>
 __global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, const T* __restrict__ V,
                                                        T* __restrict__ y, ActStrides ys, int N, int K, int Ho, int Wo,
@@ -281,40 +322,7 @@ __global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, 
         iteration(par1_t{}, g + 1);
     }
 
-    // ---- epilogue: A^T (.) A on the 16 accumulators, then store ----------------------
-    if (!SWAP) {
-        const long p = p0 + wn * 32 + l32;
-        if (p >= P) return;
-        int n, ty, tx;
-        decode_tile(p, order, N, th, tw, n, ty, tx);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (k >= K) continue;
-            float m[16];
-#pragma unroll
-            for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
-            float y00, y01, y10, y11;
-            output_tile_transform(m, y00, y01, y10, y11);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
-        }
-    } else {
-        const int k = k0 + wn * 32 + l32;
-        if (k >= K) return;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const long p = p0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (p >= P) continue;
-            int n, ty, tx;
-            decode_tile(p, order, N, th, tw, n, ty, tx);
-            float m[16];
-#pragma unroll
-            for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
-            float y00, y01, y10, y11;
-            output_tile_transform(m, y00, y01, y10, y11);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
-        }
-    }
+    winograd_epilogue<T, SWAP>(acc, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
 }
 
 }  // namespace wino

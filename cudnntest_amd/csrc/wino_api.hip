@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "fused.hpp"
 #include "gemm.hpp"
 #include "transforms.hpp"
 
@@ -254,6 +255,43 @@ int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometr
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
+template <typename T, bool SWAP, bool LOC>
+int launch_fused_t(int src, int dst, int order, unsigned flags, const Geometry& g, const void* x, const void* U,
+                   void* y, hipStream_t st) {
+    const int kTiles = (g.K + GO_T - 1) / GO_T;
+    const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
+    const int pGroups = (pTiles + 7) / 8;
+    dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
+    hipLaunchKernelGGL((fused_conv_kernel<T, SWAP, LOC>), grid, block, 0, st, (const T*)x, (const T*)U, (T*)y,
+                       act_strides(src, g.N, g.C, g.H, g.W), act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.C, g.K,
+                       g.H, g.W, g.pad, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, order,
+                       (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
+    LAUNCH_CHECK("fused_conv");
+    return WINO_OK;
+}
+
+template <typename T>
+int launch_fused_d(int src, int dst, int order, unsigned flags, const Geometry& g, const void* x, const void* U,
+                   void* y, hipStream_t st) {
+    if ((long)g.N * g.C * g.H * g.W >= (1L << 31))
+        return fail(WINO_ERR_UNSUPPORTED, "fused kernel: input tensor too large for 32-bit element offsets");
+    const bool swap = dst == WINO_NHWC, loc = src == WINO_NHWC;
+    if (swap && loc) return launch_fused_t<T, true, true>(src, dst, order, flags, g, x, U, y, st);
+    if (swap) return launch_fused_t<T, true, false>(src, dst, order, flags, g, x, U, y, st);
+    if (loc) return launch_fused_t<T, false, true>(src, dst, order, flags, g, x, U, y, st);
+    return launch_fused_t<T, false, false>(src, dst, order, flags, g, x, U, y, st);
+}
+
+int launch_fused(int src, int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* x,
+                 const void* U, void* y, hipStream_t st) {
+    switch (dtype) {
+    case WINO_F32: return launch_fused_d<float>(src, dst, order, flags, g, x, U, y, st);
+    case WINO_F16: return launch_fused_d<f16_t>(src, dst, order, flags, g, x, U, y, st);
+    case WINO_BF16: return launch_fused_d<bf16_t>(src, dst, order, flags, g, x, U, y, st);
+    }
+    return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
 #define DISPATCH_DTYPE(dtype, CALL)                          \
     switch (dtype) {                                         \
     case WINO_F32: { typedef float T; return CALL; }         \
@@ -278,7 +316,6 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     if (algo == WINO_ALGO_AUTO) algo = WINO_ALGO_STAGED;
-    if (algo == WINO_ALGO_FUSED) return fail(WINO_ERR_UNSUPPORTED, "algo %d not built yet", algo);
 
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype);
@@ -297,6 +334,10 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         StageScope t(WINO_STAGE_FILTER, st);
         rc = wino_filter_transform(src, dtype, K, C, w, U, stream);
         if (rc) return rc;
+    }
+    if (algo == WINO_ALGO_FUSED) {
+        StageScope t(WINO_STAGE_GEMM, st);
+        return launch_fused(src, dst, dtype, order, flags, g, x, U, y, st);
     }
     {
         StageScope t(WINO_STAGE_INPUT, st);

@@ -15,7 +15,7 @@ from gpu_util import TOL, dev, host
 
 pytestmark = pytest.mark.gpu
 LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
-ALGOS = [ops.ALGO_STAGED, ops.ALGO_EPILOGUE]
+ALGOS = [ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED]
 
 SMALL = [(2, 3, 4, 5, 5), (1, 8, 8, 6, 6), (3, 5, 7, 9, 9), (2, 16, 130, 7, 10), (1, 1, 1, 3, 3), (5, 40, 24, 14, 14)]
 

@@ -15,7 +15,7 @@ from gpu_util import TOL, batch_minor_perm, dev, host, pack_operand, rounded, un
 pytestmark = pytest.mark.gpu
 LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
 DTYPES = [ops.F16, ops.BF16]
-ALGOS = [ops.ALGO_STAGED, ops.ALGO_EPILOGUE]
+ALGOS = [ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
