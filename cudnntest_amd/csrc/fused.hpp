@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x
 
     // ---- this thread's (tile, channel) units: fixed for the whole kernel ----------------
     int u_tile[UNITS], u_ch[UNITS];            // tile index inside the patch, channel inside the k-group
-    unsigned u_off[UNITS][16];                 // element offset of each of the 16 patch positions (0 if outside)
+    unsigned u_row[UNITS][4], u_col[UNITS][4]; // element offsets of the patch rows (incl. image) and columns, clamped inside
     unsigned u_mask[UNITS];                    // bit i*4+j set when position (i, j) lies inside the image
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
@@ -71,15 +71,22 @@ __global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x
         const bool pvalid = p < P;
         if (pvalid) decode_tile(p, order, N, th, tw, n, ty, tx);
         u_mask[u] = 0;
+        unsigned rmask = 0, cmask = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) {
+            const int ih = 2 * ty - pad + i, iw = 2 * tx - pad + i;
+            if (ih >= 0 && ih < H) rmask |= 1u << i;
+            if (iw >= 0 && iw < W) cmask |= 1u << i;
+            const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);     // clamped: the load stays inside x, the
+            const int iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);     // value is discarded through u_mask
+            u_row[u][i] = (unsigned)(n * xs.n + ihc * xs.h);
+            u_col[u][i] = (unsigned)(iwc * xs.w);
+        }
+        if (pvalid) {
 #pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                const int ih = 2 * ty - pad + i, iw = 2 * tx - pad + jj;
-                const bool ok = pvalid && ih >= 0 && ih < H && iw >= 0 && iw < W;
-                u_off[u][i * 4 + jj] = ok ? (unsigned)(n * xs.n + ih * xs.h + iw * xs.w) : 0u;
-                if (ok) u_mask[u] |= 1u << (i * 4 + jj);
-            }
+            for (int i = 0; i < 4; ++i)
+                if ((rmask >> i) & 1u) u_mask[u] |= cmask << (4 * i);
+        }
     }
 
     floatx16 acc[16];
@@ -91,50 +98,62 @@ __global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x
     typedef std::integral_constant<int, 0> par0_t;
     typedef std::integral_constant<int, 1> par1_t;
 
-    // raw input values of the k-group after the one being multiplied
+    // Raw input patches of the k-group after the one being multiplied.
     T xr[UNITS][16];
-    auto x_load = [&](int g) {
+    auto x_load_unit = [&](int g, int u) {
+        const int c = g * GC + u_ch[u];
+        const unsigned coff = c < C ? (unsigned)(c * xs.c) : 0u;   // channel padding: masked out in v_piece
 #pragma unroll
-        for (int u = 0; u < UNITS; ++u) {
-            const int c = g * GC + u_ch[u];
-            const unsigned coff = c < C ? (unsigned)(c * xs.c) : 0u;   // channel padding: masked out below
+        for (int i = 0; i < 4; ++i) {
+            const unsigned ro = u_row[u][i] + coff;
 #pragma unroll
-            for (int q = 0; q < 16; ++q) xr[u][q] = x[u_off[u][q] + coff];
+            for (int jj = 0; jj < 4; ++jj) xr[u][i * 4 + jj] = x[ro + u_col[u][jj]];
         }
     };
-    // transform the staged patches and scatter their 16 coordinates into stage S of V
-    auto v_build = [&](auto par, int g) {
+    // Building stage S of V from the staged patches, cut into 16 pieces so that one
+    // piece can ride in the shadow of each coordinate's MFMAs:
+    //   pieces 0 .. 2*UNITS-1 : per unit, mask the patch (zero padding) then B^T d B
+    //   the remaining pieces  : the LDS writes, a few coordinates each; the first UNITS
+    //                           of them also refill the patches with k-group `gload`
+    float vt[UNITS][16];
+    float dpatch[4][4];
+    auto v_piece = [&](auto par, int g, int gload, int piece) {
         constexpr int S = decltype(par)::value;
-        float v[UNITS][16];
+        constexpr int NW = 16 - 2 * UNITS;                 // pieces that write
+        constexpr int PER = (16 + NW - 1) / NW;            // coordinates per writing piece
+        if (piece < 2 * UNITS) {
+            const int u = piece >> 1;
+            if ((piece & 1) == 0) {
+                const bool cok = g * GC + u_ch[u] < C;
+                const unsigned m = cok ? u_mask[u] : 0u;
 #pragma unroll
-        for (int u = 0; u < UNITS; ++u) {
-            const bool cok = g * GC + u_ch[u] < C;
-            const unsigned m = cok ? u_mask[u] : 0u;
-            float d[4][4];
-#pragma unroll
-            for (int q = 0; q < 16; ++q) d[q >> 2][q & 3] = ((m >> q) & 1u) ? to_f32(xr[u][q]) : 0.f;
-            input_tile_transform(d, v[u]);
-        }
-        if (LANES_ON_CHANNELS) {
-#pragma unroll
-            for (int u = 0; u < UNITS; ++u) {
-                const int h = u_ch[u] / CV, e = u_ch[u] % CV;
-#pragma unroll
-                for (int xi = 0; xi < 16; ++xi) {
-                    T* dst = reinterpret_cast<T*>(S ? &Vs1[xi][h][u_tile[u]] : &Vs0[xi][h][u_tile[u]]);
-                    dst[e] = from_f32<T>(v[u][xi]);
-                }
+                for (int q = 0; q < 16; ++q) dpatch[q >> 2][q & 3] = ((m >> q) & 1u) ? to_f32(xr[u][q]) : 0.f;
+            } else {
+                input_tile_transform(dpatch, vt[u]);
             }
-        } else {
-            // the thread's UNITS channels are consecutive elements of one channel vector: one 8-byte write
-            struct alignas(8) Chunk { T e[UNITS]; };
-            static_assert(sizeof(Chunk) == 8, "chunk must be 8 bytes");
-            const int h = u_ch[0] / CV, e0 = u_ch[0] % CV;
+            return;
+        }
+        const int w = piece - 2 * UNITS;
+        if (w < UNITS && gload >= 0) x_load_unit(gload, w);
 #pragma unroll
-            for (int xi = 0; xi < 16; ++xi) {
+        for (int t = 0; t < PER; ++t) {
+            const int xi = w * PER + t;
+            if (xi >= 16) continue;
+            if (LANES_ON_CHANNELS) {
+#pragma unroll
+                for (int u = 0; u < UNITS; ++u) {
+                    const int h = u_ch[u] / CV, e = u_ch[u] % CV;
+                    T* dst = reinterpret_cast<T*>(S ? &Vs1[xi][h][u_tile[u]] : &Vs0[xi][h][u_tile[u]]);
+                    dst[e] = from_f32<T>(vt[u][xi]);
+                }
+            } else {
+                // the thread's UNITS channels are consecutive elements of one channel vector: one 8-byte write
+                struct alignas(8) Chunk { T e[UNITS]; };
+                static_assert(sizeof(Chunk) == 8, "chunk must be 8 bytes");
+                const int h = u_ch[0] / CV, e0 = u_ch[0] % CV;
                 Chunk ck;
 #pragma unroll
-                for (int u = 0; u < UNITS; ++u) ck.e[u] = from_f32<T>(v[u][xi]);
+                for (int u = 0; u < UNITS; ++u) ck.e[u] = from_f32<T>(vt[u][xi]);
                 T* dst = reinterpret_cast<T*>(S ? &Vs1[xi][h][u_tile[0]] : &Vs0[xi][h][u_tile[0]]);
                 *reinterpret_cast<Chunk*>(dst + e0) = ck;
             }
@@ -163,17 +182,19 @@ __global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x
         };
         const int g1 = g + 1 < ngrp ? g + 1 : g;      // surplus work on the last group is never read
         const int g2 = g + 2 < ngrp ? g + 2 : g1;
+        // filter rows of group g+1 first (the whole iteration to land); the raw patches of
+        // group g+2 are requested as soon as those of g+1 have been consumed
         u_load(other_t{}, g1);
-        v_build(other_t{}, g1);                      // consumes xr (loaded one iteration ago)
-        __builtin_amdgcn_sched_barrier(0);           // keep the x loads younger than the filter rows
-        x_load(g2);                                  // refills xr for the iteration after next
         frag_load(0);
         frag_load(1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int xi = 0; xi < 16; ++xi) {
             if (xi + 2 < 16) frag_load(xi + 2);
+            v_piece(other_t{}, g1, g2, xi);
             if (SWAP) Mma<T>::run(fv[xi % 3], fu[xi % 3], acc[xi]);
             else Mma<T>::run(fu[xi % 3], fv[xi % 3], acc[xi]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         // the filter rows of the next stage must be in LDS (they were issued before the x
         // loads, and loads retire in order); the younger x loads may stay in flight
@@ -181,12 +202,13 @@ __global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x
         __syncthreads();
     };
 
-    // prologue: stage 0 of both slabs, and the raw patches of group 1
-    x_load(0);
+    // prologue: stage 0 of both slabs, and the raw patches of group 1 in flight
     u_load(par0_t{}, 0);
-    v_build(par0_t{}, 0);
     __builtin_amdgcn_sched_barrier(0);
-    x_load(ngrp > 1 ? 1 : 0);
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) x_load_unit(0, u);
+#pragma unroll
+    for (int piece = 0; piece < 16; ++piece) v_piece(par0_t{}, 0, ngrp > 1 ? 1 : 0, piece);
     __builtin_amdgcn_s_waitcnt(WAIT_IMM);
     __syncthreads();
 

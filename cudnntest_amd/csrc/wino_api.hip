@@ -306,6 +306,20 @@ int tile_order_for(int src, int /*dst*/) {
     return src == WINO_CHWN ? WINO_TILES_BATCH_MINOR : WINO_TILES_BATCH_MAJOR;
 }
 
+// Measured on MI355X over the VGG-16 layer shapes: the fewer the channels, the more
+// the transformed tensors cost relative to the multiplies, and the more fusion pays.
+int pick_algo(int dtype, const Geometry& g) {
+    const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
+    if (patches < 512) return WINO_ALGO_STAGED;          // too few 64x64 patches to fill 256 CUs
+    if (dtype == WINO_F32) {
+        if (g.C <= 64) return WINO_ALGO_FUSED;
+        if (g.C <= 128) return WINO_ALGO_EPILOGUE;
+        return WINO_ALGO_STAGED;
+    }
+    if (g.C >= 16 && g.C <= 64 && g.K <= 64) return WINO_ALGO_FUSED;
+    return WINO_ALGO_EPILOGUE;
+}
+
 int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
               const void* x, const void* w, const void* Upre, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
@@ -315,7 +329,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
-    if (algo == WINO_ALGO_AUTO) algo = WINO_ALGO_STAGED;
+    if (algo == WINO_ALGO_AUTO) algo = pick_algo(dtype, g);
 
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype);
