@@ -390,6 +390,14 @@ int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, in
     return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, y, stream);
 }
 
+int wino_pick_algo(int dtype, int N, int C, int K, int H, int W, int pad) {
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    Geometry g;
+    if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
+    return pick_algo(dtype, g);
+}
+
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp, int* Kp,
                   long* Pp) {
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);

@@ -81,6 +81,17 @@ def geometry(dtype, N, C, K, H, W, pad):
     return dict(th=th.value, tw=tw.value, P=P.value, Cp=Cp.value, Kp=Kp.value, Pp=Pp.value)
 
 
+ALGO_NAMES = {ALGO_AUTO: "auto", ALGO_STAGED: "staged", ALGO_EPILOGUE: "epilogue", ALGO_FUSED: "fused"}
+
+
+def pick_algo(dtype, N, C, K, H, W, pad=1):
+    """The algorithm ALGO_AUTO resolves to for this problem."""
+    rc = _lib.load().wino_pick_algo(dtype, N, C, K, H, W, pad)
+    if rc < 0:
+        _lib.check(rc, "wino_pick_algo")
+    return rc
+
+
 def workspace_bytes(dtype, N, C, K, H, W, pad):
     return int(_lib.load().wino_workspace_bytes(dtype, N, C, K, H, W, pad))
 
