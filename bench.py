@@ -44,7 +44,10 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (summaries and the copy-kernel scale factor under profiles/), keyed by
 # (workload, layout, dtype, resolved algo).
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # profiles/staged_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 451.8 MB fetched + 411.0 MB written
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"): 862.8e6,
+}
 
 
 def main():
@@ -57,6 +60,9 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch a plain copy kernel of the first layer's input (known size) three times, so a "
+                         "rocprofv3 --pmc run of this script can scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -97,6 +103,9 @@ def main():
             ops.conv(x, w, 1, layout, algo=algo, relu=multi, out=y)
 
     ops.warmup()
+    if args.copy_probe:
+        for _ in range(3):
+            ops.layout_transform(tensors[0][0], layout, layout)   # same layout both sides: a plain copy
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -64,15 +64,24 @@ constexpr int GEMM_BM = 128, GEMM_BN = 128;
 //             destinations whose contiguous axis is K (NHWC)
 template <typename T, int NV, bool PK>
 __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__ U, const T* __restrict__ V,
-                                                            float* __restrict__ Mo, int Cp, int Kp, long Pp) {
+                                                            float* __restrict__ Mo, int Cp, int Kp, long Pp,
+                                                            int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     __shared__ vec As[2][NV][GEMM_BM];
     __shared__ vec Bs[2][NV][GEMM_BN];
 
-    const int xi = blockIdx.z;
-    const long p0 = (long)blockIdx.x * GEMM_BN;
-    const int k0 = blockIdx.y * GEMM_BM;
+    // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so the
+    // ids that share an XCD walk the filter tiles of one tile column first and the V slab
+    // they share is fetched from HBM once, into that XCD's L2.
+    const int xi = blockIdx.y;
+    const int b = blockIdx.x;
+    const int xcd = b & 7, jj = b >> 3;
+    const int ktile = jj % kTiles;
+    const int ptile = (jj / kTiles) * 8 + xcd;
+    if (ptile >= pTiles) return;
+    const long p0 = (long)ptile * GEMM_BN;
+    const int k0 = ktile * GEMM_BM;
     const int CQ = Cp / CV;
     const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
     const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;

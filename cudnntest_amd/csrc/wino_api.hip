@@ -195,9 +195,10 @@ int launch_output_transform(int layout, int order, int porder, unsigned flags, i
 
 template <typename T, int NV, bool PK>
 int launch_gemm_t(int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
-    dim3 grid((unsigned)(Pp / GEMM_BN), Kp / GEMM_BM, 16), block(256);
+    const int kTiles = Kp / GEMM_BM, pTiles = (int)(Pp / GEMM_BN);
+    dim3 grid((unsigned)((pTiles + 7) / 8 * 8 * kTiles), 16), block(256);
     hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp, Kp,
-                       Pp);
+                       Pp, kTiles, pTiles);
     LAUNCH_CHECK("batched_gemm");
     return WINO_OK;
 }
