@@ -158,15 +158,36 @@ __global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* _
 // A workgroup takes one image n, one channel vector cq and a TR x TC block of
 // tiles.  The (2*TR+2) x (2*TC+2) input halo of each of its CV channels is read
 // once, along W (contiguous), into LDS with the zero padding materialised; each
-// thread then builds its tile from LDS with 8-byte reads (conflict-free: lanes
-// walk tx, two columns apart) and issues 16 coalesced 16-byte stores.
-template <typename T>
+// thread then builds its tile from LDS (lanes walk tx, two columns apart:
+// conflict-free) and issues 16 coalesced 16-byte stores.
+//
+// VEC = elements per lane and load in the halo copy: 1, or 2 for 2-byte types
+// when W is even (4-byte loads of image-aligned column pairs).
+template <typename T> __device__ __forceinline__ void lds_row4(const T* p, float* d);
+template <> __device__ __forceinline__ void lds_row4<float>(const float* p, float* d) {
+    const float2 a = *reinterpret_cast<const float2*>(p);
+    const float2 b = *reinterpret_cast<const float2*>(p + 2);
+    d[0] = a.x; d[1] = a.y; d[2] = b.x; d[3] = b.y;
+}
+template <> __device__ __forceinline__ void lds_row4<f16_t>(const f16_t* p, float* d) {
+    struct alignas(4) P2 { f16_t a, b; };
+    const P2 u = *reinterpret_cast<const P2*>(p), v = *reinterpret_cast<const P2*>(p + 2);
+    d[0] = (float)u.a; d[1] = (float)u.b; d[2] = (float)v.a; d[3] = (float)v.b;
+}
+template <> __device__ __forceinline__ void lds_row4<bf16_t>(const bf16_t* p, float* d) {
+    const uint32_t u = *reinterpret_cast<const uint32_t*>(p), v = *reinterpret_cast<const uint32_t*>(p + 2);
+    d[0] = __uint_as_float(u << 16); d[1] = __uint_as_float(u & 0xffff0000u);
+    d[2] = __uint_as_float(v << 16); d[3] = __uint_as_float(v & 0xffff0000u);
+}
+
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __restrict__ x, T* __restrict__ V, int N,
                                                                    int C, int H, int W, int pad, int th, int tw,
                                                                    long Pp, int Cp, int TR, int TC, int colBlocks,
                                                                    int chunkLog2) {
     constexpr int CV = ChanVec<T>::n;
-    extern __shared__ float in_smem[];   // [CV][rows][ldsW]
+    extern __shared__ __attribute__((aligned(16))) unsigned char in_smem_raw[];
+    T* in_smem = reinterpret_cast<T*>(in_smem_raw);   // [CV][rows][ldsW], the storage type
     const int cq = blockIdx.y, n = blockIdx.z;
     const int rb = blockIdx.x / colBlocks, cb = blockIdx.x % colBlocks;
     const int ty0 = rb * TR, tx0 = cb * TC;
@@ -176,34 +197,51 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     const int tid = threadIdx.x;
 
     const int per_ch = rows * ldsW;
-    // Halo copy.  A unit is 64 consecutive columns of one halo row; wave w takes
+    // Halo copy.  A unit is 64*VEC consecutive columns of one halo row; wave w takes
     // units w, w+4, ...  Loads are issued in batches of CV x MAXU before any of
     // them is written to LDS, so a wave keeps that many HBM requests in flight.
+    // With VEC = 2 a lane loads the image-aligned pair (iw, iw+1), iw even.
     const int lane = tid & 63, wv = tid >> 6;
     constexpr int MAXU = 6;
     const int nunits = rows << chunkLog2;
     const int cmask = (1 << chunkLog2) - 1;
+    const int wbase = VEC == 2 ? (w0 & ~1) : w0;       // first loaded image column (even for VEC = 2)
+    struct alignas(sizeof(T) * VEC) Ld { T e[VEC]; };
     for (int u0 = 0; u0 < nunits; u0 += 4 * MAXU) {
-        float buf[CV][MAXU];
+        Ld buf[CV][MAXU];
 #pragma unroll
         for (int i = 0; i < MAXU; ++i) {
             const int u = u0 + wv + 4 * i;
-            const int r = u >> chunkLog2, q = ((u & cmask) << 6) + lane;
-            const int ih = h0 + r, iw = w0 + q;
-            const bool ok = u < nunits && q < ldsW && ih >= 0 && ih < H && iw >= 0 && iw < W;
+            const int r = u >> chunkLog2;
+            const int iw = wbase + (((u & cmask) << 6) + lane) * VEC;
+            const int ih = h0 + r;
+            // a pair is inside the image or outside it as a whole (W even, iw even)
+            const bool ok = u < nunits && ih >= 0 && ih < H && iw >= 0 && iw < W;
 #pragma unroll
             for (int ch = 0; ch < CV; ++ch) {
                 const int c = cq * CV + ch;
-                buf[ch][i] = (ok && c < C) ? to_f32(x[(((size_t)n * C + c) * H + ih) * W + iw]) : 0.f;
+                if (ok && c < C) {
+                    buf[ch][i] = *reinterpret_cast<const Ld*>(x + (((size_t)n * C + c) * H + ih) * W + iw);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) buf[ch][i].e[e] = from_f32<T>(0.f);
+                }
             }
         }
 #pragma unroll
         for (int i = 0; i < MAXU; ++i) {
             const int u = u0 + wv + 4 * i;
-            const int r = u >> chunkLog2, q = ((u & cmask) << 6) + lane;
-            if (u < nunits && q < ldsW) {
+            const int r = u >> chunkLog2;
+            const int q0 = wbase - w0 + (((u & cmask) << 6) + lane) * VEC;   // LDS column of the first element
+            if (u < nunits) {
 #pragma unroll
-                for (int ch = 0; ch < CV; ++ch) in_smem[ch * per_ch + r * ldsW + q] = buf[ch][i];
+                for (int e = 0; e < VEC; ++e) {
+                    const int q = q0 + e;
+                    if (q >= 0 && q < ldsW) {
+#pragma unroll
+                        for (int ch = 0; ch < CV; ++ch) in_smem[ch * per_ch + r * ldsW + q] = buf[ch][i].e[e];
+                    }
+                }
             }
         }
     }
@@ -216,13 +254,9 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
 #pragma unroll
     for (int ch = 0; ch < CV; ++ch) {
         float d[4][4];
-        const float* base = in_smem + ch * per_ch + (2 * tr) * ldsW + 2 * tc;
+        const T* base = in_smem + ch * per_ch + (2 * tr) * ldsW + 2 * tc;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float2 a = *reinterpret_cast<const float2*>(base + i * ldsW);
-            const float2 b = *reinterpret_cast<const float2*>(base + i * ldsW + 2);
-            d[i][0] = a.x; d[i][1] = a.y; d[i][2] = b.x; d[i][3] = b.y;
-        }
+        for (int i = 0; i < 4; ++i) lds_row4<T>(base + i * ldsW, d[i]);
         input_tile_transform(d, v[ch]);
     }
     const long p = ((long)n * th + ty) * tw + tx;

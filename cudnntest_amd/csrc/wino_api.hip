@@ -147,12 +147,21 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
         if (TR > g.th) TR = g.th;
         const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
         const int ldsW = 2 * TC + 2;
+        // 2-byte types move image-aligned column pairs (4 bytes per lane) when every row starts 4-byte aligned
+        const bool vec2 = sizeof(T) == 2 && (g.W % 2 == 0);
+        const int span = vec2 ? ldsW + 2 : ldsW;          // loaded columns per row (one extra pair on the left)
+        const int perUnit = vec2 ? 128 : 64;
         int chunkLog2 = 0;
-        while ((64 << chunkLog2) < ldsW) ++chunkLog2;
-        const size_t lds = (size_t)CV * (2 * TR + 2) * ldsW * sizeof(float);
+        while ((perUnit << chunkLog2) < span) ++chunkLog2;
+        const size_t lds = (size_t)CV * (2 * TR + 2) * ldsW * sizeof(T);
         dim3 grid(rowBlocks * colBlocks, CQ, g.N), block(256);
-        hipLaunchKernelGGL(input_transform_nchw_kernel<T>, grid, block, lds, st, (const T*)x, (T*)V, g.N, g.C, g.H,
-                           g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, TR, TC, colBlocks, chunkLog2);
+        if (vec2)
+            hipLaunchKernelGGL((input_transform_nchw_kernel<T, (sizeof(T) == 2 ? 2 : 1)>), grid, block, lds, st,
+                               (const T*)x, (T*)V, g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, TR, TC,
+                               colBlocks, chunkLog2);
+        else
+            hipLaunchKernelGGL((input_transform_nchw_kernel<T, 1>), grid, block, lds, st, (const T*)x, (T*)V, g.N,
+                               g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, TR, TC, colBlocks, chunkLog2);
         LAUNCH_CHECK("input_transform_nchw");
         return WINO_OK;
     }
