@@ -53,6 +53,15 @@ template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
     return bf16_t{(uint16_t)(u >> 16)};
 }
 
+// v with its bits ANDed by m (m is all ones or zero).  Opaque to the optimiser on purpose:
+// written as a select, the compiler moves the load that produced v under a branch on the mask and
+// waits for every load separately, instead of issuing a batch of loads and masking afterwards.
+__device__ __forceinline__ float mask_keep(float v, unsigned m) {
+    unsigned r;
+    asm("v_and_b32 %0, %1, %2" : "=v"(r) : "v"(__float_as_uint(v)), "v"(m));
+    return __uint_as_float(r);
+}
+
 __host__ inline size_t dtype_size(int dtype) { return dtype == WINO_F32 ? 4 : 2; }
 
 // ---- channel vectors ------------------------------------------------------------

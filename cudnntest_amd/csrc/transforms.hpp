@@ -122,26 +122,31 @@ __global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* _
     int n, ty, tx;
     decode_tile(p, order, N, th, tw, n, ty, tx);
     const int h0 = 2 * ty - pad, w0 = 2 * tx - pad;
+    // Branch-free halo handling: every load goes to a clamped (always valid) address and
+    // the value is kept or zeroed by a mask, so all CV*16 loads are in flight together.
+    long roff[4], coff[4];
+    unsigned rkeep[4], ckeep[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ih = h0 + i, iw = w0 + i;
+        rkeep[i] = (ih >= 0 && ih < H) ? 0xffffffffu : 0u;
+        ckeep[i] = (iw >= 0 && iw < W) ? 0xffffffffu : 0u;
+        roff[i] = (long)(ih < 0 ? 0 : (ih >= H ? H - 1 : ih)) * s.h;
+        coff[i] = (long)(iw < 0 ? 0 : (iw >= W ? W - 1 : iw)) * s.w;
+    }
     float v[CV][16];
 #pragma unroll
     for (int e = 0; e < CV; ++e) {
         const int c = cq * CV + e;
-        if (c < C) {
-            const T* xp = x + n * s.n + c * s.c;
-            float d[4][4];
+        const unsigned chkeep = c < C ? 0xffffffffu : 0u;
+        const T* xp = x + n * s.n + (c < C ? c : C - 1) * s.c;
+        float d[4][4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int ih = h0 + i, iw = w0 + j;
-                    const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
-                    d[i][j] = ok ? to_f32(xp[ih * s.h + iw * s.w]) : 0.f;
-                }
-            input_tile_transform(d, v[e]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) v[e][i] = 0.f;
-        }
+            for (int j = 0; j < 4; ++j)
+                d[i][j] = mask_keep(to_f32(xp[roff[i] + coff[j]]), rkeep[i] & ckeep[j] & chkeep);
+        input_tile_transform(d, v[e]);
     }
     const size_t plane = (size_t)Cp * Pp;
     T* vp = V + ((size_t)cq * Pp + p) * CV;
