@@ -53,9 +53,10 @@ template <> struct Mma<bf16_t> {
 //
 // Block tile 128 filters x 128 tiles, 4 waves in a 2x2 arrangement, each wave
 // 64x64 = 2x2 MFMA tiles.  The reduction is consumed NV channel vectors at a
-// time from LDS, double-buffered: the next slab travels HBM -> registers while
-// the current one feeds the MFMAs, then registers -> the other LDS buffer, one
-// barrier per slab.
+// time from two LDS stages; the next slab travels HBM -> LDS directly
+// (global_load_lds_dwordx4: one instruction moves 64 channel vectors = 1 KB,
+// lane l to LDS row base + 16*l) while the current one feeds the MFMAs.  No
+// staging registers, no LDS store instructions; one wait + barrier per slab.
 // =============================================================================
 constexpr int GEMM_BM = 128, GEMM_BN = 128;
 
@@ -68,8 +69,9 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
                                                             int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
-    __shared__ vec As[2][NV][GEMM_BM];
-    __shared__ vec Bs[2][NV][GEMM_BN];
+    // separate arrays per stage so the compiler can tell the stage being filled from the one being read
+    __shared__ vec As0[NV][GEMM_BM], As1[NV][GEMM_BM];
+    __shared__ vec Bs0[NV][GEMM_BN], Bs1[NV][GEMM_BN];
 
     // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so the
     // ids that share an XCD walk the filter tiles of one tile column first and the V slab
@@ -90,7 +92,6 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int lrow = tid >> 7, lcol = tid & 127;   // rows lrow + 2*h
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -100,52 +101,59 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    vec ra[NV / 2], rb[NV / 2];
-    auto gload = [&](int ch) {
+    typedef std::integral_constant<int, 0> par0_t;
+    typedef std::integral_constant<int, 1> par1_t;
+    // a stage is 2*NV rows of 128 vectors = 4*NV pieces of 64 vectors; wave w issues pieces w, w+4, ...
+    auto stage_load = [&](auto par, int ch) {
+        constexpr int S = decltype(par)::value;
         const int q0 = ch * NV;
 #pragma unroll
-        for (int h = 0; h < NV / 2; ++h) {
-            ra[h] = Ub[(size_t)(q0 + lrow + 2 * h) * Kp + lcol];
-            rb[h] = Vb[(size_t)(q0 + lrow + 2 * h) * Pp + lcol];
+        for (int i = 0; i < NV; ++i) {
+            const int piece = wave + 4 * i;              // 0 .. 4*NV-1, wave-uniform
+            const int opnd = piece / (2 * NV);           // 0: U, 1: V
+            const int row = (piece >> 1) % NV, half = piece & 1;
+            const vec* src = opnd ? Vb + (size_t)(q0 + row) * Pp + half * 64 + lane
+                                  : Ub + (size_t)(q0 + row) * Kp + half * 64 + lane;
+            vec* dst = opnd ? (S ? &Bs1[row][half * 64] : &Bs0[row][half * 64])
+                            : (S ? &As1[row][half * 64] : &As0[row][half * 64]);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
         }
     };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int h = 0; h < NV / 2; ++h) {
-            As[buf][lrow + 2 * h][lcol] = ra[h];
-            Bs[buf][lrow + 2 * h][lcol] = rb[h];
-        }
-    };
-
     const int nch = CQ / NV;
-    gload(0);
-    lstore(0);
-    __syncthreads();
-
-    for (int ch = 0; ch < nch; ++ch) {
-        const int buf = ch & 1;
-        if (ch + 1 < nch) gload(ch + 1);
+    auto iteration = [&](auto par, int ch) {
+        constexpr int S = decltype(par)::value;
+        stage_load(std::integral_constant<int, 1 - S>{}, ch + 1 < nch ? ch + 1 : ch);   // surplus load never read
 #pragma unroll
         for (int g = 0; g < NV / 2; ++g) {
             vec a[2], b[2];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (PK) {
-                    a[t] = Bs[buf][2 * g + lh][wm * 64 + t * 32 + l32];
-                    b[t] = As[buf][2 * g + lh][wn * 64 + t * 32 + l32];
-                } else {
-                    a[t] = As[buf][2 * g + lh][wm * 64 + t * 32 + l32];
-                    b[t] = Bs[buf][2 * g + lh][wn * 64 + t * 32 + l32];
-                }
+            for (int q = 0; q < 2; ++q) {
+                const vec fa = S ? As1[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32]
+                                 : As0[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32];
+                const vec fb = S ? Bs1[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32]
+                                 : Bs0[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32];
+                a[q] = PK ? fb : fa;
+                b[q] = PK ? fa : fb;
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) Mma<T>::run(a[i], b[j], acc[i][j]);
         }
-        if (ch + 1 < nch) lstore(buf ^ 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's pieces of the next stage are in LDS
         __syncthreads();
+    };
+
+    stage_load(par0_t{}, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    int ch = 0;
+    for (; ch + 1 < nch; ch += 2) {
+        iteration(par0_t{}, ch);
+        iteration(par1_t{}, ch + 1);
     }
+    if (ch < nch) iteration(par0_t{}, ch);
 
     float* Mb = Mo + (size_t)xi * Kp * Pp;
 #pragma unroll
@@ -300,7 +308,8 @@ __global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, 
     };
     // One k-group per iteration: start the next stage's loads, multiply the
     // current stage (fragments fetched two coordinates ahead of their MFMAs),
-    // then wait for the loads and meet the other waves.
+    // then wait for the loads and meet the other waves.  (Handing the row loads
+    // out one per coordinate instead of as a burst measured slower.)
     vec fu[3], fv[3];
     auto iteration = [&](auto par, int g) {
         constexpr int S = decltype(par)::value;

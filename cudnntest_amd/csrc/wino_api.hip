@@ -218,9 +218,6 @@ int launch_gemm(int dtype, int porder, int Cp, int Kp, long Pp, const void* U, c
     const bool pk = porder == WINO_PRODUCT_PK;
     switch (dtype) {
     case WINO_F32:
-        if (Cp % 32 == 0 && getenv("WINO_NV8"))
-            return pk ? launch_gemm_t<float, 8, true>(Cp, Kp, Pp, U, V, Mo, st)
-                      : launch_gemm_t<float, 8, false>(Cp, Kp, Pp, U, V, Mo, st);
         return pk ? launch_gemm_t<float, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
                   : launch_gemm_t<float, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
     case WINO_F16:
@@ -326,8 +323,7 @@ int pick_algo(int dtype, const Geometry& g) {
         if (g.C <= 128) return WINO_ALGO_EPILOGUE;
         return WINO_ALGO_STAGED;
     }
-    if (g.C >= 16 && g.C <= 64 && g.K <= 64) return WINO_ALGO_FUSED;
-    return WINO_ALGO_EPILOGUE;
+    return WINO_ALGO_EPILOGUE;   // 16-bit operands: the fp32 product tensor is the largest HBM stream, drop it
 }
 
 int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
