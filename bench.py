@@ -14,7 +14,7 @@ Prints ONE JSON line:
   ms_per_step  ms per layer (per 13-layer pass for vgg16_all13)
   roofline     the dominant kernel -- the batched GEMM, or the kernel that contains it -- timed with
                HIP events recorded by the library on the launch stream, against the dense MFMA peak;
-               algorithmic flops per launch = 2*16*P*K*C
+               algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4)
   cpu_baseline the oracle's fp32 OpenMP direct convolution on this host's cores (reported, not a target)
   stages       per-stage ms and achieved GB/s (algorithmic bytes) or TFLOP/s
 """
@@ -40,6 +40,9 @@ WORKLOADS = {
     "vgg16_conv5_N64_C512_K512_H14": [(64, 512, 512, 14)],
     "vgg16_conv1_2_N32_C64_K64_H224": [(32, 64, 64, 224)],
     "vgg16_all13": None,   # filled from synth.VGG16_CONV at N=32
+    # the one shape the reference publishes latencies for (layoutTest/NHWC/result.num: NHWC, N=1..128)
+    "ref_H22_C128_K128_N64": [(64, 128, 128, 22)],
+    "ref_H22_C128_K128_N128": [(128, 128, 128, 22)],
 }
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (summaries and the copy-kernel scale factor under profiles/), keyed by
@@ -58,7 +61,7 @@ def main():
     ap.add_argument("--workload", default="vgg16_conv3_N32_C256_K256_H56", choices=sorted(WORKLOADS))
     ap.add_argument("--layout", default="NCHW", choices=["NCHW", "NHWC", "CHWN"])
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
-    ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain copy kernel of the first layer's input (known size) three times, so a "
@@ -85,7 +88,7 @@ def main():
     tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
     dt = {"f32": ops.F32, "f16": ops.F16, "bf16": ops.BF16}[args.dtype]
     algo = {"auto": ops.ALGO_AUTO, "staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE,
-            "fused": ops.ALGO_FUSED}[args.algo]
+            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4}[args.algo]
     es = 4 if args.dtype == "f32" else 2
 
     tensors, host_inputs = [], []
@@ -132,16 +135,17 @@ def main():
     gemm_flops = alg_in = alg_out = alg_flt = 0.0
     resolved = []
     for (N, C, K, H) in layers:
-        g = ops.geometry(dt, N, C, K, H, H, 1)
-        P = g["P"]
         a = ops.pick_algo(dt, N, C, K, H, H) if algo == ops.ALGO_AUTO else algo
+        f4 = a == ops.ALGO_STAGED_F4
+        g = ops.f4_geometry(dt, N, C, K, H, H, 1) if f4 else ops.geometry(dt, N, C, K, H, H, 1)
+        P, nxi = g["P"], (36 if f4 else 16)
         resolved.append(ops.ALGO_NAMES[a])
-        gemm_flops += 2.0 * 16 * P * K * C
-        alg_flt += (9 + 16) * K * C * es
+        gemm_flops += 2.0 * nxi * P * K * C
+        alg_flt += (9 + nxi) * K * C * es
         if a != ops.ALGO_FUSED:
-            alg_in += N * C * H * H * es + 16 * P * C * es
-        if a == ops.ALGO_STAGED:
-            alg_out += 16 * P * K * 4 + N * K * H * H * es
+            alg_in += N * C * H * H * es + nxi * P * C * es
+        if a in (ops.ALGO_STAGED, ops.ALGO_STAGED_F4):
+            alg_out += nxi * P * K * 4 + N * K * H * H * es
     stages = {}
     for name, nbytes in (("filter", alg_flt), ("input", alg_in), ("output", alg_out)):
         if per_step[name] > 0 and nbytes > 0:
@@ -152,7 +156,8 @@ def main():
     achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[args.dtype]
     stages["gemm"] = {"ms": round(gemm_ms, 4), "TFLOPs": round(achieved, 2)}
-    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_out_kernel", "fused": "fused_conv_kernel"}
+    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_out_kernel", "fused": "fused_conv_kernel",
+              "staged_f4": "gemm_128x128_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"
     traffic = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label))
     roofline = {"bound": "mfma", "kernel": kernel.get(algo_label, "per-layer choice"),
@@ -168,7 +173,8 @@ def main():
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": args.workload, "layers": len(layers), "N": N0, "C": C0, "K": K0, "H": H0, "W": H0,
                    "pad": 1, "layout": args.layout, "algo": args.algo, "resolved_algo": resolved,
-                   "winograd": "F(2x2,3x3)", "filter_transform_in_step": True, "relu": multi},
+                   "winograd": "F(4x4,3x3)" if algo_label == "staged_f4" else "F(2x2,3x3)",
+                   "filter_transform_in_step": True, "relu": multi},
         "roofline": roofline,
         "stages": stages,
     }

@@ -94,6 +94,7 @@ constexpr int kKPad = 128;   // filter dimension of U / Mo
 constexpr int kPPad = 128;   // tile dimension of V / Mo
 
 struct Geometry {
+    int m;          // outputs per tile side: 2 for F(2x2,3x3), 4 for F(4x4,3x3)
     int N, C, K, H, W, pad;
     int Ho, Wo, th, tw;
     long P;
@@ -103,14 +104,15 @@ struct Geometry {
 
 __host__ inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
 
-__host__ inline bool make_geometry(int dtype, int N, int C, int K, int H, int W, int pad, Geometry* g) {
+__host__ inline bool make_geometry(int dtype, int N, int C, int K, int H, int W, int pad, Geometry* g, int m = 2) {
+    g->m = m;
     if (N <= 0 || C <= 0 || K <= 0 || H <= 0 || W <= 0 || pad < 0 || pad > 1) return false;
     g->N = N; g->C = C; g->K = K; g->H = H; g->W = W; g->pad = pad;
     g->Ho = H + 2 * pad - 2;
     g->Wo = W + 2 * pad - 2;
     if (g->Ho <= 0 || g->Wo <= 0) return false;
-    g->th = (g->Ho + 1) / 2;
-    g->tw = (g->Wo + 1) / 2;
+    g->th = (g->Ho + m - 1) / m;
+    g->tw = (g->Wo + m - 1) / m;
     g->P = (long)N * g->th * g->tw;
     g->Cp = (int)round_up(C, c_pad(dtype));
     g->Kp = (int)round_up(K, kKPad);

@@ -1,0 +1,222 @@
+// Winograd F(4x4,3x3) transform kernels -- the reference's own tile size
+// (6x6 input tiles, 36 coordinates, 4x4 outputs per tile):
+//   comparison/wrapedConv_NCHW.cuh:836-855 (B^T d B), :879-899 (G g G^T), :1084-1101 (A^T m A)
+//
+//   B^T = [ 4  0 -5  0 1 0 ]   G = [ 1/4    0     0  ]   A^T = [ 1 1  1 1  1 0 ]
+//         [ 0 -4 -4  1 1 0 ]       [-1/6  -1/6  -1/6 ]         [ 0 1 -1 2 -2 0 ]
+//         [ 0  4 -4 -1 1 0 ]       [-1/6   1/6  -1/6 ]         [ 0 1  1 4  4 0 ]
+//         [ 0 -2 -1  2 1 0 ]       [ 1/24  1/12  1/6 ]         [ 0 1 -1 8 -8 1 ]
+//         [ 0  2 -1 -2 1 0 ]       [ 1/24 -1/12  1/6 ]
+//         [ 0  4  0 -5 0 1 ]       [ 0     0     1   ]
+//
+// Operand layouts are those of the F(2x2) path with 36 coordinates instead of 16:
+//   U[36][Cp/CV][Kp][CV]   V[36][Cp/CV][Pp][CV]   Mo[36][Kp][Pp] (or [36][Pp][Kp])
+// with th = ceil(Ho/4), tw = ceil(Wo/4), P = N*th*tw.
+#pragma once
+#include "common.hpp"
+
+namespace wino {
+
+__device__ __forceinline__ void bt6(const float d[6], float o[6]) {
+    o[0] = 4.f * d[0] - 5.f * d[2] + d[4];
+    o[1] = -4.f * (d[1] + d[2]) + d[3] + d[4];
+    o[2] = 4.f * (d[1] - d[2]) - d[3] + d[4];
+    o[3] = -2.f * d[1] - d[2] + 2.f * d[3] + d[4];
+    o[4] = 2.f * d[1] - d[2] - 2.f * d[3] + d[4];
+    o[5] = 4.f * d[1] - 5.f * d[3] + d[5];
+}
+
+// v (36, row-major 6x6) = B^T d B
+__device__ __forceinline__ void input_tile_transform_f4(const float d[6][6], float* v) {
+    float t[6][6];
+#pragma unroll
+    for (int j = 0; j < 6; ++j) {
+        float col[6], o[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) col[i] = d[i][j];
+        bt6(col, o);
+#pragma unroll
+        for (int i = 0; i < 6; ++i) t[i][j] = o[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 6; ++i) bt6(t[i], v + 6 * i);
+}
+
+__device__ __forceinline__ void g6(float g0, float g1, float g2, float o[6]) {
+    o[0] = 0.25f * g0;
+    o[1] = (-g0 - g1 - g2) * (1.f / 6.f);
+    o[2] = (-g0 + g1 - g2) * (1.f / 6.f);
+    o[3] = g0 * (1.f / 24.f) + g1 * (1.f / 12.f) + g2 * (1.f / 6.f);
+    o[4] = g0 * (1.f / 24.f) - g1 * (1.f / 12.f) + g2 * (1.f / 6.f);
+    o[5] = g2;
+}
+
+// u (36) = G g G^T
+__device__ __forceinline__ void filter_tile_transform_f4(const float g[3][3], float* u) {
+    float t[6][3];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+        float o[6];
+        g6(g[0][s], g[1][s], g[2][s], o);
+#pragma unroll
+        for (int i = 0; i < 6; ++i) t[i][s] = o[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 6; ++i) g6(t[i][0], t[i][1], t[i][2], u + 6 * i);
+}
+
+__device__ __forceinline__ void at6(const float m[6], float o[4]) {
+    o[0] = m[0] + m[1] + m[2] + m[3] + m[4];
+    o[1] = m[1] - m[2] + 2.f * (m[3] - m[4]);
+    o[2] = m[1] + m[2] + 4.f * (m[3] + m[4]);
+    o[3] = m[1] - m[2] + 8.f * (m[3] - m[4]) + m[5];
+}
+
+// y (4x4) = A^T m A
+__device__ __forceinline__ void output_tile_transform_f4(const float m[36], float y[4][4]) {
+    float t[4][6];
+#pragma unroll
+    for (int j = 0; j < 6; ++j) {
+        float col[6], o[4];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) col[i] = m[6 * i + j];
+        at6(col, o);
+#pragma unroll
+        for (int a = 0; a < 4; ++a) t[a][j] = o[a];
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) at6(t[a], y[a]);
+}
+
+// ---- filter transform: thread per (filter k, channel c), k fastest --------------------------
+// One channel per thread (36 live values); the CV channels of a vector are written by CV
+// different threads, 4 or 2 bytes each -- the filter bank is small and transformed once.
+template <typename T>
+__global__ __launch_bounds__(256) void filter_transform_f4_kernel(const T* __restrict__ w, T* __restrict__ U,
+                                                                   FltStrides s, int K, int C, int Kp, int Cp) {
+    constexpr int CV = ChanVec<T>::n;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    const int c = blockIdx.y;
+    if (k >= Kp) return;
+    float u[36];
+    if (k < K && c < C) {
+        float g[3][3];
+        const T* wp = w + k * s.k + c * s.c;
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
+        filter_tile_transform_f4(g, u);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 36; ++i) u[i] = 0.f;
+    }
+    const size_t plane = (size_t)Cp * Kp;
+    T* up = U + ((size_t)(c / CV) * Kp + k) * CV + (c % CV);
+#pragma unroll
+    for (int xi = 0; xi < 36; ++xi) up[xi * plane] = from_f32<T>(u[xi]);
+}
+
+// ---- input transform, layout-generic -------------------------------------------------------
+// Thread per (channel-in-vector e, tile p, channel vector cq) with e fastest: the CV lanes of
+// one tile write the CV elements of one 16-byte vector, so a wave's store is one contiguous
+// run of V.  One channel per thread keeps the 36 + 36 live values in registers.  Loads go to
+// clamped addresses and are masked afterwards (all 36 in flight together).
+template <typename T>
+__global__ __launch_bounds__(256) void input_transform_f4_generic_kernel(const T* __restrict__ x, T* __restrict__ V,
+                                                                          ActStrides s, int N, int C, int H, int W,
+                                                                          int pad, int th, int tw, long P, long Pp,
+                                                                          int Cp, int order) {
+    constexpr int CV = ChanVec<T>::n;
+    const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int e = (int)(gid % CV);
+    const long p = gid / CV;
+    const int cq = blockIdx.y;
+    if (p >= P) return;
+    const int c = cq * CV + e;
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    const int h0 = 4 * ty - pad, w0 = 4 * tx - pad;
+    long roff[6], coff[6];
+    unsigned rkeep[6], ckeep[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+        const int ih = h0 + i, iw = w0 + i;
+        rkeep[i] = (ih >= 0 && ih < H) ? 0xffffffffu : 0u;
+        ckeep[i] = (iw >= 0 && iw < W) ? 0xffffffffu : 0u;
+        roff[i] = (long)(ih < 0 ? 0 : (ih >= H ? H - 1 : ih)) * s.h;
+        coff[i] = (long)(iw < 0 ? 0 : (iw >= W ? W - 1 : iw)) * s.w;
+    }
+    const unsigned chkeep = c < C ? 0xffffffffu : 0u;
+    const T* xp = x + n * s.n + (c < C ? c : C - 1) * s.c;
+    float d[6][6], v[36];
+#pragma unroll
+    for (int i = 0; i < 6; ++i)
+#pragma unroll
+        for (int j = 0; j < 6; ++j) d[i][j] = mask_keep(to_f32(xp[roff[i] + coff[j]]), rkeep[i] & ckeep[j] & chkeep);
+    input_tile_transform_f4(d, v);
+    const size_t plane = (size_t)Cp * Pp;
+    T* vp = V + ((size_t)cq * Pp + p) * CV + e;
+#pragma unroll
+    for (int xi = 0; xi < 36; ++xi) vp[xi * plane] = from_f32<T>(v[xi]);
+}
+
+// ---- output transform ------------------------------------------------------------------------------
+// PK = false: Mo[36][Kp][Pp], thread per (tile p, filter k), p fastest
+// PK = true : Mo[36][Pp][Kp], thread per (filter k, tile p), k fastest
+template <typename T, bool PK>
+__global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* __restrict__ Mo, T* __restrict__ y,
+                                                                   ActStrides s, int N, int K, int Ho, int Wo, int th,
+                                                                   int tw, long P, long Pp, int Kp, int order,
+                                                                   int relu) {
+    long p;
+    int k;
+    if (PK) {
+        k = blockIdx.x * blockDim.x + threadIdx.x;
+        p = (long)blockIdx.y * blockDim.y + threadIdx.y;
+    } else {
+        p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+        k = blockIdx.y;
+    }
+    if (p >= P || k >= K) return;
+    const size_t plane = (size_t)Kp * Pp;
+    const float* mp = PK ? Mo + (size_t)p * Kp + k : Mo + (size_t)k * Pp + p;
+    float m[36];
+#pragma unroll
+    for (int xi = 0; xi < 36; ++xi) m[xi] = mp[xi * plane];
+    float o[4][4];
+    output_tile_transform_f4(m, o);
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    if (relu) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) o[a][b] = fmaxf(o[a][b], 0.f);
+    }
+    T* yp = y + n * s.n + k * s.c;
+    if (s.w == 1 && (Wo & 3) == 0 && (s.h & 3) == 0 && (s.c & 3) == 0 && (s.n & 3) == 0) {
+        // W-contiguous destination, rows a multiple of 4 wide: one 4-element store per output row
+        struct alignas(4 * sizeof(T)) Quad { T e[4]; };
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int oh = 4 * ty + a;
+            if (oh < Ho) {
+                Quad q;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) q.e[b] = from_f32<T>(o[a][b]);
+                *reinterpret_cast<Quad*>(yp + oh * s.h + 4 * tx) = q;
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int oh = 4 * ty + a, ow = 4 * tx + b;
+            if (oh < Ho && ow < Wo) yp[oh * s.h + ow * s.w] = from_f32<T>(o[a][b]);
+        }
+}
+
+}  // namespace wino

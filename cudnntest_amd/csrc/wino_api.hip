@@ -11,6 +11,7 @@
 #include "fused.hpp"
 #include "gemm.hpp"
 #include "transforms.hpp"
+#include "transforms_f4.hpp"
 
 using namespace wino;
 
@@ -114,12 +115,13 @@ struct Scratch {
 
 Scratch scratch_layout(const Geometry& g, int dtype) {
     const size_t es = dtype_size(dtype);
+    const size_t nxi = (size_t)(g.m + 2) * (g.m + 2);
     auto al = [](size_t v) { return (v + 255) / 256 * 256; };
     Scratch s;
     s.u_off = 0;
-    s.v_off = al(16 * (size_t)g.Cp * g.Kp * es);
-    s.m_off = s.v_off + al(16 * (size_t)g.Cp * g.Pp * es);
-    s.total = s.m_off + al(16 * (size_t)g.Kp * g.Pp * sizeof(float));
+    s.v_off = al(nxi * (size_t)g.Cp * g.Kp * es);
+    s.m_off = s.v_off + al(nxi * (size_t)g.Cp * g.Pp * es);
+    s.total = s.m_off + al(nxi * (size_t)g.Kp * g.Pp * sizeof(float));
     return s;
 }
 
@@ -203,29 +205,29 @@ int launch_output_transform(int layout, int order, int porder, unsigned flags, i
 }
 
 template <typename T, int NV, bool PK>
-int launch_gemm_t(int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
+int launch_gemm_t(int nxi, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
     const int kTiles = Kp / GEMM_BM, pTiles = (int)(Pp / GEMM_BN);
-    dim3 grid((unsigned)((pTiles + 7) / 8 * 8 * kTiles), 16), block(256);
+    dim3 grid((unsigned)((pTiles + 7) / 8 * 8 * kTiles), nxi), block(256);
     hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp, Kp,
                        Pp, kTiles, pTiles);
     LAUNCH_CHECK("batched_gemm");
     return WINO_OK;
 }
 
-int launch_gemm(int dtype, int porder, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo,
+int launch_gemm(int nxi, int dtype, int porder, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo,
                 hipStream_t st) {
     // slab per barrier: 4 channel vectors = 16 channels (fp32) or 32 (16-bit); Cp is a multiple of that
     const bool pk = porder == WINO_PRODUCT_PK;
     switch (dtype) {
     case WINO_F32:
-        return pk ? launch_gemm_t<float, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
-                  : launch_gemm_t<float, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<float, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, st)
+                  : launch_gemm_t<float, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, st);
     case WINO_F16:
-        return pk ? launch_gemm_t<f16_t, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
-                  : launch_gemm_t<f16_t, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<f16_t, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, st)
+                  : launch_gemm_t<f16_t, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, st);
     case WINO_BF16:
-        return pk ? launch_gemm_t<bf16_t, 4, true>(Cp, Kp, Pp, U, V, Mo, st)
-                  : launch_gemm_t<bf16_t, 4, false>(Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<bf16_t, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, st)
+                  : launch_gemm_t<bf16_t, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -299,6 +301,47 @@ int launch_fused(int src, int dst, int dtype, int order, unsigned flags, const G
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
+// ---- F(4x4,3x3) stage launchers -----------------------------------------------------------------
+template <typename T>
+int launch_f4_filter(int layout, int K, int C, int Kp, int Cp, const void* w, void* U, hipStream_t st) {
+    dim3 grid((Kp + 255) / 256, Cp), block(256);
+    hipLaunchKernelGGL(filter_transform_f4_kernel<T>, grid, block, 0, st, (const T*)w, (T*)U,
+                       flt_strides(layout, K, C), K, C, Kp, Cp);
+    LAUNCH_CHECK("f4_filter_transform");
+    return WINO_OK;
+}
+
+template <typename T>
+int launch_f4_input(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st) {
+    constexpr int CV = ChanVec<T>::n;
+    dim3 grid((unsigned)((g.P * CV + 255) / 256), g.Cp / CV), block(256);
+    hipLaunchKernelGGL(input_transform_f4_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
+                       act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
+                       g.Cp, order);
+    LAUNCH_CHECK("f4_input_transform");
+    return WINO_OK;
+}
+
+template <typename T>
+int launch_f4_output(int layout, int order, int porder, unsigned flags, int N, int K, int Ho, int Wo, int Kp, long P,
+                     long Pp, const float* Mo, void* y, hipStream_t st) {
+    const int th = (Ho + 3) / 4, tw = (Wo + 3) / 4;
+    const int relu = (flags & WINO_FLAG_RELU) ? 1 : 0;
+    if (porder == WINO_PRODUCT_PK) {
+        int bx = 64;
+        while (bx < K && bx < 256) bx *= 2;
+        dim3 block(bx, 256 / bx), grid((K + bx - 1) / bx, (unsigned)((P + block.y - 1) / block.y));
+        hipLaunchKernelGGL((output_transform_f4_kernel<T, true>), grid, block, 0, st, Mo, (T*)y,
+                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+    } else {
+        dim3 grid((unsigned)((P + 255) / 256), K), block(256);
+        hipLaunchKernelGGL((output_transform_f4_kernel<T, false>), grid, block, 0, st, Mo, (T*)y,
+                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+    }
+    LAUNCH_CHECK("f4_output_transform");
+    return WINO_OK;
+}
+
 #define DISPATCH_DTYPE(dtype, CALL)                          \
     switch (dtype) {                                         \
     case WINO_F32: { typedef float T; return CALL; }         \
@@ -326,16 +369,54 @@ int pick_algo(int dtype, const Geometry& g) {
     return WINO_ALGO_EPILOGUE;   // 16-bit operands: the fp32 product tensor is the largest HBM stream, drop it
 }
 
+int conv_f4_impl(int src, int dst, int dtype, unsigned flags, int N, int C, int K, int H, int W, int pad,
+                 const void* x, const void* w, const void* Upre, void* y, void* stream) {
+    Geometry g;
+    if (!make_geometry(dtype, N, C, K, H, W, pad, &g, 4))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
+    hipStream_t st = (hipStream_t)stream;
+    const Scratch sc = scratch_layout(g, dtype);
+    void* base = nullptr;
+    int rc = arena_get(sc.total, &base);
+    if (rc) return rc;
+    char* b = (char*)base;
+    void* U = b + sc.u_off;
+    void* V = b + sc.v_off;
+    float* Mo = (float*)(b + sc.m_off);
+    const int order = tile_order_for(src, dst);
+    const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
+    if (Upre) {
+        U = const_cast<void*>(Upre);
+    } else {
+        StageScope t(WINO_STAGE_FILTER, st);
+        rc = wino_f4_filter_transform(src, dtype, K, C, w, U, stream);
+        if (rc) return rc;
+    }
+    {
+        StageScope t(WINO_STAGE_INPUT, st);
+        rc = wino_f4_input_transform(src, dtype, order, N, C, H, W, pad, x, V, stream);
+        if (rc) return rc;
+    }
+    {
+        StageScope t(WINO_STAGE_GEMM, st);
+        rc = launch_gemm(36, dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
+        if (rc) return rc;
+    }
+    StageScope t(WINO_STAGE_OUTPUT, st);
+    return wino_f4_output_transform(dst, dtype, order, porder, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
+}
+
 int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
               const void* x, const void* w, const void* Upre, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
-    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_FUSED) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
+    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_STAGED_F4) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
     if (!x || (!w && !Upre) || !y) return fail(WINO_ERR_INVALID, "null tensor pointer");
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     if (algo == WINO_ALGO_AUTO) algo = pick_algo(dtype, g);
+    if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(src, dst, dtype, flags, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype);
@@ -371,7 +452,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
     {
         StageScope t(WINO_STAGE_GEMM, st);
-        rc = launch_gemm(dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
+        rc = launch_gemm(16, dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
         if (rc) return rc;
     }
     StageScope t(WINO_STAGE_OUTPUT, st);
@@ -465,7 +546,7 @@ int wino_batched_gemm(int dtype, int product_order, int C, int K, long P, const 
     if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
     if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
-    return launch_gemm(dtype, product_order, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
+    return launch_gemm(16, dtype, product_order, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
                        (hipStream_t)stream);
 }
 
@@ -515,6 +596,68 @@ int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int 
                            a, dst, N, C, H, W);
     LAUNCH_CHECK("layout_transform");
     return WINO_OK;
+}
+
+int wino_f4_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp,
+                     int* Kp, long* Pp) {
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    Geometry g;
+    if (!make_geometry(dtype, N, C, K, H, W, pad, &g, 4))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
+    if (th) *th = g.th;
+    if (tw) *tw = g.tw;
+    if (P) *P = g.P;
+    if (Cp) *Cp = g.Cp;
+    if (Kp) *Kp = g.Kp;
+    if (Pp) *Pp = g.Pp;
+    return WINO_OK;
+}
+
+int wino_f4_filter_transform(int layout, int dtype, int K, int C, const void* w, void* U, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!w || !U) return fail(WINO_ERR_INVALID, "null pointer");
+    if (K <= 0 || C <= 0) return fail(WINO_ERR_INVALID, "bad filter bank K=%d C=%d", K, C);
+    const int Kp = (int)round_up(K, kKPad), Cp = (int)round_up(C, c_pad(dtype));
+    DISPATCH_DTYPE(dtype, launch_f4_filter<T>(layout, K, C, Kp, Cp, w, U, (hipStream_t)stream));
+}
+
+int wino_f4_input_transform(int layout, int dtype, int tile_order, int N, int C, int H, int W, int pad, const void* x,
+                            void* V, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
+    if (!x || !V) return fail(WINO_ERR_INVALID, "null pointer");
+    Geometry g;
+    if (!make_geometry(dtype, N, C, 1, H, W, pad, &g, 4))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d H=%d W=%d pad=%d", N, C, H, W, pad);
+    DISPATCH_DTYPE(dtype, launch_f4_input<T>(layout, tile_order, g, x, V, (hipStream_t)stream));
+}
+
+int wino_f4_batched_gemm(int dtype, int product_order, int C, int K, long P, const void* U, const void* V, float* Mo,
+                         void* stream) {
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
+    if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
+    if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
+    return launch_gemm(36, dtype, product_order, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad),
+                       round_up(P, kPPad), U, V, Mo, (hipStream_t)stream);
+}
+
+int wino_f4_output_transform(int layout, int dtype, int tile_order, int product_order, unsigned flags, int N, int K,
+                             int Ho, int Wo, const float* Mo, void* y, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
+    if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
+    if (!Mo || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    if (N <= 0 || K <= 0 || Ho <= 0 || Wo <= 0)
+        return fail(WINO_ERR_INVALID, "bad shape N=%d K=%d Ho=%d Wo=%d", N, K, Ho, Wo);
+    const long P = (long)N * ((Ho + 3) / 4) * ((Wo + 3) / 4);
+    const int Kp = (int)round_up(K, kKPad);
+    const long Pp = round_up(P, kPPad);
+    DISPATCH_DTYPE(dtype, launch_f4_output<T>(layout, tile_order, product_order, flags, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
+                                              (hipStream_t)stream));
 }
 
 int wino_stage_timing(int enable) {

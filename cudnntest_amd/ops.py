@@ -23,7 +23,7 @@ from . import _lib
 
 NCHW, NHWC, CHWN = 0, 1, 2
 F32, F16, BF16 = 0, 1, 2
-ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED = 0, 1, 2, 3
+ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED, ALGO_STAGED_F4 = 0, 1, 2, 3, 4
 TILES_BATCH_MAJOR, TILES_BATCH_MINOR = 0, 1
 PRODUCT_KP, PRODUCT_PK = 0, 1
 FLAG_RELU = 1
@@ -81,7 +81,8 @@ def geometry(dtype, N, C, K, H, W, pad):
     return dict(th=th.value, tw=tw.value, P=P.value, Cp=Cp.value, Kp=Kp.value, Pp=Pp.value)
 
 
-ALGO_NAMES = {ALGO_AUTO: "auto", ALGO_STAGED: "staged", ALGO_EPILOGUE: "epilogue", ALGO_FUSED: "fused"}
+ALGO_NAMES = {ALGO_AUTO: "auto", ALGO_STAGED: "staged", ALGO_EPILOGUE: "epilogue", ALGO_FUSED: "fused",
+              ALGO_STAGED_F4: "staged_f4"}
 
 
 def pick_algo(dtype, N, C, K, H, W, pad=1):
@@ -195,6 +196,53 @@ def gemm_output(U, V, N, C, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR
     y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=U.dtype, device=U.device)
     _lib.check(_lib.load().wino_gemm_output(int(layout), _dt(U), tile_order, FLAG_RELU if relu else 0, N, C, K, Ho,
                                             Wo, _ptr(U), _ptr(V), _ptr(y), _stream()), "wino_gemm_output")
+    return y
+
+
+# ---- F(4x4,3x3) stages -------------------------------------------------------------------
+
+def f4_geometry(dtype, N, C, K, H, W, pad):
+    import ctypes
+    th, tw, Cp, Kp = (ctypes.c_int() for _ in range(4))
+    P, Pp = ctypes.c_long(), ctypes.c_long()
+    _lib.check(_lib.load().wino_f4_geometry(dtype, N, C, K, H, W, pad, th, tw, P, Cp, Kp, Pp), "wino_f4_geometry")
+    return dict(th=th.value, tw=tw.value, P=P.value, Cp=Cp.value, Kp=Kp.value, Pp=Pp.value)
+
+
+def f4_filter_transform(w, layout=NCHW):
+    K, C = flt_dims(layout, w)
+    g = f4_geometry(_dt(w), 1, C, K, 6, 6, 1)
+    cv = 16 // w.element_size()
+    U = torch.empty((36, g["Cp"] // cv, g["Kp"], cv), dtype=w.dtype, device=w.device)
+    _lib.check(_lib.load().wino_f4_filter_transform(int(layout), _dt(w), K, C, _ptr(w), _ptr(U), _stream()),
+               "wino_f4_filter_transform")
+    return U
+
+
+def f4_input_transform(x, pad=1, layout=NCHW, tile_order=TILES_BATCH_MAJOR):
+    N, C, H, W = act_dims(layout, x)
+    g = f4_geometry(_dt(x), N, C, 1, H, W, pad)
+    cv = 16 // x.element_size()
+    V = torch.zeros((36, g["Cp"] // cv, g["Pp"], cv), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().wino_f4_input_transform(int(layout), _dt(x), tile_order, N, C, H, W, pad, _ptr(x),
+                                                   _ptr(V), _stream()), "wino_f4_input_transform")
+    return V
+
+
+def f4_batched_gemm(U, V, C, K, P, product_order=PRODUCT_KP):
+    shape = (36, U.shape[2], V.shape[2]) if product_order == PRODUCT_KP else (36, V.shape[2], U.shape[2])
+    Mo = torch.empty(shape, dtype=torch.float32, device=U.device)
+    _lib.check(_lib.load().wino_f4_batched_gemm(_dt(U), product_order, C, K, P, _ptr(U), _ptr(V), _ptr(Mo),
+                                                _stream()), "wino_f4_batched_gemm")
+    return Mo
+
+
+def f4_output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False,
+                        dtype=torch.float32, product_order=PRODUCT_KP):
+    y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=dtype, device=Mo.device)
+    _lib.check(_lib.load().wino_f4_output_transform(int(layout), _DTYPES[dtype], tile_order, product_order,
+                                                    FLAG_RELU if relu else 0, N, K, Ho, Wo, _ptr(Mo), _ptr(y),
+                                                    _stream()), "wino_f4_output_transform")
     return y
 
 

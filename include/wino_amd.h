@@ -35,8 +35,11 @@ typedef enum {
     WINO_ALGO_STAGED = 1,   /* four kernels: input/filter transform, 16-way GEMM, output transform
                                (the pipeline of comparison/wrapedConv_NCHW.cuh:408-452) */
     WINO_ALGO_EPILOGUE = 2, /* output transform applied in the GEMM epilogue (no product tensor in HBM) */
-    WINO_ALGO_FUSED = 3     /* one kernel: input transform, multiply-accumulate and output transform
+    WINO_ALGO_FUSED = 3,    /* one kernel: input transform, multiply-accumulate and output transform
                                (the structure of fusedTest/winotrans.cuh:1452 Winofuse4433) */
+    WINO_ALGO_STAGED_F4 = 4 /* the staged pipeline in F(4x4,3x3) -- 6x6 tiles, 36 coordinates, the reference's
+                               own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101).
+                               Never chosen by WINO_ALGO_AUTO. */
 } wino_algo_t;
 
 /* order of the tile index p inside the transformed operands */
@@ -130,6 +133,18 @@ int wino_output_transform(int layout, int dtype, int tile_order, int product_ord
 /* GEMM with the output transform in its epilogue: y directly from U and V. */
 int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int N, int C, int K,
                      int Ho, int Wo, const void *U, const void *V, void *y, void *stream);
+
+/* ---- the same four stages in F(4x4,3x3): 36 coordinates, th = ceil(Ho/4), tw = ceil(Wo/4).
+ * Operand layouts as above with 36 in place of 16; sizes from wino_f4_geometry. */
+int wino_f4_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int *th, int *tw, long *P,
+                     int *Cp, int *Kp, long *Pp);
+int wino_f4_filter_transform(int layout, int dtype, int K, int C, const void *w, void *U, void *stream);
+int wino_f4_input_transform(int layout, int dtype, int tile_order, int N, int C, int H, int W, int pad,
+                            const void *x, void *V, void *stream);
+int wino_f4_batched_gemm(int dtype, int product_order, int C, int K, long P, const void *U, const void *V,
+                         float *Mo, void *stream);
+int wino_f4_output_transform(int layout, int dtype, int tile_order, int product_order, unsigned flags, int N,
+                             int K, int Ho, int Wo, const float *Mo, void *y, void *stream);
 
 /* ---- plain layout permutation (bench harness; the reference has no such kernel) */
 int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void *in,
