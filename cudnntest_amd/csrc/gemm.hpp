@@ -124,22 +124,29 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
     auto iteration = [&](auto par, int ch) {
         constexpr int S = decltype(par)::value;
         stage_load(std::integral_constant<int, 1 - S>{}, ch + 1 < nch ? ch + 1 : ch);   // surplus load never read
-#pragma unroll
-        for (int g = 0; g < NV / 2; ++g) {
-            vec a[2], b[2];
+        // fence: without it the compiler sinks the loads to the end of the slab, right before the wait
+        __builtin_amdgcn_sched_barrier(0);
+        vec a[2][2], b[2][2];                      // fragments of k-group g live in set g&1, fetched one group ahead
+        auto frag_load = [&](int g) {
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
                 const vec fa = S ? As1[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32]
                                  : As0[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32];
                 const vec fb = S ? Bs1[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32]
                                  : Bs0[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32];
-                a[q] = PK ? fb : fa;
-                b[q] = PK ? fa : fb;
+                a[g & 1][q] = PK ? fb : fa;
+                b[g & 1][q] = PK ? fa : fb;
             }
+        };
+        frag_load(0);
+#pragma unroll
+        for (int g = 0; g < NV / 2; ++g) {
+            if (g + 1 < NV / 2) frag_load(g + 1);
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) Mma<T>::run(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < 2; ++j) Mma<T>::run(a[g & 1][i], b[g & 1][j], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's pieces of the next stage are in LDS
         __syncthreads();
@@ -154,6 +161,110 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
         iteration(par1_t{}, ch + 1);
     }
     if (ch < nch) iteration(par0_t{}, ch);
+
+    float* Mb = Mo + (size_t)xi * Kp * Pp;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ri = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);   // MFMA row
+                const int ci = wn * 64 + j * 32 + l32;                               // MFMA column (lane)
+                if (PK) Mb[(size_t)(p0 + ri) * Kp + k0 + ci] = acc[i][j][r];
+                else Mb[(size_t)(k0 + ri) * Pp + p0 + ci] = acc[i][j][r];
+            }
+}
+
+// Register-staged variant of the same tile: the next slab travels HBM -> registers while the
+// current one feeds the MFMAs, then registers -> the other LDS buffer.  Measured faster than the
+// direct-to-LDS version for fp32 (115 vs 106 TFLOP/s on N=32, C=K=256, H=56: LDS writes of the
+// in-flight DMA compete with the fragment reads of the long fp32 MFMAs), slower for 16-bit
+// operands (257 vs 355 TFLOP/s), so fp32 uses this one.
+template <typename T, int NV, bool PK>
+__global__ __launch_bounds__(256) void gemm_128x128_reg_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                            float* __restrict__ Mo, int Cp, int Kp, long Pp,
+                                                            int kTiles, int pTiles) {
+    typedef typename Mma<T>::vec vec;
+    constexpr int CV = ChanVec<T>::n;
+    __shared__ vec As[2][NV][GEMM_BM];
+    __shared__ vec Bs[2][NV][GEMM_BN];
+
+    // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so the
+    // ids that share an XCD walk the filter tiles of one tile column first and the V slab
+    // they share is fetched from HBM once, into that XCD's L2.
+    const int xi = blockIdx.y;
+    const int b = blockIdx.x;
+    const int xcd = b & 7, jj = b >> 3;
+    const int ktile = jj % kTiles;
+    const int ptile = (jj / kTiles) * 8 + xcd;
+    if (ptile >= pTiles) return;
+    const long p0 = (long)ptile * GEMM_BN;
+    const int k0 = ktile * GEMM_BM;
+    const int CQ = Cp / CV;
+    const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
+    const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int lrow = tid >> 7, lcol = tid & 127;   // rows lrow + 2*h
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    vec ra[NV / 2], rb[NV / 2];
+    auto gload = [&](int ch) {
+        const int q0 = ch * NV;
+#pragma unroll
+        for (int h = 0; h < NV / 2; ++h) {
+            ra[h] = Ub[(size_t)(q0 + lrow + 2 * h) * Kp + lcol];
+            rb[h] = Vb[(size_t)(q0 + lrow + 2 * h) * Pp + lcol];
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < NV / 2; ++h) {
+            As[buf][lrow + 2 * h][lcol] = ra[h];
+            Bs[buf][lrow + 2 * h][lcol] = rb[h];
+        }
+    };
+
+    const int nch = CQ / NV;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+
+    for (int ch = 0; ch < nch; ++ch) {
+        const int buf = ch & 1;
+        if (ch + 1 < nch) gload(ch + 1);
+#pragma unroll
+        for (int g = 0; g < NV / 2; ++g) {
+            vec a[2], b[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (PK) {
+                    a[t] = Bs[buf][2 * g + lh][wm * 64 + t * 32 + l32];
+                    b[t] = As[buf][2 * g + lh][wn * 64 + t * 32 + l32];
+                } else {
+                    a[t] = As[buf][2 * g + lh][wm * 64 + t * 32 + l32];
+                    b[t] = Bs[buf][2 * g + lh][wn * 64 + t * 32 + l32];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) Mma<T>::run(a[i], b[j], acc[i][j]);
+        }
+        if (ch + 1 < nch) lstore(buf ^ 1);
+        __syncthreads();
+    }
 
     float* Mb = Mo + (size_t)xi * Kp * Pp;
 #pragma unroll
