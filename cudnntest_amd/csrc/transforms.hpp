@@ -77,22 +77,45 @@ __global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restri
     const int cq = blockIdx.y;
     if (k >= Kp) return;
     float u[CV][16];
+    float g[CV][3][3];
+    // all CV channels of this vector exist, and the filter bank allows 16-byte loads
+    const bool full = k < K && (cq + 1) * CV <= C && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
+    if (full && s.c == 9 && s.s == 1 && (C * 9) % CV == 0) {
+        // [K][C][3][3]: the CV channels of this thread are 9*CV contiguous elements -> nine 16-byte loads
+        const Pack16<T>* wp = reinterpret_cast<const Pack16<T>*>(w + k * s.k + (long)cq * CV * 9);
 #pragma unroll
-    for (int e = 0; e < CV; ++e) {
-        const int c = cq * CV + e;
-        if (k < K && c < C) {
-            float g[3][3];
-            const T* wp = w + k * s.k + c * s.c;
+        for (int i = 0; i < 9; ++i) {
+            const Pack16<T> pk = wp[i];
+#pragma unroll
+            for (int j = 0; j < CV; ++j) {
+                const int f = i * CV + j;                 // flat index: channel f/9, tap f%9
+                g[f / 9][(f % 9) / 3][f % 3] = to_f32(pk.e[j]);
+            }
+        }
+    } else if (full && s.c == 1 && C % CV == 0) {
+        // [K][3][3][C]: each tap holds the CV channels contiguously -> one 16-byte load per tap
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                const Pack16<T> pk = *reinterpret_cast<const Pack16<T>*>(w + k * s.k + r * s.r + q * s.s + cq * CV);
+#pragma unroll
+                for (int e = 0; e < CV; ++e) g[e][r][q] = to_f32(pk.e[e]);
+            }
+    } else {
+#pragma unroll
+        for (int e = 0; e < CV; ++e) {
+            const int c = cq * CV + e;
+            const bool ok = k < K && c < C;
+            const T* wp = w + (ok ? k : 0) * s.k + (ok ? c : 0) * s.c;
 #pragma unroll
             for (int r = 0; r < 3; ++r)
 #pragma unroll
-                for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
-            filter_tile_transform(g, u[e]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) u[e][i] = 0.f;
+                for (int q = 0; q < 3; ++q) g[e][r][q] = ok ? to_f32(wp[r * s.r + q * s.s]) : 0.f;
         }
     }
+#pragma unroll
+    for (int e = 0; e < CV; ++e) filter_tile_transform(g[e], u[e]);
     const size_t plane = (size_t)Cp * Kp;   // elements per coordinate
     T* up = U + ((size_t)cq * Kp + k) * CV;
 #pragma unroll
