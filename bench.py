@@ -156,7 +156,7 @@ def main():
     achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[args.dtype]
     stages["gemm"] = {"ms": round(gemm_ms, 4), "TFLOPs": round(achieved, 2)}
-    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_out_kernel", "fused": "fused_conv_kernel",
+    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_conv_kernel",
               "staged_f4": "gemm_128x128_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"
     traffic = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label))

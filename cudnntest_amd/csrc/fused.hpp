@@ -7,8 +7,9 @@
 // accumulator advances, and A^T(.)A runs on the accumulators at the end -- here
 // for 4x4 tiles, all three layouts, zero padding, any C and K, on MFMA.
 //
-// A workgroup owns 64 filters x 64 tiles for all 16 coordinates (the geometry
-// of gemm_out_kernel, whose MFMA core and epilogue it shares).  Per k-group
+// A workgroup owns 64 filters x 64 tiles for all 16 coordinates: each of its 4
+// waves keeps sixteen 32x32 MFMA accumulators (256 AGPRs), so the output
+// transform runs in registers (winograd_epilogue in gemm.hpp).  Per k-group
 // (GC = 2*CV channels):
 //   U slab  <- HBM by direct-to-LDS loads (pre-transformed filters, as in the reference)
 //   V slab  <- built in the kernel: each thread owns UNITS (tile, channel) pairs, keeps

@@ -281,16 +281,8 @@ __global__ __launch_bounds__(256) void gemm_128x128_reg_kernel(const T* __restri
 }
 
 // =============================================================================
-// GEMM with the output transform in its epilogue.
-//
-// A workgroup owns a 64-filter x 64-tile patch for ALL 16 Winograd coordinates:
-// each of its 4 waves keeps sixteen 32x32 MFMA accumulators (256 accumulation
-// registers, the whole AGPR file of a wave), so when the reduction over
-// channels ends every lane holds the 16 coordinates of its (filter, tile) pairs
-// and applies A^T(.)A in registers; the product tensor never reaches HBM.
-//
-// The reduction runs one k-group at a time through LDS ([xi][2][64] channel
-// vectors for U and for V), double-buffered through registers.
+// Shared pieces of the kernels that apply the output transform in registers
+// (patch = 64 filters x 64 tiles per workgroup, 4 waves of 32x32 MFMA tiles).
 //
 // SWAP = false: MFMA rows = filters, lanes = tiles  (stores contiguous along the
 //               tile axis: NCHW, or CHWN with batch-minor tiles)
@@ -361,26 +353,46 @@ __device__ __forceinline__ void winograd_epilogue(const floatx16 (&acc)[16], T* 
     }
 }
 
-template <typename T, bool SWAP>
-__global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, const T* __restrict__ V,
-                                                       T* __restrict__ y, ActStrides ys, int N, int K, int Ho, int Wo,
-                                                       int th, int tw, long P, int Cp, int Kp, long Pp, int order,
-                                                       int relu, int kTiles, int pTiles) {
+// =============================================================================
+// GEMM with the output transform in its epilogue, one Winograd ROW at a time.
+//
+// A workgroup owns a 64-filter x 64-tile patch; only the 4 coordinates of one
+// row i of the 4x4 coordinate grid are resident at a time: a wave
+// keeps four 32x32 MFMA accumulators (64 AGPRs) and, in VGPRs, the four output
+// planes y00, y01, y10, y11 of its (filter, tile) pairs.  When the channel
+// reduction of row i ends, the row is folded into the outputs,
+//     T_b = (A^T-column transform of m_i0..m_i3)_b,   y_ab += (A^T)_{a i} * T_b,
+// and the accumulators restart for row i+1.  A wave needs ~170 registers instead
+// of 512, so three workgroups share a CU: their barriers and load latencies
+// overlap, and three times as many waves pull operands from L2 (one 4-wave
+// workgroup per CU cannot draw more than ~38 B/clk, which is what a kernel that
+// keeps all 16 coordinates resident -- one wave per SIMD -- needs at fp32 MFMA
+// peak; that variant measured 8-14 % slower on every shape).
+//
+// A stage is NVG k-groups of one row: [4][2*NVG][64] channel vectors of U and of V,
+// moved HBM -> LDS by global_load_lds_dwordx4, two static stages.  The 4 * nst
+// stages of a patch form one pipeline that runs across the row boundaries.
+// =============================================================================
+template <typename T, bool SWAP, int NVG>
+__global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                           T* __restrict__ y, ActStrides ys, int N, int K, int Ho,
+                                                           int Wo, int th, int tw, long P, int Cp, int Kp, long Pp,
+                                                           int order, int relu, int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
-    // two stages, each a U slab and a V slab of [xi][lane half][64] channel vectors (4 x 32 KB);
-    // separate arrays so the compiler can tell the stage being filled from the stage being read
-    __shared__ vec Us0[16][2][GO_T], Us1[16][2][GO_T];
-    __shared__ vec Vs0[16][2][GO_T], Vs1[16][2][GO_T];
+    constexpr int NV = 2 * NVG;                     // channel vectors per stage and coordinate
+    __shared__ vec Us0[4][NV][GO_T], Us1[4][NV][GO_T];
+    __shared__ vec Vs0[4][NV][GO_T], Vs1[4][NV][GO_T];
 
     const int b = blockIdx.x;
-    const int xcd = b & 7, j = b >> 3;
-    const int ktile = j % kTiles;
-    const int ptile = (j / kTiles) * 8 + xcd;
+    const int xcd = b & 7, jb = b >> 3;
+    const int ktile = jb % kTiles;
+    const int ptile = (jb / kTiles) * 8 + xcd;
     if (ptile >= pTiles) return;
     const int k0 = ktile * GO_T;
     const long p0 = (long)ptile * GO_T;
     const int CQ = Cp / CV;
+    const int nst = CQ / NV;                        // stages per row (even)
     const vec* Ug = reinterpret_cast<const vec*>(U);
     const vec* Vg = reinterpret_cast<const vec*>(V);
 
@@ -389,69 +401,104 @@ __global__ __launch_bounds__(256) void gemm_out_kernel(const T* __restrict__ U, 
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    floatx16 acc[16];
+    floatx16 acc[4];
+    floatx16 yo[4];                                  // y00, y01, y10, y11
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[xi][r] = 0.f;
+        for (int r = 0; r < 16; ++r) { acc[j][r] = 0.f; yo[j][r] = 0.f; }
 
-    // HBM -> LDS without passing through registers: one global_load_lds_dwordx4 moves a
-    // whole (xi, lane-half) row of 64 channel vectors (lane l -> LDS row base + 16*l).
-    // A stage is 64 such rows (32 of U, 32 of V); wave w issues rows w, w+4, ...
-    const int ngrp = CQ / 2;
     typedef std::integral_constant<int, 0> par0_t;
     typedef std::integral_constant<int, 1> par1_t;
-    auto stage_load = [&](auto par, int g) {
+    // a stage is 8*NV rows of 64 vectors (4 coordinates x NV vectors, U and V); wave w issues rows w, w+4, ...
+    auto stage_load = [&](auto par, int row_i, int st) {
         constexpr int S = decltype(par)::value;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = wave + 4 * i;            // 0..31, wave-uniform
-            const int xi = row >> 1, h = row & 1;
-            const vec* usrc = Ug + ((size_t)xi * CQ + 2 * g + h) * Kp + k0 + lane;
-            const vec* vsrc = Vg + ((size_t)xi * CQ + 2 * g + h) * Pp + p0 + lane;
-            vec* udst = S ? &Us1[xi][h][0] : &Us0[xi][h][0];
-            vec* vdst = S ? &Vs1[xi][h][0] : &Vs0[xi][h][0];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)usrc,
-                                             (__attribute__((address_space(3))) void*)udst, 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc,
-                                             (__attribute__((address_space(3))) void*)vdst, 16, 0, 0);
+        for (int q = 0; q < 2 * NV; ++q) {
+            const int r = wave + 4 * q;              // 0 .. 8*NV-1, wave-uniform
+            const int opnd = r / (4 * NV);           // 0: U, 1: V
+            const int j = (r / NV) & 3, v = r % NV;
+            const size_t cvec = (size_t)(4 * row_i + j) * CQ + (size_t)st * NV + v;
+            const vec* src = opnd ? Vg + cvec * Pp + p0 + lane : Ug + cvec * Kp + k0 + lane;
+            vec* dst = opnd ? (S ? &Vs1[j][v][0] : &Vs0[j][v][0]) : (S ? &Us1[j][v][0] : &Us0[j][v][0]);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
         }
     };
-    // One k-group per iteration: start the next stage's loads, multiply the
-    // current stage (fragments fetched two coordinates ahead of their MFMAs),
-    // then wait for the loads and meet the other waves.  (Handing the row loads
-    // out one per coordinate instead of as a burst measured slower.)
-    vec fu[3], fv[3];
-    auto iteration = [&](auto par, int g) {
+    int ni = 0, nstg = 0;                            // (row, stage) of the next stage to request
+    auto advance = [&]() {
+        if (++nstg == nst) { nstg = 0; ++ni; }
+        if (ni > 3) { ni = 3; nstg = nst - 1; }      // past the end: re-request the last stage (never read)
+    };
+    auto iteration = [&](auto par) {
         constexpr int S = decltype(par)::value;
-        auto frag_load = [&](int xi) {
-            fu[xi % 3] = S ? Us1[xi][lh][(SWAP ? wn : wm) * 32 + l32] : Us0[xi][lh][(SWAP ? wn : wm) * 32 + l32];
-            fv[xi % 3] = S ? Vs1[xi][lh][(SWAP ? wm : wn) * 32 + l32] : Vs0[xi][lh][(SWAP ? wm : wn) * 32 + l32];
-        };
-        stage_load(std::integral_constant<int, 1 - S>{}, g + 1 < ngrp ? g + 1 : g);   // surplus load never read
-        frag_load(0);
-        frag_load(1);
+        stage_load(std::integral_constant<int, 1 - S>{}, ni, nstg);
+        advance();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int xi = 0; xi < 16; ++xi) {
-            if (xi + 2 < 16) frag_load(xi + 2);
-            if (SWAP) Mma<T>::run(fv[xi % 3], fu[xi % 3], acc[xi]);
-            else Mma<T>::run(fu[xi % 3], fv[xi % 3], acc[xi]);
-        }
+        for (int g = 0; g < NVG; ++g)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const vec fu = S ? Us1[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32] : Us0[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32];
+                const vec fv = S ? Vs1[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32] : Vs0[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32];
+                if (SWAP) Mma<T>::run(fv, fu, acc[j]);
+                else Mma<T>::run(fu, fv, acc[j]);
+            }
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's rows of the next stage are in LDS
+        __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's rows of the next stage are in LDS
         __syncthreads();
     };
 
-    stage_load(par0_t{}, 0);
+    stage_load(par0_t{}, 0, 0);
+    advance();
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    for (int g = 0; g < ngrp; g += 2) {   // ngrp is even: Cp is a multiple of 4 channel vectors
-        iteration(par0_t{}, g);
-        iteration(par1_t{}, g + 1);
+
+    for (int i = 0; i < 4; ++i) {
+        for (int st = 0; st < nst; st += 2) {
+            iteration(par0_t{});
+            iteration(par1_t{});
+        }
+        // fold row i:  A^T = [1 1 1 0; 0 1 -1 -1], column i = (c0, c1); the products with 0 and +-1 are exact
+        const float c0 = i < 3 ? 1.f : 0.f;
+        const float c1 = i == 0 ? 0.f : (i == 1 ? 1.f : -1.f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float t0 = acc[0][r] + acc[1][r] + acc[2][r];
+            const float t1 = acc[1][r] - acc[2][r] - acc[3][r];
+            yo[0][r] = fmaf(c0, t0, yo[0][r]);
+            yo[1][r] = fmaf(c0, t1, yo[1][r]);
+            yo[2][r] = fmaf(c1, t0, yo[2][r]);
+            yo[3][r] = fmaf(c1, t1, yo[3][r]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
+        }
     }
 
-    winograd_epilogue<T, SWAP>(acc, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
+    // ---- stores: register r is MFMA row 8*(r/4) + 4*lh + r%4, the lane's l32 the MFMA column ----
+    if (!SWAP) {
+        const long p = p0 + wn * 32 + l32;
+        if (p >= P) return;
+        int n, ty, tx;
+        decode_tile(p, order, N, th, tw, n, ty, tx);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (k >= K) continue;
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
+        }
+    } else {
+        const int k = k0 + wn * 32 + l32;
+        if (k >= K) return;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const long p = p0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (p >= P) continue;
+            int n, ty, tx;
+            decode_tile(p, order, N, th, tw, n, ty, tx);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
+        }
+    }
 }
 
 }  // namespace wino

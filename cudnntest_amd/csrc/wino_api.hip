@@ -236,34 +236,40 @@ int launch_gemm(int nxi, int dtype, int porder, int Cp, int Kp, long Pp, const v
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
-template <typename T, bool SWAP>
-int launch_gemm_out_t(int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y, int dst,
-                      hipStream_t st) {
-    auto kern = gemm_out_kernel<T, SWAP>;
+template <typename T, bool SWAP, int NVG>
+int launch_gemm_rows_t(int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y, int dst,
+                       hipStream_t st) {
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
-    hipLaunchKernelGGL(kern, grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
+    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG>), grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
                        act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
                        g.Pp, order, (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
-    LAUNCH_CHECK("gemm_output");
+    LAUNCH_CHECK("gemm_rows");
     return WINO_OK;
 }
 
 template <typename T>
-int launch_gemm_out_d(int dst, int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y,
-                      hipStream_t st) {
-    if (dst == WINO_NHWC) return launch_gemm_out_t<T, true>(order, flags, g, U, V, y, dst, st);
-    return launch_gemm_out_t<T, false>(order, flags, g, U, V, y, dst, st);
+int launch_gemm_rows_d(int dst, int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y,
+                       hipStream_t st) {
+    // stages per row must be even: one k-group per stage always is (Cp is a multiple of 4 channel
+    // vectors); two k-groups per stage (fewer barriers, measured faster) when Cp allows it
+    constexpr int CV = ChanVec<T>::n;
+    const bool two = (g.Cp / CV) % 8 == 0;
+    if (dst == WINO_NHWC)
+        return two ? launch_gemm_rows_t<T, true, 2>(order, flags, g, U, V, y, dst, st)
+                   : launch_gemm_rows_t<T, true, 1>(order, flags, g, U, V, y, dst, st);
+    return two ? launch_gemm_rows_t<T, false, 2>(order, flags, g, U, V, y, dst, st)
+               : launch_gemm_rows_t<T, false, 1>(order, flags, g, U, V, y, dst, st);
 }
 
 int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* U, const void* V,
                     void* y, hipStream_t st) {
     switch (dtype) {
-    case WINO_F32: return launch_gemm_out_d<float>(dst, order, flags, g, U, V, y, st);
-    case WINO_F16: return launch_gemm_out_d<f16_t>(dst, order, flags, g, U, V, y, st);
-    case WINO_BF16: return launch_gemm_out_d<bf16_t>(dst, order, flags, g, U, V, y, st);
+    case WINO_F32: return launch_gemm_rows_d<float>(dst, order, flags, g, U, V, y, st);
+    case WINO_F16: return launch_gemm_rows_d<f16_t>(dst, order, flags, g, U, V, y, st);
+    case WINO_BF16: return launch_gemm_rows_d<bf16_t>(dst, order, flags, g, U, V, y, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -366,9 +372,9 @@ int pick_algo(int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
     if (patches < 512) return WINO_ALGO_STAGED;          // too few 64x64 patches to fill 256 CUs
     if (dtype == WINO_F32) {
-        if (g.C <= 64) return WINO_ALGO_FUSED;
+        if (g.C >= 16 && g.C <= 64 && g.K <= 64) return WINO_ALGO_FUSED;   // conv1_2: V would be 4x the input
         if (g.C <= 128) return WINO_ALGO_EPILOGUE;
-        return WINO_ALGO_STAGED;
+        return WINO_ALGO_STAGED;      // C >= 256: the 128x128 GEMM's lower L2 traffic per flop wins (tie at 256)
     }
     return WINO_ALGO_EPILOGUE;   // 16-bit operands: the fp32 product tensor is the largest HBM stream, drop it
 }
