@@ -90,3 +90,18 @@ def test_datalayout_enum_order_matches_reference():
     # enum class DataLayout { NCHW, NHWC, CHWN }  comparison/DataLayoutTrans.cuh:587-591
     assert [int(v) for v in ops.DataLayout] == [0, 1, 2]
     assert [v.name for v in ops.DataLayout] == ["NCHW", "NHWC", "CHWN"]
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """There is no fallback path: without the built library, loading raises."""
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libwino_amd.so"))
+    monkeypatch.setattr(_lib, "_lib", None)
+    with pytest.raises(RuntimeError, match="missing"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    import glob
+    for f in glob.glob(os.path.join(ROOT, "cudnntest_amd", "*.py")):
+        text = open(f).read()
+        assert "import oracle" not in text and "from oracle" not in text, f

@@ -108,3 +108,27 @@ def test_properties_at_full_size():
     y_chwn = ops.conv(x1.permute(1, 2, 3, 0).contiguous(), w.permute(1, 2, 3, 0).contiguous(), src=ops.CHWN)
     assert ((y_nhwc.permute(0, 3, 1, 2) - y1).norm() / y1.norm()).item() < 1e-6
     assert ((y_chwn.permute(3, 0, 1, 2) - y1).norm() / y1.norm()).item() < 1e-6
+
+
+def test_caller_owned_workspace(oracle):
+    """wino_set_workspace: too small a buffer is refused with WINO_ERR_WORKSPACE, a big enough one is used."""
+    from cudnntest_amd import _lib
+    L = _lib.load()
+    N, C, K, H, W = 2, 16, 24, 12, 12
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=8, integer=True)
+    xd, wd = dev(x), dev(w)
+    want = oracle.direct_conv(x, w, 1)
+    need = ops.workspace_bytes(ops.F32, N, C, K, H, W, 1)
+    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    big = torch.empty(need, dtype=torch.uint8, device="cuda")
+    try:
+        assert L.wino_set_workspace(small.data_ptr(), small.numel()) == 0
+        with pytest.raises(_lib.WinoError) as e:
+            ops.conv(xd, wd, algo=ops.ALGO_STAGED)
+        assert e.value.code == -4
+        assert L.wino_set_workspace(big.data_ptr(), big.numel()) == 0
+        for algo in ALGOS:
+            assert np.array_equal(host(ops.conv(xd, wd, algo=algo)), want)
+    finally:
+        assert L.wino_set_workspace(None, 0) == 0
+    assert np.array_equal(host(ops.conv(xd, wd)), want)
