@@ -135,7 +135,7 @@ def main():
     gemm_flops = alg_in = alg_out = alg_flt = 0.0
     resolved = []
     for (N, C, K, H) in layers:
-        a = ops.pick_algo(dt, N, C, K, H, H) if algo == ops.ALGO_AUTO else algo
+        a = ops.pick_algo(layout, dt, N, C, K, H, H) if algo == ops.ALGO_AUTO else algo
         f4 = a == ops.ALGO_STAGED_F4
         g = ops.f4_geometry(dt, N, C, K, H, H, 1) if f4 else ops.geometry(dt, N, C, K, H, H, 1)
         P, nxi = g["P"], (36 if f4 else 16)
@@ -156,7 +156,7 @@ def main():
     achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[args.dtype]
     stages["gemm"] = {"ms": round(gemm_ms, 4), "TFLOPs": round(achieved, 2)}
-    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_conv_kernel",
+    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
               "staged_f4": "gemm_128x128_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"
     traffic = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label))

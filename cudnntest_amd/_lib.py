@@ -21,7 +21,7 @@ _l = ctypes.c_long
 SYMBOLS = {
     "wino_conv": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
     "wino_conv_prepared": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
-    "wino_pick_algo": (_i, [_i] * 7),
+    "wino_pick_algo": (_i, [_i] * 8),
     "wino_geometry": (_i, [_i] * 7 + [ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l),
                                      ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l)]),
     "wino_workspace_bytes": (ctypes.c_size_t, [_i] * 7),

@@ -47,10 +47,9 @@ __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint
 template <typename T> __device__ __forceinline__ T from_f32(float f);
 template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
 template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) { return (f16_t)f; }
+// round to nearest even; gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32)
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7f800000u) != 0x7f800000u) u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-    return bf16_t{(uint16_t)(u >> 16)};
+    return bf16_t{__builtin_bit_cast(uint16_t, (__bf16)f)};
 }
 
 // v with its bits ANDed by m (m is all ones or zero).  Opaque to the optimiser on purpose:

@@ -2,51 +2,83 @@
 // multiply-accumulate over channels and output transform in one launch, with no
 // transformed-input or product tensor in HBM.  The structure of the reference's
 // fusedTest/winotrans.cuh:1452 (Winofuse4433): per channel slab, half of the
-// work is "load a raw input patch, B^T d B in registers, scatter to LDS", the
-// other half "copy the pre-transformed filter slab to LDS", then every
-// accumulator advances, and A^T(.)A runs on the accumulators at the end -- here
-// for 4x4 tiles, all three layouts, zero padding, any C and K, on MFMA.
-//
-// A workgroup owns 64 filters x 64 tiles for all 16 coordinates: each of its 4
-// waves keeps sixteen 32x32 MFMA accumulators (256 AGPRs), so the output
-// transform runs in registers (winograd_epilogue in gemm.hpp).  Per k-group
-// (GC = 2*CV channels):
-//   U slab  <- HBM by direct-to-LDS loads (pre-transformed filters, as in the reference)
-//   V slab  <- built in the kernel: each thread owns UNITS (tile, channel) pairs, keeps
-//              their 16 raw input values in registers one k-group ahead, transforms
-//              them and writes the 16 coordinates into the idle LDS stage.
+// work is "load a raw input patch, transform it in registers, scatter to LDS",
+// the other half "copy the pre-transformed filter slab to LDS", then the
+// accumulators advance, and A^T(.)A runs on the accumulators -- here for 4x4
+// tiles, all three layouts, zero padding, any C and K, on MFMA.
 #pragma once
 #include "gemm.hpp"
 
 namespace wino {
 
-// LANES_ON_CHANNELS = false: lanes walk tiles (coalesced when W or N is the contiguous axis)
-// LANES_ON_CHANNELS = true : lanes walk the GC channels of a k-group first (NHWC)
-template <typename T, bool SWAP, bool LANES_ON_CHANNELS>
-__global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x, const T* __restrict__ U,
-                                                         T* __restrict__ y, ActStrides xs, ActStrides ys, int N,
-                                                         int C, int K, int H, int W, int pad, int Ho, int Wo, int th,
-                                                         int tw, long P, int Cp, int Kp, int order, int relu,
-                                                         int kTiles, int pTiles) {
+// =============================================================================
+// The kernel has the row-at-a-time structure of gemm_rows_kernel: a workgroup
+// owns 64 filters x 64 tiles, keeps the 4 coordinates of ONE row i of the 4x4
+// coordinate grid resident, folds the row into the output tile when its channel
+// reduction ends, and is small enough (one wave ~ 240 registers, 32-64 KB of
+// LDS) for two workgroups to share a CU.  The filter rows of a stage travel
+// HBM -> LDS directly, as in gemm_rows_kernel; the tile rows are built here.
+//
+// Row i of V = B^T d B needs only two rows of the raw patch:
+//     (B^T d)_i = d_ra + sg * d_rb,   (ra, rb, sg) = (0,2,-), (1,2,+), (2,1,-), (1,3,-)
+// followed by the column transform.  Per stage (NC = NV*CV channels of one row) a
+// thread owns one tile and UN = NC/4 consecutive channels, loads 2 x 4 raw values
+// per channel one stage ahead, and writes the four coordinates as one UN-element
+// chunk each.  The raw input is read four times in total (once per row), from
+// L2 after the first.
+//
+// How a thread reads its 2 x 4 x UN raw values (the load path, not HBM, bounds this kernel):
+//   XM_SCALAR  one element per load, any strides; lanes walk tiles (coalesced for CHWN)
+//   XM_CHANVEC channels contiguous (NHWC) and C % UN == 0: the UN channels of a position are
+//              one load, and 4 neighbouring lanes cover the NC channels of a position
+//   XM_ROW     columns contiguous (NCHW) and W >= 4: the 4 columns of a patch row are one
+//              load that starts at a column clamped into [0, W-4]; lanes of edge tiles pick
+//              their columns out of the shifted quadruple
+// =============================================================================
+enum { XM_SCALAR = 0, XM_CHANVEC = 1, XM_ROW = 2 };
+
+// b in the lanes whose bit is set in the lane mask m, a in the others.  Opaque to the optimiser on
+// purpose: written with ?: on a per-lane index, the compiler turns the column shuffle of XM_ROW into
+// an indexed array in scratch memory.
+__device__ __forceinline__ float lane_select(float a, float b, unsigned long m) {
+    float r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(m));
+    return r;
+}
+
+template <typename T> struct alignas(sizeof(T)) Quad { T v[4]; };
+
+template <typename T, bool SWAP, int XM, int NVG>
+__global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict__ x, const T* __restrict__ U,
+                                                            T* __restrict__ y, ActStrides xs, ActStrides ys, int N,
+                                                            int C, int K, int H, int W, int pad, int Ho, int Wo,
+                                                            int th, int tw, long P, int Cp, int Kp, int order,
+                                                            int relu, int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
-    constexpr int GC = 2 * CV;                 // channels per k-group
-    constexpr int UNITS = 64 * GC / 256;       // (tile, channel) pairs per thread: 2 (fp32) or 4 (16-bit)
-    // s_waitcnt vmcnt(VM) lgkmcnt(0): at most VM (the x loads of one k-group, capped by the 6-bit field) still in flight
-    constexpr int VM = 16 * UNITS < 63 ? 16 * UNITS : 63;
+    constexpr int NV = 2 * NVG;                // channel vectors per stage and coordinate
+    constexpr int NC = NV * CV;                // channels per stage
+    constexpr int UN = NC / 4;                 // channels per thread (64 tiles x NC channels over 256 threads)
+    static_assert(CV % UN == 0, "a thread's channels must lie inside one channel vector");
+    constexpr int XL = XM == XM_CHANVEC ? 8 : (XM == XM_ROW ? 2 * UN : 8 * UN);   // x loads per thread and stage
+    // s_waitcnt vmcnt(VM) lgkmcnt(0): the filter rows (issued before the x loads) have landed
+    constexpr int VM = XL < 63 ? XL : 63;      // 6-bit field
     constexpr int WAIT_IMM = (VM & 0xF) | (0x7 << 4) | (0 << 8) | ((VM >> 4) << 14);
-    __shared__ vec Us0[16][2][GO_T], Us1[16][2][GO_T];
-    __shared__ vec Vs0[16][2][GO_T], Vs1[16][2][GO_T];
+    typedef typename std::conditional<UN * sizeof(T) == 16, uint4, uint2>::type chunk_t;   // UN channels
+    static_assert(sizeof(chunk_t) == UN * sizeof(T), "chunk size");
+    constexpr int VPAD = XM == XM_CHANVEC ? 2 : 0;   // V rows padded where lanes walk channel vectors first
+    __shared__ vec Us0[4][NV][GO_T], Us1[4][NV][GO_T];
+    __shared__ vec Vs0[4][NV][GO_T + VPAD], Vs1[4][NV][GO_T + VPAD];
 
     const int b = blockIdx.x;
-    const int xcd = b & 7, j = b >> 3;
-    const int ktile = j % kTiles;
-    const int ptile = (j / kTiles) * 8 + xcd;
+    const int xcd = b & 7, jb = b >> 3;
+    const int ktile = jb % kTiles;
+    const int ptile = (jb / kTiles) * 8 + xcd;
     if (ptile >= pTiles) return;
     const int k0 = ktile * GO_T;
     const long p0 = (long)ptile * GO_T;
     const int CQ = Cp / CV;
-    const int ngrp = CQ / 2;
+    const int nst = CQ / NV;                   // stages per row (even)
     const vec* Ug = reinterpret_cast<const vec*>(U);
 
     const int tid = threadIdx.x;
@@ -54,171 +86,229 @@ __global__ __launch_bounds__(256) void fused_conv_kernel(const T* __restrict__ x
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    // ---- this thread's (tile, channel) units: fixed for the whole kernel ----------------
-    int u_tile[UNITS], u_ch[UNITS];            // tile index inside the patch, channel inside the k-group
-    unsigned u_row[UNITS][4], u_col[UNITS][4]; // element offsets of the patch rows (incl. image) and columns, clamped inside
-    unsigned u_mask[UNITS];                    // bit i*4+j set when position (i, j) lies inside the image
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-        if (LANES_ON_CHANNELS) {
-            u_ch[u] = tid % GC;
-            u_tile[u] = tid / GC + u * (256 / GC);
-        } else {
-            u_tile[u] = tid & 63;
-            u_ch[u] = (tid >> 6) * UNITS + u;
-        }
-        const long p = p0 + u_tile[u];
+    // ---- this thread's tile and channels: fixed for the whole kernel --------------------
+    const int tile = XM == XM_CHANVEC ? tid >> 2 : tid & 63;
+    const int ch0 = (XM == XM_CHANVEC ? tid & 3 : tid >> 6) * UN;   // first of its UN channels inside a stage
+    unsigned u_col[4];                         // XM_ROW: [0] = offset of the clamped first column; else the 4 clamped columns
+    unsigned cw[4];                            // all ones when column j of the patch lies inside the image (and the tile exists)
+    unsigned img_off;                          // element offset of the tile's image
+    int ih0;                                   // image row of patch row 0
+    int dcol = 0;                              // XM_ROW: patch column j is element j + dcol of the loaded quadruple
+    {
+        const long p = p0 + tile;
         int n = 0, ty = 0, tx = 0;
         const bool pvalid = p < P;
         if (pvalid) decode_tile(p, order, N, th, tw, n, ty, tx);
-        u_mask[u] = 0;
-        unsigned rmask = 0, cmask = 0;
+        img_off = (unsigned)(n * xs.n);
+        ih0 = 2 * ty - pad;
+        const int iw0 = 2 * tx - pad;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int ih = 2 * ty - pad + i, iw = 2 * tx - pad + i;
-            if (ih >= 0 && ih < H) rmask |= 1u << i;
-            if (iw >= 0 && iw < W) cmask |= 1u << i;
-            const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);     // clamped: the load stays inside x, the
-            const int iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);     // value is discarded through u_mask
-            u_row[u][i] = (unsigned)(n * xs.n + ihc * xs.h);
-            u_col[u][i] = (unsigned)(iwc * xs.w);
+            const int iw = iw0 + i;
+            cw[i] = (pvalid && iw >= 0 && iw < W) ? 0xFFFFFFFFu : 0u;
+            const int iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);     // clamped: the load stays inside x, the
+            u_col[i] = (unsigned)(iwc * xs.w);                       // value is discarded through the masks
         }
-        if (pvalid) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if ((rmask >> i) & 1u) u_mask[u] |= cmask << (4 * i);
+        if (XM == XM_ROW) {
+            const int s0 = min(max(iw0, 0), W - 4);
+            dcol = iw0 - s0;                   // -1 at the left edge, 1 or 2 at the right edge, else 0
+            u_col[0] = (unsigned)s0;
         }
     }
+    // lane masks of the edge tiles (wave-uniform 64-bit values, fixed for the whole kernel)
+    const unsigned long laneL = __ballot(dcol == -1), laneR1 = __ballot(dcol == 1), laneR2 = __ballot(dcol == 2);
 
-    floatx16 acc[16];
+    floatx16 acc[4];
+    floatx16 yo[4];                            // y00, y01, y10, y11
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[xi][r] = 0.f;
+        for (int r = 0; r < 16; ++r) { acc[j][r] = 0.f; yo[j][r] = 0.f; }
 
     typedef std::integral_constant<int, 0> par0_t;
     typedef std::integral_constant<int, 1> par1_t;
 
-    // Raw input patches of the k-group after the one being multiplied.
-    T xr[UNITS][16];
-    auto x_load_unit = [&](int g, int u) {
-        const int c = g * GC + u_ch[u];
-        const unsigned coff = c < C ? (unsigned)(c * xs.c) : 0u;   // channel padding: masked out in v_piece
+    // ---- raw rows ra, rb of the patch, requested one stage ahead ----------------------------
+    // x_prep fixes the stage to request (offsets, masks, sign); x_load_unit / x_load_all issue the
+    // loads; v_unit turns the staged values of one channel into row i of B^T d B; v_write stores
+    // the four coordinates into stage S of V.  The masks and sign of the staged values (`c` set)
+    // are those x_prep computed one iteration earlier (`n` set).
+    T xa[4][UN], xb[4][UN];                    // [column][channel]; XM_ROW: [element of the quadruple][channel]
+    unsigned ma_c = 0, mb_c = 0, cok_c = 0;    // all ones when patch row ra / rb lies inside the image; bit u: channel u is real
+    float sg_c = 0.f;
+    unsigned ma_n, mb_n, cok_n, ra_off, rb_off;
+    float sg_n;
+    int c_n;
+    auto x_prep = [&](int row_i, int st) {
+        const int ra = row_i == 0 ? 0 : (row_i == 2 ? 2 : 1);
+        const int rb = row_i < 2 ? 2 : (row_i == 2 ? 1 : 3);
+        const int iha = ih0 + ra, ihb = ih0 + rb;
+        ma_n = (iha >= 0 && iha < H) ? 0xFFFFFFFFu : 0u;
+        mb_n = (ihb >= 0 && ihb < H) ? 0xFFFFFFFFu : 0u;
+        ra_off = img_off + (unsigned)(min(max(iha, 0), H - 1) * xs.h);
+        rb_off = img_off + (unsigned)(min(max(ihb, 0), H - 1) * xs.h);
+        sg_n = row_i == 1 ? 1.f : -1.f;
+        c_n = st * NC + ch0;
+        cok_n = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned ro = u_row[u][i] + coff;
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) xr[u][i * 4 + jj] = x[ro + u_col[u][jj]];
-        }
+        for (int u = 0; u < UN; ++u) cok_n |= (c_n + u < C) ? 1u << u : 0u;
     };
-    // Building stage S of V from the staged patches, cut into 16 pieces so that one
-    // piece can ride in the shadow of each coordinate's MFMAs:
-    //   pieces 0 .. 2*UNITS-1 : per unit, mask the patch (zero padding) then B^T d B
-    //   the remaining pieces  : the LDS writes, a few coordinates each; the first UNITS
-    //                           of them also refill the patches with k-group `gload`
-    float vt[UNITS][16];
-    float dpatch[4][4];
-    auto v_piece = [&](auto par, int g, int gload, int piece) {
-        constexpr int S = decltype(par)::value;
-        constexpr int NW = 16 - 2 * UNITS;                 // pieces that write
-        constexpr int PER = (16 + NW - 1) / NW;            // coordinates per writing piece
-        if (piece < 2 * UNITS) {
-            const int u = piece >> 1;
-            if ((piece & 1) == 0) {
-                const bool cok = g * GC + u_ch[u] < C;
-                const unsigned m = cok ? u_mask[u] : 0u;
+    auto x_load_unit = [&](int u) {            // XM_SCALAR, XM_ROW
+        const unsigned coff = ((cok_n >> u) & 1u) ? (unsigned)((c_n + u) * xs.c) : 0u;
+        if (XM == XM_ROW) {
+            const Quad<T> qa = *reinterpret_cast<const Quad<T>*>(x + (ra_off + coff + u_col[0]));
+            const Quad<T> qb = *reinterpret_cast<const Quad<T>*>(x + (rb_off + coff + u_col[0]));
 #pragma unroll
-                for (int q = 0; q < 16; ++q) dpatch[q >> 2][q & 3] = ((m >> q) & 1u) ? to_f32(xr[u][q]) : 0.f;
-            } else {
-                input_tile_transform(dpatch, vt[u]);
-            }
-            return;
-        }
-        const int w = piece - 2 * UNITS;
-        if (w < UNITS && gload >= 0) x_load_unit(gload, w);
+            for (int jj = 0; jj < 4; ++jj) { xa[jj][u] = qa.v[jj]; xb[jj][u] = qb.v[jj]; }
+        } else {
 #pragma unroll
-        for (int t = 0; t < PER; ++t) {
-            const int xi = w * PER + t;
-            if (xi >= 16) continue;
-            if (LANES_ON_CHANNELS) {
-#pragma unroll
-                for (int u = 0; u < UNITS; ++u) {
-                    const int h = u_ch[u] / CV, e = u_ch[u] % CV;
-                    T* dst = reinterpret_cast<T*>(S ? &Vs1[xi][h][u_tile[u]] : &Vs0[xi][h][u_tile[u]]);
-                    dst[e] = from_f32<T>(vt[u][xi]);
-                }
-            } else {
-                // the thread's UNITS channels are consecutive elements of one channel vector: one 8-byte write
-                struct alignas(8) Chunk { T e[UNITS]; };
-                static_assert(sizeof(Chunk) == 8, "chunk must be 8 bytes");
-                const int h = u_ch[0] / CV, e0 = u_ch[0] % CV;
-                Chunk ck;
-#pragma unroll
-                for (int u = 0; u < UNITS; ++u) ck.e[u] = from_f32<T>(vt[u][xi]);
-                T* dst = reinterpret_cast<T*>(S ? &Vs1[xi][h][u_tile[0]] : &Vs0[xi][h][u_tile[0]]);
-                *reinterpret_cast<Chunk*>(dst + e0) = ck;
+            for (int jj = 0; jj < 4; ++jj) {
+                xa[jj][u] = x[ra_off + coff + u_col[jj]];
+                xb[jj][u] = x[rb_off + coff + u_col[jj]];
             }
         }
     };
-    auto u_load = [&](auto par, int g) {
-        constexpr int S = decltype(par)::value;
+    auto x_load_all = [&]() {                  // XM_CHANVEC: C % UN == 0, all UN channels real or none
+        const unsigned coff = cok_n ? (unsigned)c_n : 0u;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = wave + 4 * i;            // 0..31, wave-uniform
-            const int xi = row >> 1, h = row & 1;
-            const vec* usrc = Ug + ((size_t)xi * CQ + 2 * g + h) * Kp + k0 + lane;
-            vec* udst = S ? &Us1[xi][h][0] : &Us0[xi][h][0];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)usrc,
-                                             (__attribute__((address_space(3))) void*)udst, 16, 0, 0);
+        for (int jj = 0; jj < 4; ++jj) {
+            const chunk_t va = *reinterpret_cast<const chunk_t*>(x + (ra_off + coff + u_col[jj]));
+            const chunk_t vb = *reinterpret_cast<const chunk_t*>(x + (rb_off + coff + u_col[jj]));
+            __builtin_memcpy(xa[jj], &va, sizeof(chunk_t));
+            __builtin_memcpy(xb[jj], &vb, sizeof(chunk_t));
         }
     };
-
-    vec fu[3], fv[3];
-    auto iteration = [&](auto par, int g) {
+    auto take_next = [&]() { ma_c = ma_n; mb_c = mb_n; cok_c = cok_n; sg_c = sg_n; };
+    T out[4][UN];
+    auto v_unit = [&](int u) {
+        const bool ok = (cok_c >> u) & 1u;
+        const unsigned mau = ok ? ma_c : 0u, mbu = ok ? mb_c : 0u;
+        float da[4], db[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { da[q] = to_f32(xa[q][u]); db[q] = to_f32(xb[q][u]); }
+        if (XM == XM_ROW) {
+            // patch column j = element j + dcol of the quadruple; elements that fall outside it are
+            // columns outside the image, zeroed by cw below
+            auto pick = [&](float (&d)[4]) {
+                const float e0 = lane_select(lane_select(d[0], d[2], laneR2), d[1], laneR1);
+                const float e1 = lane_select(lane_select(lane_select(d[1], d[3], laneR2), d[2], laneR1), d[0], laneL);
+                const float e2 = lane_select(lane_select(d[2], d[3], laneR1), d[1], laneL);
+                const float e3 = lane_select(d[3], d[2], laneL);
+                d[0] = e0; d[1] = e1; d[2] = e2; d[3] = e3;
+            };
+            pick(da);
+            pick(db);
+        }
+        float r[4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+            r[jj] = mask_keep(fmaf(sg_c, mask_keep(db[jj], mbu), mask_keep(da[jj], mau)), cw[jj]);
+        out[0][u] = from_f32<T>(r[0] - r[2]);
+        out[1][u] = from_f32<T>(r[1] + r[2]);
+        out[2][u] = from_f32<T>(r[2] - r[1]);
+        out[3][u] = from_f32<T>(r[1] - r[3]);
+    };
+    auto v_write = [&](auto par) {
+        constexpr int S = decltype(par)::value;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            T* dst = reinterpret_cast<T*>(S ? &Vs1[j][ch0 / CV][tile] : &Vs0[j][ch0 / CV][tile]);
+            chunk_t ck;
+            __builtin_memcpy(&ck, out[j], sizeof(chunk_t));
+            *reinterpret_cast<chunk_t*>(dst + ch0 % CV) = ck;
+        }
+    };
+    // Building the next stage of V is cut into pieces that ride between the MFMA runs of the
+    // current stage (two workgroups of a CU run in lockstep, so VALU work that is not interleaved
+    // with a wave's own MFMAs does not overlap anybody's): pieces 0 .. WP-1 each transform UPP
+    // channels and request their values for the stage after; piece WP writes the stage.
+    constexpr int NR = 4 * NVG;                // MFMA runs per stage
+    constexpr int UPP = (UN + NR - 2) / (NR - 1);
+    constexpr int WP = (UN + UPP - 1) / UPP;
+    static_assert(WP < NR, "pieces must fit the runs");
+    auto v_piece = [&](auto par, int piece) {
+        if (piece < WP) {
+#pragma unroll
+            for (int u = piece * UPP; u < (piece + 1) * UPP && u < UN; ++u) {
+                v_unit(u);
+                if (XM != XM_CHANVEC) x_load_unit(u);
+            }
+        } else if (piece == WP) {
+            v_write(par);
+            if (XM == XM_CHANVEC) x_load_all();
+        }
+    };
+    // ---- the filter rows of a stage: 4*NV rows of 64 vectors, wave w issues rows w, w+4, ... --
+    auto u_load = [&](auto par, int row_i, int st) {
+        constexpr int S = decltype(par)::value;
+#pragma unroll
+        for (int q = 0; q < NV; ++q) {
+            const int r = wave + 4 * q;
+            const int j = r / NV, v = r % NV;
+            const vec* src = Ug + ((size_t)(4 * row_i + j) * CQ + (size_t)st * NV + v) * Kp + k0 + lane;
+            vec* dst = S ? &Us1[j][v][0] : &Us0[j][v][0];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        }
+    };
+    int ni = 0, nstg = 0;                      // (row, stage) after the one being multiplied
+    auto advance = [&]() {
+        if (++nstg == nst) { nstg = 0; ++ni; }
+        if (ni > 3) { ni = 3; nstg = nst - 1; }      // past the end: repeat the last stage (never read)
+    };
+    vec fu[2], fv[2];
+    auto iteration = [&](auto par) {
         constexpr int S = decltype(par)::value;
         typedef std::integral_constant<int, 1 - S> other_t;
-        auto frag_load = [&](int xi) {
-            fu[xi % 3] = S ? Us1[xi][lh][(SWAP ? wn : wm) * 32 + l32] : Us0[xi][lh][(SWAP ? wn : wm) * 32 + l32];
-            fv[xi % 3] = S ? Vs1[xi][lh][(SWAP ? wm : wn) * 32 + l32] : Vs0[xi][lh][(SWAP ? wm : wn) * 32 + l32];
+        auto frag_load = [&](int r) {
+            const int j = r & 3, v = 2 * (r >> 2) + lh;
+            fu[r & 1] = S ? Us1[j][v][(SWAP ? wn : wm) * 32 + l32] : Us0[j][v][(SWAP ? wn : wm) * 32 + l32];
+            fv[r & 1] = S ? Vs1[j][v][(SWAP ? wm : wn) * 32 + l32] : Vs0[j][v][(SWAP ? wm : wn) * 32 + l32];
         };
-        const int g1 = g + 1 < ngrp ? g + 1 : g;      // surplus work on the last group is never read
-        const int g2 = g + 2 < ngrp ? g + 2 : g1;
-        // filter rows of group g+1 first (the whole iteration to land); the raw patches of
-        // group g+2 are requested as soon as those of g+1 have been consumed
-        u_load(other_t{}, g1);
+        u_load(other_t{}, ni, nstg);
+        take_next();
+        advance();
+        x_prep(ni, nstg);
         frag_load(0);
-        frag_load(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int xi = 0; xi < 16; ++xi) {
-            if (xi + 2 < 16) frag_load(xi + 2);
-            v_piece(other_t{}, g1, g2, xi);
-            if (SWAP) Mma<T>::run(fv[xi % 3], fu[xi % 3], acc[xi]);
-            else Mma<T>::run(fu[xi % 3], fv[xi % 3], acc[xi]);
+        for (int r = 0; r < NR; ++r) {
+            if (r + 1 < NR) frag_load(r + 1);
+            v_piece(other_t{}, r);
+            if (SWAP) Mma<T>::run(fv[r & 1], fu[r & 1], acc[r & 3]);
+            else Mma<T>::run(fu[r & 1], fv[r & 1], acc[r & 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        // the filter rows of the next stage must be in LDS (they were issued before the x
-        // loads, and loads retire in order); the younger x loads may stay in flight
         __builtin_amdgcn_s_waitcnt(WAIT_IMM);
         __syncthreads();
     };
 
-    // prologue: stage 0 of both slabs, and the raw patches of group 1 in flight
-    u_load(par0_t{}, 0);
+    // prologue: stage (0, 0) of both operands in LDS, the raw rows of the stage after it in flight
+    x_prep(0, 0);
+    if (XM == XM_CHANVEC) x_load_all();
+    else {
+#pragma unroll
+        for (int u = 0; u < UN; ++u) x_load_unit(u);
+    }
+    u_load(par0_t{}, 0, 0);
+    take_next();
+    advance();
+    x_prep(ni, nstg);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) x_load_unit(0, u);
-#pragma unroll
-    for (int piece = 0; piece < 16; ++piece) v_piece(par0_t{}, 0, ngrp > 1 ? 1 : 0, piece);
+    for (int piece = 0; piece <= WP; ++piece) v_piece(par0_t{}, piece);
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(WAIT_IMM);
     __syncthreads();
 
-    for (int g = 0; g < ngrp; g += 2) {   // ngrp is even: Cp is a multiple of 4 channel vectors
-        iteration(par0_t{}, g);
-        iteration(par1_t{}, g + 1);
+    for (int i = 0; i < 4; ++i) {
+        for (int st = 0; st < nst; st += 2) {
+            iteration(par0_t{});
+            iteration(par1_t{});
+        }
+        rows_fold(acc, yo, i);
     }
-
-    winograd_epilogue<T, SWAP>(acc, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
+    rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
 }
 
 }  // namespace wino

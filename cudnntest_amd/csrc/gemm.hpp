@@ -312,12 +312,31 @@ __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const A
     }
 }
 
-// A^T (.) A on a wave's sixteen 32x32 accumulators, then the stores.  Register r of
-// an accumulator is MFMA row 8*(r/4) + 4*lh + r%4, the lane's l32 is the MFMA column.
+// Row i of the 4x4 product tile (its four coordinates in acc) folded into the four outputs
+// y00, y01, y10, y11 of the tile, then acc cleared:  A^T = [1 1 1 0; 0 1 -1 -1], column i =
+// (c0, c1); the products with 0 and +-1 are exact.
+__device__ __forceinline__ void rows_fold(floatx16 (&acc)[4], floatx16 (&yo)[4], int i) {
+    const float c0 = i < 3 ? 1.f : 0.f;
+    const float c1 = i == 0 ? 0.f : (i == 1 ? 1.f : -1.f);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float t0 = acc[0][r] + acc[1][r] + acc[2][r];
+        const float t1 = acc[1][r] - acc[2][r] - acc[3][r];
+        yo[0][r] = fmaf(c0, t0, yo[0][r]);
+        yo[1][r] = fmaf(c0, t1, yo[1][r]);
+        yo[2][r] = fmaf(c1, t0, yo[2][r]);
+        yo[3][r] = fmaf(c1, t1, yo[3][r]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
+    }
+}
+
+// Stores of a wave's 32x32 patch of output tiles: register r is MFMA row 8*(r/4) + 4*lh + r%4,
+// the lane's l32 the MFMA column.
 template <typename T, bool SWAP>
-__device__ __forceinline__ void winograd_epilogue(const floatx16 (&acc)[16], T* __restrict__ y, const ActStrides& ys,
-                                                  int N, int K, int Ho, int Wo, int th, int tw, long P, int order,
-                                                  int relu, int k0, long p0, int wm, int wn, int l32, int lh) {
+__device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restrict__ y, const ActStrides& ys, int N,
+                                           int K, int Ho, int Wo, int th, int tw, long P, int order, int relu, int k0,
+                                           long p0, int wm, int wn, int l32, int lh) {
     if (!SWAP) {
         const long p = p0 + wn * 32 + l32;
         if (p >= P) return;
@@ -327,12 +346,7 @@ __device__ __forceinline__ void winograd_epilogue(const floatx16 (&acc)[16], T* 
         for (int r = 0; r < 16; ++r) {
             const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
             if (k >= K) continue;
-            float m[16];
-#pragma unroll
-            for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
-            float y00, y01, y10, y11;
-            output_tile_transform(m, y00, y01, y10, y11);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
         }
     } else {
         const int k = k0 + wn * 32 + l32;
@@ -343,12 +357,7 @@ __device__ __forceinline__ void winograd_epilogue(const floatx16 (&acc)[16], T* 
             if (p >= P) continue;
             int n, ty, tx;
             decode_tile(p, order, N, th, tw, n, ty, tx);
-            float m[16];
-#pragma unroll
-            for (int xi = 0; xi < 16; ++xi) m[xi] = acc[xi][r];
-            float y00, y01, y10, y11;
-            output_tile_transform(m, y00, y01, y10, y11);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, y00, y01, y10, y11, relu);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
         }
     }
 }
@@ -459,46 +468,10 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
             iteration(par0_t{});
             iteration(par1_t{});
         }
-        // fold row i:  A^T = [1 1 1 0; 0 1 -1 -1], column i = (c0, c1); the products with 0 and +-1 are exact
-        const float c0 = i < 3 ? 1.f : 0.f;
-        const float c1 = i == 0 ? 0.f : (i == 1 ? 1.f : -1.f);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float t0 = acc[0][r] + acc[1][r] + acc[2][r];
-            const float t1 = acc[1][r] - acc[2][r] - acc[3][r];
-            yo[0][r] = fmaf(c0, t0, yo[0][r]);
-            yo[1][r] = fmaf(c0, t1, yo[1][r]);
-            yo[2][r] = fmaf(c1, t0, yo[2][r]);
-            yo[3][r] = fmaf(c1, t1, yo[3][r]);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
-        }
+        rows_fold(acc, yo, i);
     }
 
-    // ---- stores: register r is MFMA row 8*(r/4) + 4*lh + r%4, the lane's l32 the MFMA column ----
-    if (!SWAP) {
-        const long p = p0 + wn * 32 + l32;
-        if (p >= P) return;
-        int n, ty, tx;
-        decode_tile(p, order, N, th, tw, n, ty, tx);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (k >= K) continue;
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
-        }
-    } else {
-        const int k = k0 + wn * 32 + l32;
-        if (k >= K) return;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const long p = p0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (p >= P) continue;
-            int n, ty, tx;
-            decode_tile(p, order, N, th, tw, n, ty, tx);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
-        }
-    }
+    rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
 }
 
 }  // namespace wino

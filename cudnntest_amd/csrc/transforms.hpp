@@ -234,45 +234,59 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     const int nunits = rows << chunkLog2;
     const int cmask = (1 << chunkLog2) - 1;
     const int wbase = VEC == 2 ? (w0 & ~1) : w0;       // first loaded image column (even for VEC = 2)
-    struct alignas(sizeof(T) * VEC) Ld { T e[VEC]; };
-    for (int u0 = 0; u0 < nunits; u0 += 4 * MAXU) {
-        Ld buf[CV][MAXU];
+    // Every load is unconditional, from an address clamped into the image, and its bits are
+    // ANDed with an all-ones / zero mask afterwards (zero padding, channel padding, units past
+    // the halo): loads under a branch are waited for one by one.
+    typedef typename std::conditional<sizeof(T) * VEC == 4, uint32_t, uint16_t>::type raw_t;
+    typedef typename std::conditional<sizeof(T) == 4, uint32_t, uint16_t>::type elem_t;
+    elem_t* smem_bits = reinterpret_cast<elem_t*>(in_smem_raw);
+    auto copy_batch = [&](auto nb_c, int u0) {
+        constexpr int NB = decltype(nb_c)::value;
+        raw_t buf[CV][NB];
+        unsigned keep[NB];
 #pragma unroll
-        for (int i = 0; i < MAXU; ++i) {
+        for (int i = 0; i < NB; ++i) {
             const int u = u0 + wv + 4 * i;
             const int r = u >> chunkLog2;
             const int iw = wbase + (((u & cmask) << 6) + lane) * VEC;
             const int ih = h0 + r;
             // a pair is inside the image or outside it as a whole (W even, iw even)
             const bool ok = u < nunits && ih >= 0 && ih < H && iw >= 0 && iw < W;
+            keep[i] = ok ? 0xFFFFFFFFu : 0u;
+            const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - VEC);
 #pragma unroll
             for (int ch = 0; ch < CV; ++ch) {
-                const int c = cq * CV + ch;
-                if (ok && c < C) {
-                    buf[ch][i] = *reinterpret_cast<const Ld*>(x + (((size_t)n * C + c) * H + ih) * W + iw);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) buf[ch][i].e[e] = from_f32<T>(0.f);
-                }
+                const int c = min(cq * CV + ch, C - 1);
+                buf[ch][i] = *reinterpret_cast<const raw_t*>(x + (((size_t)n * C + c) * H + ihc) * W + iwc);
             }
         }
 #pragma unroll
-        for (int i = 0; i < MAXU; ++i) {
+        for (int i = 0; i < NB; ++i) {
             const int u = u0 + wv + 4 * i;
             const int r = u >> chunkLog2;
             const int q0 = wbase - w0 + (((u & cmask) << 6) + lane) * VEC;   // LDS column of the first element
             if (u < nunits) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const int q = q0 + e;
-                    if (q >= 0 && q < ldsW) {
+                for (int ch = 0; ch < CV; ++ch) {
+                    const unsigned m = cq * CV + ch < C ? keep[i] : 0u;
+                    const unsigned bits = __float_as_uint(mask_keep(__uint_as_float((unsigned)buf[ch][i]), m));
 #pragma unroll
-                        for (int ch = 0; ch < CV; ++ch) in_smem[ch * per_ch + r * ldsW + q] = buf[ch][i].e[e];
+                    for (int e = 0; e < VEC; ++e) {
+                        const int q = q0 + e;
+                        if (q >= 0 && q < ldsW)
+                            smem_bits[ch * per_ch + r * ldsW + q] = (elem_t)(bits >> (8 * sizeof(T) * e));
                     }
                 }
             }
         }
-    }
+    };
+    int u0 = 0;
+    for (; u0 + 4 * MAXU <= nunits; u0 += 4 * MAXU) copy_batch(std::integral_constant<int, MAXU>{}, u0);
+    // the remainder in the smallest batch that holds it: a unit past the halo still costs its loads
+    const int rem = nunits - u0;
+    if (rem > 16) copy_batch(std::integral_constant<int, MAXU>{}, u0);
+    else if (rem > 8) copy_batch(std::integral_constant<int, 4>{}, u0);
+    else if (rem > 0) copy_batch(std::integral_constant<int, 2>{}, u0);
     __syncthreads();
 
     const int tr = tid / TC, tc = tid % TC;

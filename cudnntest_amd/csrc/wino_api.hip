@@ -274,18 +274,18 @@ int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometr
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
-template <typename T, bool SWAP, bool LOC>
-int launch_fused_t(int src, int dst, int order, unsigned flags, const Geometry& g, const void* x, const void* U,
-                   void* y, hipStream_t st) {
+template <typename T, bool SWAP, int XM, int NVG>
+int launch_fused_rows_t(int src, int dst, int order, unsigned flags, const Geometry& g, const void* x, const void* U,
+                        void* y, hipStream_t st) {
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
-    hipLaunchKernelGGL((fused_conv_kernel<T, SWAP, LOC>), grid, block, 0, st, (const T*)x, (const T*)U, (T*)y,
+    hipLaunchKernelGGL((fused_rows_kernel<T, SWAP, XM, NVG>), grid, block, 0, st, (const T*)x, (const T*)U, (T*)y,
                        act_strides(src, g.N, g.C, g.H, g.W), act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.C, g.K,
                        g.H, g.W, g.pad, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, order,
                        (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
-    LAUNCH_CHECK("fused_conv");
+    LAUNCH_CHECK("fused_rows");
     return WINO_OK;
 }
 
@@ -294,11 +294,32 @@ int launch_fused_d(int src, int dst, int order, unsigned flags, const Geometry& 
                    void* y, hipStream_t st) {
     if ((long)g.N * g.C * g.H * g.W >= (1L << 31))
         return fail(WINO_ERR_UNSUPPORTED, "fused kernel: input tensor too large for 32-bit element offsets");
-    const bool swap = dst == WINO_NHWC, loc = src == WINO_NHWC;
-    if (swap && loc) return launch_fused_t<T, true, true>(src, dst, order, flags, g, x, U, y, st);
-    if (swap) return launch_fused_t<T, true, false>(src, dst, order, flags, g, x, U, y, st);
-    if (loc) return launch_fused_t<T, false, true>(src, dst, order, flags, g, x, U, y, st);
-    return launch_fused_t<T, false, false>(src, dst, order, flags, g, x, U, y, st);
+    constexpr int CV = ChanVec<T>::n;
+    const bool swap = dst == WINO_NHWC, chan_contig = src == WINO_NHWC;
+    // two k-groups per stage when Cp allows an even stage count; a 2-byte source without
+    // channel-vector loads would then hold 64 raw values per thread (spills): one k-group there
+    bool two = (g.Cp / CV) % 8 == 0;
+    if (sizeof(T) == 2 && !(chan_contig && g.C % CV == 0)) two = false;
+    const int un = (two ? 2 : 1) * CV / 2;     // channels per thread
+    const int xm = (chan_contig && g.C % un == 0) ? XM_CHANVEC : ((src == WINO_NCHW && g.W >= 4) ? XM_ROW : XM_SCALAR);
+#define FR(SW, XM, NG) return launch_fused_rows_t<T, SW, XM, NG>(src, dst, order, flags, g, x, U, y, st)
+#define FR2(SW, NG)                               \
+    if (xm == XM_CHANVEC) FR(SW, XM_CHANVEC, NG); \
+    if (xm == XM_ROW) FR(SW, XM_ROW, NG);         \
+    FR(SW, XM_SCALAR, NG)
+    if (two) {
+        if constexpr (sizeof(T) == 2) {        // here two implies channel-vector loads
+            if (swap) FR(true, XM_CHANVEC, 2);
+            FR(false, XM_CHANVEC, 2);
+        } else {
+            if (swap) { FR2(true, 2); }
+            FR2(false, 2);
+        }
+    }
+    if (swap) { FR2(true, 1); }
+    FR2(false, 1);
+#undef FR2
+#undef FR
 }
 
 int launch_fused(int src, int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* x,
@@ -368,15 +389,24 @@ int tile_order_for(int src, int /*dst*/) {
 
 // Measured on MI355X over the VGG-16 layer shapes: the fewer the channels, the more
 // the transformed tensors cost relative to the multiplies, and the more fusion pays.
-int pick_algo(int dtype, const Geometry& g) {
+// Chosen from sweeps of the VGG-16 shapes over the three algorithms, per layout and element type.
+int pick_algo(int layout, int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
     if (patches < 512) return WINO_ALGO_STAGED;          // too few 64x64 patches to fill 256 CUs
+    const bool nhwc = layout == WINO_NHWC;
     if (dtype == WINO_F32) {
-        if (g.C >= 16 && g.C <= 64 && g.K <= 64) return WINO_ALGO_FUSED;   // conv1_2: V would be 4x the input
-        if (g.C <= 128) return WINO_ALGO_EPILOGUE;
-        return WINO_ALGO_STAGED;      // C >= 256: the 128x128 GEMM's lower L2 traffic per flop wins (tie at 256)
+        // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
+        if (g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
+        if (g.C <= 256 && g.K <= 256) return nhwc ? WINO_ALGO_FUSED : WINO_ALGO_EPILOGUE;
+        return WINO_ALGO_STAGED;      // the 128x128 GEMM's lower L2 traffic per flop wins
     }
-    return WINO_ALGO_EPILOGUE;   // 16-bit operands: the fp32 product tensor is the largest HBM stream, drop it
+    // 16-bit operands: the fp32 product tensor is the largest HBM stream, so never STAGED; the in-kernel
+    // input transform is VALU work repeated per filter tile and pays only with few filter tiles and
+    // cheap loads (channel vectors for NHWC, coalesced elements for CHWN)
+    if (nhwc && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
+    if (layout == WINO_CHWN && g.C <= 64 && g.K <= 64) return WINO_ALGO_FUSED;
+    if (g.C < 16) return WINO_ALGO_FUSED;
+    return WINO_ALGO_EPILOGUE;
 }
 
 int conv_f4_impl(int src, int dst, int dtype, unsigned flags, int N, int C, int K, int H, int W, int pad,
@@ -425,7 +455,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
-    if (algo == WINO_ALGO_AUTO) algo = pick_algo(dtype, g);
+    if (algo == WINO_ALGO_AUTO) algo = pick_algo(src, dtype, g);
     if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(src, dst, dtype, flags, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
     hipStream_t st = (hipStream_t)stream;
@@ -487,12 +517,13 @@ int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, in
     return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, y, stream);
 }
 
-int wino_pick_algo(int dtype, int N, int C, int K, int H, int W, int pad) {
+int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int pad) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
-    return pick_algo(dtype, g);
+    return pick_algo(layout, dtype, g);
 }
 
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp, int* Kp,

@@ -85,9 +85,9 @@ ALGO_NAMES = {ALGO_AUTO: "auto", ALGO_STAGED: "staged", ALGO_EPILOGUE: "epilogue
               ALGO_STAGED_F4: "staged_f4"}
 
 
-def pick_algo(dtype, N, C, K, H, W, pad=1):
-    """The algorithm ALGO_AUTO resolves to for this problem."""
-    rc = _lib.load().wino_pick_algo(dtype, N, C, K, H, W, pad)
+def pick_algo(layout, dtype, N, C, K, H, W, pad=1):
+    """The algorithm ALGO_AUTO resolves to for this problem (layout: that of the input tensor)."""
+    rc = _lib.load().wino_pick_algo(layout, dtype, N, C, K, H, W, pad)
     if rc < 0:
         _lib.check(rc, "wino_pick_algo")
     return rc

@@ -86,8 +86,9 @@ int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
 int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K,
                        int H, int W, int pad, const void *x, const void *U, void *y, void *stream);
 
-/* the algorithm WINO_ALGO_AUTO resolves to for this problem (a wino_algo_t), or a negative status */
-int wino_pick_algo(int dtype, int N, int C, int K, int H, int W, int pad);
+/* the algorithm WINO_ALGO_AUTO resolves to for this problem (a wino_algo_t), or a negative status;
+ * layout is that of the input tensor */
+int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int pad);
 
 /* ---- padded operand geometry ------------------------------------------------
  * With th = ceil(Ho/2), tw = ceil(Wo/2), P = N*th*tw and CV = 16/sizeof(element)

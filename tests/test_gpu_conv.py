@@ -17,7 +17,9 @@ pytestmark = pytest.mark.gpu
 LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
 ALGOS = [ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED]
 
-SMALL = [(2, 3, 4, 5, 5), (1, 8, 8, 6, 6), (3, 5, 7, 9, 9), (2, 16, 130, 7, 10), (1, 1, 1, 3, 3), (5, 40, 24, 14, 14)]
+SMALL = [(2, 3, 4, 5, 5), (1, 8, 8, 6, 6), (3, 5, 7, 9, 9), (2, 16, 130, 7, 10), (1, 1, 1, 3, 3), (5, 40, 24, 14, 14),
+         # channel counts that take two k-groups per stage in the single-kernel path; odd and minimal widths
+         (2, 32, 20, 11, 13), (1, 64, 70, 8, 4), (3, 36, 9, 6, 7)]
 
 
 @pytest.mark.parametrize("algo", ALGOS)
