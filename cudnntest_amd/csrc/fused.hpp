@@ -22,9 +22,11 @@ namespace wino {
 // Row i of V = B^T d B needs only two rows of the raw patch:
 //     (B^T d)_i = d_ra + sg * d_rb,   (ra, rb, sg) = (0,2,-), (1,2,+), (2,1,-), (1,3,-)
 // followed by the column transform.  Per stage (NC = NV*CV channels of one row) a
-// thread owns one tile and UN = NC/4 consecutive channels, loads 2 x 4 raw values
-// per channel one stage ahead, and writes the four coordinates as one UN-element
-// chunk each.  The raw input is read four times in total (once per row), from
+// thread owns one tile and UN = NC/4 consecutive channels, requests their 2 x 4 raw
+// values at the start of the stage before, transforms them during that stage's last
+// MFMA runs, and writes the four coordinates as one UN-element chunk each.  (Register
+// loads that stay in flight across a wait on direct-to-LDS loads gain nothing: while
+// such a load is pending the compiler turns every vmcnt wait into vmcnt(0).)  The raw input is read four times in total (once per row), from
 // L2 after the first.
 //
 // How a thread reads its 2 x 4 x UN raw values (the load path, not HBM, bounds this kernel):
@@ -60,10 +62,6 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     constexpr int NC = NV * CV;                // channels per stage
     constexpr int UN = NC / 4;                 // channels per thread (64 tiles x NC channels over 256 threads)
     static_assert(CV % UN == 0, "a thread's channels must lie inside one channel vector");
-    constexpr int XL = XM == XM_CHANVEC ? 8 : (XM == XM_ROW ? 2 * UN : 8 * UN);   // x loads per thread and stage
-    // s_waitcnt vmcnt(VM) lgkmcnt(0): the filter rows (issued before the x loads) have landed
-    constexpr int VM = XL < 63 ? XL : 63;      // 6-bit field
-    constexpr int WAIT_IMM = (VM & 0xF) | (0x7 << 4) | (0 << 8) | ((VM >> 4) << 14);
     typedef typename std::conditional<UN * sizeof(T) == 16, uint4, uint2>::type chunk_t;   // UN channels
     static_assert(sizeof(chunk_t) == UN * sizeof(T), "chunk size");
     constexpr int VPAD = XM == XM_CHANVEC ? 2 : 0;   // V rows padded where lanes walk channel vectors first
@@ -71,9 +69,12 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     __shared__ vec Vs0[4][NV][GO_T + VPAD], Vs1[4][NV][GO_T + VPAD];
 
     const int b = blockIdx.x;
+    // Workgroup ids go round-robin to the 8 XCDs.  The ids of one XCD walk the filter tiles of a
+    // tile patch first (they share its raw input), then CONSECUTIVE tile patches: neighbouring
+    // patches are neighbouring tile rows, whose raw input rows overlap, and an XCD has its own L2.
     const int xcd = b & 7, jb = b >> 3;
     const int ktile = jb % kTiles;
-    const int ptile = (jb / kTiles) * 8 + xcd;
+    const int ptile = xcd * ((pTiles + 7) / 8) + jb / kTiles;
     if (ptile >= pTiles) return;
     const int k0 = ktile * GO_T;
     const long p0 = (long)ptile * GO_T;
@@ -82,7 +83,8 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     const vec* Ug = reinterpret_cast<const vec*>(U);
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
@@ -128,11 +130,10 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     typedef std::integral_constant<int, 0> par0_t;
     typedef std::integral_constant<int, 1> par1_t;
 
-    // ---- raw rows ra, rb of the patch, requested one stage ahead ----------------------------
+    // ---- raw rows ra, rb of the patch for the next stage -----------------------------------
     // x_prep fixes the stage to request (offsets, masks, sign); x_load_unit / x_load_all issue the
     // loads; v_unit turns the staged values of one channel into row i of B^T d B; v_write stores
-    // the four coordinates into stage S of V.  The masks and sign of the staged values (`c` set)
-    // are those x_prep computed one iteration earlier (`n` set).
+    // the four coordinates into stage S of V.
     T xa[4][UN], xb[4][UN];                    // [column][channel]; XM_ROW: [element of the quadruple][channel]
     unsigned ma_c = 0, mb_c = 0, cok_c = 0;    // all ones when patch row ra / rb lies inside the image; bit u: channel u is real
     float sg_c = 0.f;
@@ -229,13 +230,18 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     auto v_piece = [&](auto par, int piece) {
         if (piece < WP) {
 #pragma unroll
-            for (int u = piece * UPP; u < (piece + 1) * UPP && u < UN; ++u) {
-                v_unit(u);
-                if (XM != XM_CHANVEC) x_load_unit(u);
-            }
+            for (int u = piece * UPP; u < (piece + 1) * UPP && u < UN; ++u) v_unit(u);
         } else if (piece == WP) {
             v_write(par);
-            if (XM == XM_CHANVEC) x_load_all();
+        }
+    };
+    auto x_load_stage = [&](int row_i, int st) {
+        x_prep(row_i, st);
+        take_next();
+        if (XM == XM_CHANVEC) x_load_all();
+        else {
+#pragma unroll
+            for (int u = 0; u < UN; ++u) x_load_unit(u);
         }
     };
     // ---- the filter rows of a stage: 4*NV rows of 64 vectors, wave w issues rows w, w+4, ... --
@@ -265,40 +271,34 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
             fu[r & 1] = S ? Us1[j][v][(SWAP ? wn : wm) * 32 + l32] : Us0[j][v][(SWAP ? wn : wm) * 32 + l32];
             fv[r & 1] = S ? Vs1[j][v][(SWAP ? wm : wn) * 32 + l32] : Vs0[j][v][(SWAP ? wm : wn) * 32 + l32];
         };
+        // the next stage: filter rows and raw patch rows requested first, multiplied stage in between,
+        // the raw rows transformed and written during the last MFMA runs
         u_load(other_t{}, ni, nstg);
-        take_next();
+        x_load_stage(ni, nstg);
         advance();
-        x_prep(ni, nstg);
         frag_load(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             if (r + 1 < NR) frag_load(r + 1);
-            v_piece(other_t{}, r);
+            if (r >= NR - 1 - WP) v_piece(other_t{}, r - (NR - 1 - WP));
             if (SWAP) Mma<T>::run(fv[r & 1], fu[r & 1], acc[r & 3]);
             else Mma<T>::run(fu[r & 1], fv[r & 1], acc[r & 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+        __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0) lgkmcnt(0)
         __syncthreads();
     };
 
-    // prologue: stage (0, 0) of both operands in LDS, the raw rows of the stage after it in flight
-    x_prep(0, 0);
-    if (XM == XM_CHANVEC) x_load_all();
-    else {
-#pragma unroll
-        for (int u = 0; u < UN; ++u) x_load_unit(u);
-    }
+    // prologue: stage (0, 0) of both operands in LDS
+    x_load_stage(0, 0);
     u_load(par0_t{}, 0, 0);
-    take_next();
     advance();
-    x_prep(ni, nstg);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int piece = 0; piece <= WP; ++piece) v_piece(par0_t{}, piece);
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+    __builtin_amdgcn_s_waitcnt(0x0070);
     __syncthreads();
 
     for (int i = 0; i < 4; ++i) {

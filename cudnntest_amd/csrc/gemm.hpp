@@ -89,7 +89,8 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
     const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
@@ -206,7 +207,8 @@ __global__ __launch_bounds__(256) void gemm_128x128_reg_kernel(const T* __restri
     const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
     const int lrow = tid >> 7, lcol = tid & 127;   // rows lrow + 2*h
@@ -406,7 +408,8 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     const vec* Vg = reinterpret_cast<const vec*>(V);
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
@@ -473,5 +476,6 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
 
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
 }
+
 
 }  // namespace wino

@@ -229,7 +229,8 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     // units w, w+4, ...  Loads are issued in batches of CV x MAXU before any of
     // them is written to LDS, so a wave keeps that many HBM requests in flight.
     // With VEC = 2 a lane loads the image-aligned pair (iw, iw+1), iw even.
-    const int lane = tid & 63, wv = tid >> 6;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);     // wave-uniform: keeps the unit arithmetic on the scalar unit
     constexpr int MAXU = 6;
     const int nunits = rows << chunkLog2;
     const int cmask = (1 << chunkLog2) - 1;
@@ -246,12 +247,12 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
         unsigned keep[NB];
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
-            const int u = u0 + wv + 4 * i;
+            const int u = min(u0 + wv + 4 * i, nunits - 1);   // a unit past the halo repeats the last one (not stored)
             const int r = u >> chunkLog2;
             const int iw = wbase + (((u & cmask) << 6) + lane) * VEC;
             const int ih = h0 + r;
             // a pair is inside the image or outside it as a whole (W even, iw even)
-            const bool ok = u < nunits && ih >= 0 && ih < H && iw >= 0 && iw < W;
+            const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
             keep[i] = ok ? 0xFFFFFFFFu : 0u;
             const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - VEC);
 #pragma unroll

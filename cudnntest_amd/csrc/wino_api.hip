@@ -253,9 +253,9 @@ int launch_gemm_rows_t(int order, unsigned flags, const Geometry& g, const void*
 template <typename T>
 int launch_gemm_rows_d(int dst, int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y,
                        hipStream_t st) {
+    constexpr int CV = ChanVec<T>::n;
     // stages per row must be even: one k-group per stage always is (Cp is a multiple of 4 channel
     // vectors); two k-groups per stage (fewer barriers, measured faster) when Cp allows it
-    constexpr int CV = ChanVec<T>::n;
     const bool two = (g.Cp / CV) % 8 == 0;
     if (dst == WINO_NHWC)
         return two ? launch_gemm_rows_t<T, true, 2>(order, flags, g, U, V, y, dst, st)
@@ -402,10 +402,14 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     }
     // 16-bit operands: the fp32 product tensor is the largest HBM stream, so never STAGED; the in-kernel
     // input transform is VALU work repeated per filter tile and pays only with few filter tiles and
-    // cheap loads (channel vectors for NHWC, coalesced elements for CHWN)
-    if (nhwc && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
-    if (layout == WINO_CHWN && g.C <= 64 && g.K <= 64) return WINO_ALGO_FUSED;
-    if (g.C < 16) return WINO_ALGO_FUSED;
+    // cheap loads (channel vectors for NHWC, which need C % 8 == 0; coalesced elements for CHWN)
+    if (nhwc) {
+        if (g.C >= 16 && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
+    } else if (layout == WINO_CHWN) {
+        if (g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
+    } else if (g.C <= 64 && g.K <= 64) {
+        return WINO_ALGO_FUSED;
+    }
     return WINO_ALGO_EPILOGUE;
 }
 
