@@ -103,15 +103,22 @@ __global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restri
                 for (int e = 0; e < CV; ++e) g[e][r][q] = to_f32(pk.e[e]);
             }
     } else {
+        // any strides ([C][3][3][K]: lanes along k read contiguously).  All 9*CV loads are issued
+        // from clamped addresses before the first use and masked afterwards: a load under a branch
+        // is waited for on its own, and this kernel is all latency.
+        T raw[CV][9];
 #pragma unroll
         for (int e = 0; e < CV; ++e) {
             const int c = cq * CV + e;
-            const bool ok = k < K && c < C;
-            const T* wp = w + (ok ? k : 0) * s.k + (ok ? c : 0) * s.c;
+            const T* wp = w + (k < K ? k : K - 1) * s.k + (c < C ? c : C - 1) * s.c;
 #pragma unroll
-            for (int r = 0; r < 3; ++r)
+            for (int t = 0; t < 9; ++t) raw[e][t] = wp[(t / 3) * s.r + (t % 3) * s.s];
+        }
 #pragma unroll
-                for (int q = 0; q < 3; ++q) g[e][r][q] = ok ? to_f32(wp[r * s.r + q * s.s]) : 0.f;
+        for (int e = 0; e < CV; ++e) {
+            const unsigned m = (k < K && cq * CV + e < C) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) g[e][t / 3][t % 3] = mask_keep(to_f32(raw[e][t]), m);
         }
     }
 #pragma unroll
