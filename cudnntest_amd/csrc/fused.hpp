@@ -245,16 +245,27 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
         }
     };
     // ---- the filter rows of a stage: 4*NV rows of 64 vectors, wave w issues rows w, w+4, ... --
+    // one running scalar address per row slot, as in gemm_rows_kernel; u_load requests the stage
+    // (ni, nstg) and moves the addresses to the one after it
+    const unsigned lane_off = lane * 16;
+    uint64_t uptr[NV];
+    const uint64_t stepU = (uint64_t)NV * Kp * 16, wrapU = (uint64_t)(NV + 3 * CQ) * Kp * 16;
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int r = wave + 4 * q;
+        const int j = r / NV, v = r % NV;
+        uptr[q] = reinterpret_cast<uint64_t>(Ug + ((size_t)j * CQ + v) * Kp + k0);
+    }
     auto u_load = [&](auto par, int row_i, int st) {
         constexpr int S = decltype(par)::value;
+        const bool last = row_i == 3 && st == nst - 1;               // the clamped stage past the end repeats it
+        const uint64_t inc = last ? 0 : (st == nst - 1 ? wrapU : stepU);
 #pragma unroll
         for (int q = 0; q < NV; ++q) {
             const int r = wave + 4 * q;
             const int j = r / NV, v = r % NV;
-            const vec* src = Ug + ((size_t)(4 * row_i + j) * CQ + (size_t)st * NV + v) * Kp + k0 + lane;
-            vec* dst = S ? &Us1[j][v][0] : &Us0[j][v][0];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+            dma_row(uptr[q], lane_off, S ? &Us1[j][v][0] : &Us0[j][v][0]);
+            uptr[q] += inc;
         }
     };
     int ni = 0, nstg = 0;                      // (row, stage) after the one being multiplied
@@ -306,7 +317,7 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
             iteration(par0_t{});
             iteration(par1_t{});
         }
-        rows_fold(acc, yo, i);
+        rows_fold<true>(acc, yo, i);
     }
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
 }

@@ -48,6 +48,17 @@ template <> struct Mma<bf16_t> {
     }
 };
 
+// One direct-to-LDS load of 64 channel vectors (1 KB): lane l moves the 16 bytes at sbase + 16*l to
+// lds_dst + 16*l.  sbase is wave-uniform (a scalar register pair, advanced with scalar adds): at
+// 16-bit MFMA rates the address arithmetic of these loads, vector or scalar, costs as much as the
+// multiplies of a stage, so the kernels keep one running address per load slot instead of
+// recomputing row * pitch products.
+__device__ __forceinline__ void dma_row(uint64_t sbase, unsigned lane_off, void* lds_dst) {
+    const char* src = reinterpret_cast<const char*>(sbase) + lane_off;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+}
+
 // =============================================================================
 // Plain batched GEMM, product written to HBM as Mo[xi][Kp][Pp] (fp32).
 //
@@ -296,16 +307,30 @@ __global__ __launch_bounds__(256) void gemm_128x128_reg_kernel(const T* __restri
 // =============================================================================
 constexpr int GO_T = 64;   // patch edge (filters and tiles)
 
+// The 2x2 outputs of tile (n, ty, tx), filter k.  pair: the destination is W-contiguous with even
+// rows and an aligned base (checked once per kernel by pair_stores_ok), so the two outputs of a tile row
+// go out as one store.
+template <typename OutT> __device__ __forceinline__ bool pair_stores_ok(const OutT* y, const ActStrides& ys, int Wo) {
+    return ys.w == 1 && (Wo & 1) == 0 && (ys.h & 1) == 0 && (ys.c & 1) == 0 && (ys.n & 1) == 0 &&
+           (reinterpret_cast<uintptr_t>(y) & (2 * sizeof(OutT) - 1)) == 0;
+}
+
 template <typename OutT>
 __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const ActStrides& ys, int n, int k, int ty,
                                                    int tx, int Ho, int Wo, float y00, float y01, float y10, float y11,
-                                                   int relu) {
+                                                   int relu, bool pair) {
     if (relu) {
         y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f);
     }
     const int oh = 2 * ty, ow = 2 * tx;
     OutT* yp = y + n * ys.n + k * ys.c + oh * ys.h + ow * ys.w;
     const bool w1 = ow + 1 < Wo, h1 = oh + 1 < Ho;
+    if (pair) {
+        struct alignas(2 * sizeof(OutT)) Pair { OutT a, b; };
+        *reinterpret_cast<Pair*>(yp) = Pair{from_f32<OutT>(y00), from_f32<OutT>(y01)};
+        if (h1) *reinterpret_cast<Pair*>(yp + ys.h) = Pair{from_f32<OutT>(y10), from_f32<OutT>(y11)};
+        return;
+    }
     yp[0] = from_f32<OutT>(y00);
     if (w1) yp[ys.w] = from_f32<OutT>(y01);
     if (h1) {
@@ -315,9 +340,9 @@ __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const A
 }
 
 // Row i of the 4x4 product tile (its four coordinates in acc) folded into the four outputs
-// y00, y01, y10, y11 of the tile, then acc cleared:  A^T = [1 1 1 0; 0 1 -1 -1], column i =
+// y00, y01, y10, y11 of the tile, then acc cleared if CLEAR:  A^T = [1 1 1 0; 0 1 -1 -1], column i =
 // (c0, c1); the products with 0 and +-1 are exact.
-__device__ __forceinline__ void rows_fold(floatx16 (&acc)[4], floatx16 (&yo)[4], int i) {
+template <bool CLEAR> __device__ __forceinline__ void rows_fold(floatx16 (&acc)[4], floatx16 (&yo)[4], int i) {
     const float c0 = i < 3 ? 1.f : 0.f;
     const float c1 = i == 0 ? 0.f : (i == 1 ? 1.f : -1.f);
 #pragma unroll
@@ -328,8 +353,10 @@ __device__ __forceinline__ void rows_fold(floatx16 (&acc)[4], floatx16 (&yo)[4],
         yo[1][r] = fmaf(c0, t1, yo[1][r]);
         yo[2][r] = fmaf(c1, t0, yo[2][r]);
         yo[3][r] = fmaf(c1, t1, yo[3][r]);
+        if (CLEAR) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
+            for (int j = 0; j < 4; ++j) acc[j][r] = 0.f;
+        }
     }
 }
 
@@ -339,6 +366,7 @@ template <typename T, bool SWAP>
 __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restrict__ y, const ActStrides& ys, int N,
                                            int K, int Ho, int Wo, int th, int tw, long P, int order, int relu, int k0,
                                            long p0, int wm, int wn, int l32, int lh) {
+    const bool pair = pair_stores_ok(y, ys, Wo);
     if (!SWAP) {
         const long p = p0 + wn * 32 + l32;
         if (p >= P) return;
@@ -348,7 +376,7 @@ __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restric
         for (int r = 0; r < 16; ++r) {
             const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
             if (k >= K) continue;
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu, pair);
         }
     } else {
         const int k = k0 + wn * 32 + l32;
@@ -359,7 +387,7 @@ __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restric
             if (p >= P) continue;
             int n, ty, tx;
             decode_tile(p, order, N, th, tw, n, ty, tx);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu, pair);
         }
     }
 }
@@ -423,29 +451,44 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     typedef std::integral_constant<int, 0> par0_t;
     typedef std::integral_constant<int, 1> par1_t;
     // a stage is 8*NV rows of 64 vectors (4 coordinates x NV vectors, U and V); wave w issues rows w, w+4, ...
-    auto stage_load = [&](auto par, int row_i, int st) {
+    // Row r of a stage is (operand, coordinate j of the row, vector v); its address advances by NV
+    // vectors per stage and by NV + 3*CQ vectors when the Winograd row changes.
+    const unsigned lane_off = lane * 16;
+    uint64_t sptr[2 * NV];
+    const uint64_t stepU = (uint64_t)NV * Kp * 16, wrapU = (uint64_t)(NV + 3 * CQ) * Kp * 16;
+    const uint64_t stepV = (uint64_t)NV * Pp * 16, wrapV = (uint64_t)(NV + 3 * CQ) * Pp * 16;
+#pragma unroll
+    for (int q = 0; q < 2 * NV; ++q) {
+        const int r = wave + 4 * q;                  // 0 .. 8*NV-1, wave-uniform
+        const int opnd = q / NV;                     // 0: U, 1: V  (= r / (4*NV), known at compile time)
+        const int j = (r / NV) & 3, v = r % NV;
+        const size_t cvec = (size_t)j * CQ + v;
+        sptr[q] = opnd ? reinterpret_cast<uint64_t>(Vg + cvec * Pp + p0) : reinterpret_cast<uint64_t>(Ug + cvec * Kp + k0);
+    }
+    const int total = 4 * nst;
+    int issued = 0, in_row = 0;                      // stages requested so far, and of the current row
+    auto stage_load = [&](auto par) {
         constexpr int S = decltype(par)::value;
+        ++issued;
+        const bool wrap = ++in_row == nst, last = issued >= total;   // past the end: the last stage again (never read)
+        if (wrap) in_row = 0;
+        const uint64_t incU = last ? 0 : (wrap ? wrapU : stepU), incV = last ? 0 : (wrap ? wrapV : stepV);
 #pragma unroll
         for (int q = 0; q < 2 * NV; ++q) {
-            const int r = wave + 4 * q;              // 0 .. 8*NV-1, wave-uniform
-            const int opnd = r / (4 * NV);           // 0: U, 1: V
+            const int r = wave + 4 * q;
+            const int opnd = q / NV;
             const int j = (r / NV) & 3, v = r % NV;
-            const size_t cvec = (size_t)(4 * row_i + j) * CQ + (size_t)st * NV + v;
-            const vec* src = opnd ? Vg + cvec * Pp + p0 + lane : Ug + cvec * Kp + k0 + lane;
             vec* dst = opnd ? (S ? &Vs1[j][v][0] : &Vs0[j][v][0]) : (S ? &Us1[j][v][0] : &Us0[j][v][0]);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+            dma_row(sptr[q], lane_off, dst);
+            sptr[q] += opnd ? incV : incU;
         }
     };
-    int ni = 0, nstg = 0;                            // (row, stage) of the next stage to request
-    auto advance = [&]() {
-        if (++nstg == nst) { nstg = 0; ++ni; }
-        if (ni > 3) { ni = 3; nstg = nst - 1; }      // past the end: re-request the last stage (never read)
-    };
-    auto iteration = [&](auto par) {
+    // first: the stage opens a row, its MFMAs start from a zero accumulator (an inline constant,
+    // instead of 64 register clears per row)
+    auto iteration = [&](auto par, auto first) {
         constexpr int S = decltype(par)::value;
-        stage_load(std::integral_constant<int, 1 - S>{}, ni, nstg);
-        advance();
+        constexpr bool FIRST = decltype(first)::value;
+        stage_load(std::integral_constant<int, 1 - S>{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < NVG; ++g)
@@ -453,6 +496,10 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
             for (int j = 0; j < 4; ++j) {
                 const vec fu = S ? Us1[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32] : Us0[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32];
                 const vec fv = S ? Vs1[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32] : Vs0[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32];
+                if (FIRST && g == 0) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+                }
                 if (SWAP) Mma<T>::run(fv, fu, acc[j]);
                 else Mma<T>::run(fu, fv, acc[j]);
             }
@@ -461,17 +508,18 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         __syncthreads();
     };
 
-    stage_load(par0_t{}, 0, 0);
-    advance();
+    stage_load(par0_t{});
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
     for (int i = 0; i < 4; ++i) {
-        for (int st = 0; st < nst; st += 2) {
-            iteration(par0_t{});
-            iteration(par1_t{});
+        iteration(par0_t{}, std::true_type{});
+        iteration(par1_t{}, std::false_type{});
+        for (int st = 2; st < nst; st += 2) {
+            iteration(par0_t{}, std::false_type{});
+            iteration(par1_t{}, std::false_type{});
         }
-        rows_fold(acc, yo, i);
+        rows_fold<false>(acc, yo, i);
     }
 
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);

@@ -323,73 +323,96 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
 
 // ---- input transform, NHWC source, LDS-transposed ---------------------------------------
 // Reads run along C (contiguous in NHWC), stores along p, so the block
-// transposes through LDS.  A workgroup takes one (n, ty), TC consecutive tx and
-// NQ channel vectors: phase 1 copies the 4 x (2*TC+2) pixel halo, 16 bytes per
-// (pixel, cq) with cq fastest across lanes; phase 2 gives thread (tile, cq) its
-// 16 pixels as 16-byte LDS reads (even/odd columns kept apart so lanes walking
-// tx read consecutive vectors) and stores 16 coalesced vectors of V.
-template <typename T, int TC, int NQ>
+// transposes through LDS.  A workgroup takes one image, TR tile rows, TC
+// consecutive tx and NQ channel vectors (C % CV == 0, checked by the host):
+// phase 1 copies the (2*TR+2) x (2*TC+2) pixel halo, 16 bytes per (pixel, cq)
+// with cq fastest across lanes, all loads of a thread issued from clamped
+// addresses before the first LDS write and masked afterwards (zero padding,
+// channel padding); phase 2 gives thread (tile column, cq) its TR tiles one
+// after the other, 16 pixels each as 16-byte LDS reads (even/odd columns kept
+// apart so lanes walking tx read consecutive vectors), and stores 16 coalesced
+// vectors of V per tile.
+template <typename T, int TC, int NQ, int TR>
 __global__ __launch_bounds__(TC * NQ) void input_transform_nhwc_kernel(const T* __restrict__ x, T* __restrict__ V,
                                                                        int N, int C, int H, int W, int pad, int th,
-                                                                       int tw, long Pp, int Cp, int colBlocks) {
+                                                                       int tw, long Pp, int Cp, int colBlocks,
+                                                                       int rowBlocks) {
     constexpr int CV = ChanVec<T>::n;
     constexpr int HALF = TC + 1;                       // columns of one parity
-    __shared__ Pack16<T> sm[NQ][4][2][HALF];           // [cq][row][col parity][col/2]
+    constexpr int ROWS = 2 * TR + 2, COLS = 2 * TC + 2;
+    constexpr int NT = TC * NQ;
+    constexpr int UNITS = ROWS * COLS * NQ;            // 16-byte vectors in the halo
+    constexpr int NLOAD = (UNITS + NT - 1) / NT;
+    __shared__ uint4 sm[NQ][ROWS][2][HALF];            // [cq][row][col parity][col/2]
+    static_assert(sizeof(Pack16<T>) == sizeof(uint4), "vector size");
     const int cq0 = blockIdx.y * NQ;
     const int cb = blockIdx.x % colBlocks, rowid = blockIdx.x / colBlocks;
-    const int ty = rowid % th, n = rowid / th;
-    const int tx0 = cb * TC;
-    const int h0 = 2 * ty - pad, w0 = 2 * tx0 - pad;
+    const int rb = rowid % rowBlocks, n = rowid / rowBlocks;
+    const int ty0 = rb * TR, tx0 = cb * TC;
+    const int h0 = 2 * ty0 - pad, w0 = 2 * tx0 - pad;
     const int tid = threadIdx.x;
-    const int CQ = Cp / CV;
+    const int CQ = Cp / CV, CQreal = C / CV;
 
-    constexpr int COLS = 2 * TC + 2;
-    for (int e = tid; e < 4 * COLS * NQ; e += TC * NQ) {
-        const int q = e % NQ, col = (e / NQ) % COLS, r = e / (NQ * COLS);
-        const int ih = h0 + r, iw = w0 + col, cq = cq0 + q;
-        Pack16<T> v;
+    {
+        uint4 buf[NLOAD];
+        unsigned keep[NLOAD];
 #pragma unroll
-        for (int i = 0; i < CV; ++i) v.e[i] = from_f32<T>(0.f);
-        if (ih >= 0 && ih < H && iw >= 0 && iw < W && cq < CQ) {
-            const T* src = x + (((size_t)n * H + ih) * W + iw) * C + cq * CV;
-            if ((cq + 1) * CV <= C && (C % CV) == 0) {
-                v = *reinterpret_cast<const Pack16<T>*>(src);
-            } else {
+        for (int i = 0; i < NLOAD; ++i) {
+            const int e = min(tid + i * NT, UNITS - 1);      // a unit past the halo repeats the last one (not stored)
+            const int q = e % NQ, col = (e / NQ) % COLS, r = e / (NQ * COLS);
+            const int ih = h0 + r, iw = w0 + col, cq = cq0 + q;
+            keep[i] = (ih >= 0 && ih < H && iw >= 0 && iw < W && cq < CQreal) ? 0xFFFFFFFFu : 0u;
+            const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - 1), cqc = min(cq, CQreal - 1);
+            buf[i] = *reinterpret_cast<const uint4*>(x + (((size_t)n * H + ihc) * W + iwc) * C + cqc * CV);
+        }
 #pragma unroll
-                for (int i = 0; i < CV; ++i)
-                    if (cq * CV + i < C) v.e[i] = src[i];
+        for (int i = 0; i < NLOAD; ++i) {
+            const int e = tid + i * NT;
+            if (e < UNITS) {
+                const int q = e % NQ, col = (e / NQ) % COLS, r = e / (NQ * COLS);
+                uint4 v;
+                v.x = __float_as_uint(mask_keep(__uint_as_float(buf[i].x), keep[i]));
+                v.y = __float_as_uint(mask_keep(__uint_as_float(buf[i].y), keep[i]));
+                v.z = __float_as_uint(mask_keep(__uint_as_float(buf[i].z), keep[i]));
+                v.w = __float_as_uint(mask_keep(__uint_as_float(buf[i].w), keep[i]));
+                sm[q][r][col & 1][col >> 1] = v;
             }
         }
-        sm[q][r][col & 1][col >> 1] = v;
     }
     __syncthreads();
 
     const int tc = tid % TC, q = tid / TC;
     const int tx = tx0 + tc, cq = cq0 + q;
     if (tx >= tw || cq >= CQ) return;
-    float v[CV][16];
-    {
-        float d[CV][4][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const Pack16<T> pk = sm[q][i][j & 1][tc + (j >> 1)];
-#pragma unroll
-                for (int e = 0; e < CV; ++e) d[e][i][j] = to_f32(pk.e[e]);
-            }
-#pragma unroll
-        for (int e = 0; e < CV; ++e) input_tile_transform(d[e], v[e]);
-    }
-    const long p = ((long)n * th + ty) * tw + tx;
     const size_t plane = (size_t)Cp * Pp;
-    T* vp = V + ((size_t)cq * Pp + p) * CV;
+    for (int tr = 0; tr < TR; ++tr) {
+        const int ty = ty0 + tr;
+        if (ty >= th) break;
+        float v[CV][16];
+        {
+            float d[CV][4][4];
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi) {
-        float o[CV];
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
-        store_chan_vec<T>(vp + xi * plane, o);
+                for (int j = 0; j < 4; ++j) {
+                    const uint4 raw = sm[q][2 * tr + i][j & 1][tc + (j >> 1)];
+                    Pack16<T> pk;
+                    __builtin_memcpy(&pk, &raw, sizeof(pk));
+#pragma unroll
+                    for (int e = 0; e < CV; ++e) d[e][i][j] = to_f32(pk.e[e]);
+                }
+#pragma unroll
+            for (int e = 0; e < CV; ++e) input_tile_transform(d[e], v[e]);
+        }
+        const long p = ((long)n * th + ty) * tw + tx;
+        T* vp = V + ((size_t)cq * Pp + p) * CV;
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi) {
+            float o[CV];
+#pragma unroll
+            for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
+            store_chan_vec<T>(vp + xi * plane, o);
+        }
     }
 }
 

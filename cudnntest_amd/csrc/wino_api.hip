@@ -140,13 +140,13 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
     constexpr int CV = ChanVec<T>::n;
     const int CQ = g.Cp / CV;
     if (layout == WINO_NCHW && order == WINO_TILES_BATCH_MAJOR && g.th * g.tw >= 64) {
-        // TR x TC tiles per workgroup, TR*TC <= 256, halo of CV channels in LDS (<= 44 KB).
+        // TR x TC tiles per workgroup, TR*TC <= 256, halo of CV channels in LDS (<= 60 KB).
         // TR is kept a multiple of 8 when it can be, so a workgroup's run of V (TR*tw
         // 16-byte vectors per coordinate) starts and ends on a 128-byte boundary.
         const int TC = g.tw < 128 ? g.tw : 128;
         int TR = 256 / TC;
-        if (TR > 8) TR = 8;
-        if (TR > g.th) TR = g.th;
+        if (TR >= g.th) TR = g.th;                        // a whole image per workgroup
+        else if (TR > 8) TR &= ~7;
         const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
         const int ldsW = 2 * TC + 2;
         // 2-byte types move image-aligned column pairs (4 bytes per lane) when every row starts 4-byte aligned
@@ -167,12 +167,13 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
         LAUNCH_CHECK("input_transform_nchw");
         return WINO_OK;
     }
-    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR) {
-        constexpr int TC = 32, NQ = 8;
-        const int colBlocks = (g.tw + TC - 1) / TC;
-        dim3 grid((unsigned)((long)g.N * g.th * colBlocks), (CQ + NQ - 1) / NQ), block(TC * NQ);
-        hipLaunchKernelGGL((input_transform_nhwc_kernel<T, TC, NQ>), grid, block, 0, st, (const T*)x, (T*)V, g.N, g.C,
-                           g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks);
+    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && g.C % CV == 0 &&
+        (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        constexpr int TC = 32, NQ = 8, TR = 2;
+        const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
+        dim3 grid((unsigned)((long)g.N * rowBlocks * colBlocks), (CQ + NQ - 1) / NQ), block(TC * NQ);
+        hipLaunchKernelGGL((input_transform_nhwc_kernel<T, TC, NQ, TR>), grid, block, 0, st, (const T*)x, (T*)V, g.N,
+                           g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, rowBlocks);
         LAUNCH_CHECK("input_transform_nhwc");
         return WINO_OK;
     }
@@ -256,7 +257,7 @@ int launch_gemm_rows_d(int dst, int order, unsigned flags, const Geometry& g, co
     constexpr int CV = ChanVec<T>::n;
     // stages per row must be even: one k-group per stage always is (Cp is a multiple of 4 channel
     // vectors); two k-groups per stage (fewer barriers, measured faster) when Cp allows it
-    const bool two = (g.Cp / CV) % 8 == 0;
+    const bool two = (g.Cp / CV) % 8 == 0 && !getenv("WINO_ROWS_ONE");
     if (dst == WINO_NHWC)
         return two ? launch_gemm_rows_t<T, true, 2>(order, flags, g, U, V, y, dst, st)
                    : launch_gemm_rows_t<T, true, 1>(order, flags, g, U, V, y, dst, st);
