@@ -7,7 +7,8 @@ forms; inputs already in HBM).  The default workload is the VGG-16 conv3-style
 layer the headline metric is quoted on: 3x3, stride 1, pad 1, N=32, C=K=256,
 H=W=56, fp32, NCHW.  `--workload vgg16_all13` makes a step the thirteen VGG-16
 convolutions (ReLU fused into the output stage) on synthetic activations of each
-layer's shape.
+layer's shape; `--workload vgg16_stack` chains them through the conv-stack driver
+(bias, ReLU and the five 2x2 poolings in the output stages, cached filter transforms).
 
 Prints ONE JSON line:
   value        effective TFLOP/s = direct-convolution FLOPs (2*N*K*C*H*W*9) / time
@@ -40,6 +41,9 @@ WORKLOADS = {
     "vgg16_conv5_N64_C512_K512_H14": [(64, 512, 512, 14)],
     "vgg16_conv1_2_N32_C64_K64_H224": [(32, 64, 64, 224)],
     "vgg16_all13": None,   # filled from synth.VGG16_CONV at N=32
+    # the same thirteen layers as ONE stack (wino_stack_*): bias + ReLU in every output stage, 2x2 pooling after
+    # conv 2, 4, 7, 10 and 13, activations handed from layer to layer, filter transforms cached outside the step
+    "vgg16_stack": None,
     # the one shape the reference publishes latencies for (layoutTest/NHWC/result.num: NHWC, N=1..128)
     "ref_H22_C128_K128_N64": [(64, 128, 128, 22)],
     "ref_H22_C128_K128_N128": [(128, 128, 128, 22)],
@@ -86,7 +90,7 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
 
-    layers = WORKLOADS[args.workload] or [(32, C, K, H) for (C, K, H) in synth.VGG16_CONV]
+    layers = WORKLOADS[args.workload] or [(32, C, K, H) for (C, K, H) in synth.VGG16_CONV]   # (N, C, K, H)
     multi = len(layers) > 1
     layout = {"NCHW": ops.NCHW, "NHWC": ops.NHWC, "CHWN": ops.CHWN}[args.layout]
     tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
@@ -95,8 +99,23 @@ def main():
             "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4}[args.algo]
     es = 4 if args.dtype == "f32" else 2
 
+    stack = None
+    if args.workload == "vgg16_stack":
+        if args.algo == "staged_f4":
+            print("bench.py: the stack driver has no F(4x4,3x3) mode", file=sys.stderr)
+            sys.exit(2)
+        pools = {1, 3, 6, 9, 12}
+        descs = [dict(K=K, layout_in=layout, layout_out=layout, relu=True, pool=i in pools, algo=algo)
+                 for i, (N, C, K, H) in enumerate(layers)]
+        stack = ops.ConvStack(tdt, 32, 3, 224, 224, descs)
+        for i, (N, C, K, H) in enumerate(layers):
+            _, w_h = synth.conv_inputs(1, C, K, 4, 4, seed=0x5EED + i, layout=layout)
+            b_h = synth.normal(K, 0xB1A5 + i, 0.05)
+            stack.set_layer(i, torch.from_numpy(w_h).cuda().to(tdt).contiguous(), torch.from_numpy(b_h).float().cuda().to(tdt))
     tensors, host_inputs = [], []
     for i, (N, C, K, H) in enumerate(layers):
+        if stack is not None and i > 0:
+            break
         x_h, w_h = synth.conv_inputs(N, C, K, H, H, seed=0x5EED + i, layout=layout)
         x = torch.from_numpy(x_h).cuda().to(tdt).contiguous()
         w = torch.from_numpy(w_h).cuda().to(tdt).contiguous()
@@ -105,7 +124,12 @@ def main():
         if i == 0:
             host_inputs = (x_h, w_h)
 
+    stack_out = torch.empty(stack.out_shape, dtype=tdt, device="cuda") if stack is not None else None
+
     def step():
+        if stack is not None:
+            stack.forward(tensors[0][0], out=stack_out)
+            return
         for (x, w, y) in tensors:
             ops.conv(x, w, 1, layout, algo=algo, relu=multi, out=y)
 
@@ -145,11 +169,13 @@ def main():
         P, nxi = g["P"], (36 if f4 else 16)
         resolved.append(ops.ALGO_NAMES[a])
         gemm_flops += 2.0 * nxi * P * K * C
-        alg_flt += (9 + nxi) * K * C * es
+        if stack is None:
+            alg_flt += (9 + nxi) * K * C * es
         if a != ops.ALGO_FUSED:
             alg_in += N * C * H * H * es + nxi * P * C * es
         if a in (ops.ALGO_STAGED, ops.ALGO_STAGED_F4):
-            alg_out += nxi * P * K * 4 + N * K * H * H * es
+            pooled = stack is not None and len(resolved) - 1 in (1, 3, 6, 9, 12)
+            alg_out += nxi * P * K * 4 + N * K * H * H * es // (4 if pooled else 1)
     stages = {}
     for name, nbytes in (("filter", alg_flt), ("input", alg_in), ("output", alg_out)):
         if per_step[name] > 0 and nbytes > 0:
@@ -178,7 +204,8 @@ def main():
         "config": {"workload": args.workload, "layers": len(layers), "N": N0, "C": C0, "K": K0, "H": H0, "W": H0,
                    "pad": 1, "layout": args.layout, "algo": args.algo, "resolved_algo": resolved,
                    "winograd": "F(4x4,3x3)" if algo_label == "staged_f4" else "F(2x2,3x3)",
-                   "filter_transform_in_step": True, "relu": multi},
+                   "filter_transform_in_step": stack is None, "relu": multi,
+                   "bias_and_pooling_in_step": stack is not None},
         "roofline": roofline,
         "stages": stages,
     }
@@ -197,7 +224,7 @@ def main():
         out["cpu_baseline"] = {"value": round(fl / (c1 - c0) / 1e12, 4), "unit": "TFLOP/s",
                                "cores": oracle.num_threads(), "kind": "port",
                                "sample": ("the whole layer once (all N images)" if not multi else
-                                          "the first of the 13 layers once (all N images)") +
+                                          "the first of the 13 layers once (all N images, convolution and ReLU)") +
                                          ", fp32 direct convolution, OpenMP",
                                "ms": round((c1 - c0) * 1e3, 1)}
     print(json.dumps(out), flush=True)

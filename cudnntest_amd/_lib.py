@@ -17,10 +17,26 @@ _i = ctypes.c_int
 _u = ctypes.c_uint
 _l = ctypes.c_long
 
+
+
+class StackLayer(ctypes.Structure):
+    """wino_stack_layer_t"""
+    _fields_ = [("K", _i), ("layout_in", _i), ("layout_out", _i), ("flags", _u), ("algo", _i)]
+
+
+_ip = ctypes.POINTER(_i)
+
 # every symbol include/wino_amd.h declares: name -> (restype, argtypes)
 SYMBOLS = {
+    "wino_stack_create": (_i, [_i] * 6 + [ctypes.POINTER(StackLayer), ctypes.POINTER(_vp)]),
+    "wino_stack_set_layer": (_i, [_vp, _i, _vp, _vp, _vp]),
+    "wino_stack_output": (_i, [_vp, _ip, _ip, _ip, _ip, _ip]),
+    "wino_stack_forward": (_i, [_vp, _vp, _vp, _vp]),
+    "wino_stack_destroy": (_i, [_vp]),
     "wino_conv": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
     "wino_conv_prepared": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
+    "wino_conv_ex": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp, _vp]),
+    "wino_conv_prepared_ex": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp, _vp]),
     "wino_pick_algo": (_i, [_i] * 8),
     "wino_geometry": (_i, [_i] * 7 + [ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l),
                                      ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l)]),

@@ -52,6 +52,20 @@ template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
     return bf16_t{__builtin_bit_cast(uint16_t, (__bf16)f)};
 }
 
+// What the output stage applies to the 2x2 outputs of a tile before storing them:
+//     y = pool2x2( relu( conv + bias[k] ) )        (each step optional)
+// bias holds K elements of the tensor's element type.  With pool the destination has
+// floor(Ho/2) x floor(Wo/2) outputs per image and filter: the 2x2 outputs of an F(2x2,3x3) tile are
+// exactly one pooling window (the reference applies addBias_CHWN, relu_CHWN and maxPool_CHWN as
+// separate passes over y: netTest/cudnn_test_0124/VGG_Batched/CHWN_support.cuh:107,512,248).
+struct Epilogue {
+    const void* bias;
+    int relu, pool;
+};
+template <typename T> __device__ __forceinline__ float bias_of(const Epilogue& ep, int k) {
+    return ep.bias ? to_f32(static_cast<const T*>(ep.bias)[k]) : 0.f;
+}
+
 // v with its bits ANDed by m (m is all ones or zero).  Opaque to the optimiser on purpose:
 // written as a select, the compiler moves the load that produced v under a branch on the mask and
 // waits for every load separately, instead of issuing a batch of loads and masking afterwards.

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
                                                             T* __restrict__ y, ActStrides xs, ActStrides ys, int N,
                                                             int C, int K, int H, int W, int pad, int Ho, int Wo,
                                                             int th, int tw, long P, int Cp, int Kp, int order,
-                                                            int relu, int kTiles, int pTiles) {
+                                                            Epilogue ep, int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     constexpr int NV = 2 * NVG;                // channel vectors per stage and coordinate
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
         }
         rows_fold<true>(acc, yo, i);
     }
-    rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
+    rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);
 }
 
 }  // namespace wino

@@ -318,13 +318,18 @@ template <typename OutT> __device__ __forceinline__ bool pair_stores_ok(const Ou
 template <typename OutT>
 __device__ __forceinline__ void store_tile_outputs(OutT* __restrict__ y, const ActStrides& ys, int n, int k, int ty,
                                                    int tx, int Ho, int Wo, float y00, float y01, float y10, float y11,
-                                                   int relu, bool pair) {
-    if (relu) {
+                                                   const Epilogue& ep, float bias, bool pair) {
+    y00 += bias; y01 += bias; y10 += bias; y11 += bias;
+    if (ep.relu) {
         y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f);
     }
     const int oh = 2 * ty, ow = 2 * tx;
-    OutT* yp = y + n * ys.n + k * ys.c + oh * ys.h + ow * ys.w;
     const bool w1 = ow + 1 < Wo, h1 = oh + 1 < Ho;
+    if (ep.pool) {                               // ys describes the pooled tensor; a window cut by the edge is dropped
+        if (w1 && h1) y[n * ys.n + k * ys.c + ty * ys.h + tx * ys.w] = from_f32<OutT>(fmaxf(fmaxf(y00, y01), fmaxf(y10, y11)));
+        return;
+    }
+    OutT* yp = y + n * ys.n + k * ys.c + oh * ys.h + ow * ys.w;
     if (pair) {
         struct alignas(2 * sizeof(OutT)) Pair { OutT a, b; };
         *reinterpret_cast<Pair*>(yp) = Pair{from_f32<OutT>(y00), from_f32<OutT>(y01)};
@@ -364,9 +369,9 @@ template <bool CLEAR> __device__ __forceinline__ void rows_fold(floatx16 (&acc)[
 // the lane's l32 the MFMA column.
 template <typename T, bool SWAP>
 __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restrict__ y, const ActStrides& ys, int N,
-                                           int K, int Ho, int Wo, int th, int tw, long P, int order, int relu, int k0,
+                                           int K, int Ho, int Wo, int th, int tw, long P, int order, const Epilogue& ep, int k0,
                                            long p0, int wm, int wn, int l32, int lh) {
-    const bool pair = pair_stores_ok(y, ys, Wo);
+    const bool pair = !ep.pool && pair_stores_ok(y, ys, Wo);
     if (!SWAP) {
         const long p = p0 + wn * 32 + l32;
         if (p >= P) return;
@@ -376,18 +381,19 @@ __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restric
         for (int r = 0; r < 16; ++r) {
             const int k = k0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
             if (k >= K) continue;
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu, pair);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], ep, bias_of<T>(ep, k), pair);
         }
     } else {
         const int k = k0 + wn * 32 + l32;
         if (k >= K) return;
+        const float bk = bias_of<T>(ep, k);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const long p = p0 + wm * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
             if (p >= P) continue;
             int n, ty, tx;
             decode_tile(p, order, N, th, tw, n, ty, tx);
-            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], relu, pair);
+            store_tile_outputs<T>(y, ys, n, k, ty, tx, Ho, Wo, yo[0][r], yo[1][r], yo[2][r], yo[3][r], ep, bk, pair);
         }
     }
 }
@@ -416,7 +422,7 @@ template <typename T, bool SWAP, int NVG>
 __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__ U, const T* __restrict__ V,
                                                            T* __restrict__ y, ActStrides ys, int N, int K, int Ho,
                                                            int Wo, int th, int tw, long P, int Cp, int Kp, long Pp,
-                                                           int order, int relu, int kTiles, int pTiles) {
+                                                           int order, Epilogue ep, int kTiles, int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     constexpr int NV = 2 * NVG;                     // channel vectors per stage and coordinate
@@ -522,7 +528,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         rows_fold<false>(acc, yo, i);
     }
 
-    rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, relu, k0, p0, wm, wn, l32, lh);
+    rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);
 }
 
 

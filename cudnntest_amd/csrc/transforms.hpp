@@ -420,31 +420,24 @@ __global__ __launch_bounds__(TC * NQ) void input_transform_nhwc_kernel(const T* 
 // One thread per (tile p, filter k), p fastest: the 16 loads of a wave are
 // contiguous runs of Mo[xi][k][.].  Stores go through the destination strides.
 template <typename T>
-__global__ __launch_bounds__(256) void output_transform_generic_kernel(const float* __restrict__ Mo,
-                                                                        T* __restrict__ y, ActStrides s, int N,
-                                                                        int K, int Ho, int Wo, int th, int tw,
-                                                                        long P, long Pp, int Kp, int order,
-                                                                        int relu) {
-    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const int k = blockIdx.y;
-    if (p >= P || k >= K) return;
-    const size_t plane = (size_t)Kp * Pp;
-    const float* mp = Mo + (size_t)k * Pp + p;
-    float m[16];
+__device__ __forceinline__ void output_tile_store(T* __restrict__ y, const ActStrides& s, int n, int k, int ty, int tx,
+                                                  int Ho, int Wo, float (&o)[2][2], const Epilogue& ep) {
+    const float bk = bias_of<T>(ep, k);
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];
-    float o[2][2];
-    output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
-    int n, ty, tx;
-    decode_tile(p, order, N, th, tw, n, ty, tx);
-    T* yp = y + n * s.n + k * s.c;
-    if (relu) {
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-            for (int b = 0; b < 2; ++b) o[a][b] = fmaxf(o[a][b], 0.f);
+        for (int b = 0; b < 2; ++b) {
+            o[a][b] += bk;
+            if (ep.relu) o[a][b] = fmaxf(o[a][b], 0.f);
+        }
+    if (ep.pool) {                               // s describes the pooled tensor; a window cut by the edge is dropped
+        if (2 * ty + 1 < Ho && 2 * tx + 1 < Wo)
+            y[n * s.n + k * s.c + ty * s.h + tx * s.w] = from_f32<T>(fmaxf(fmaxf(o[0][0], o[0][1]), fmaxf(o[1][0], o[1][1])));
+        return;
     }
-    if (s.w == 1 && (Wo & 1) == 0 && (s.h & 1) == 0 && (s.c & 1) == 0 && (s.n & 1) == 0) {
+    T* yp = y + n * s.n + k * s.c;
+    if (s.w == 1 && (Wo & 1) == 0 && (s.h & 1) == 0 && (s.c & 1) == 0 && (s.n & 1) == 0 &&
+        (reinterpret_cast<uintptr_t>(y) & (2 * sizeof(T) - 1)) == 0) {
         // W-contiguous destination with even rows: the two outputs of a tile row go out as one store
         struct alignas(2 * sizeof(T)) Pair { T a, b; };
 #pragma unroll
@@ -466,6 +459,27 @@ __global__ __launch_bounds__(256) void output_transform_generic_kernel(const flo
         }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void output_transform_generic_kernel(const float* __restrict__ Mo,
+                                                                        T* __restrict__ y, ActStrides s, int N,
+                                                                        int K, int Ho, int Wo, int th, int tw,
+                                                                        long P, long Pp, int Kp, int order,
+                                                                        Epilogue ep) {
+    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int k = blockIdx.y;
+    if (p >= P || k >= K) return;
+    const size_t plane = (size_t)Kp * Pp;
+    const float* mp = Mo + (size_t)k * Pp + p;
+    float m[16];
+#pragma unroll
+    for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];
+    float o[2][2];
+    output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    output_tile_store<T>(y, s, n, k, ty, tx, Ho, Wo, o, ep);
+}
+
 // ---- output transform from the K-contiguous product Mo[xi][Pp][Kp] ------------------------
 // One thread per (filter k, tile p), k fastest: loads are contiguous along K and
 // so are the stores of a K-contiguous destination (NHWC).
@@ -473,7 +487,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void output_transform_pk_kernel(const float* __restrict__ Mo, T* __restrict__ y,
                                                                    ActStrides s, int N, int K, int Ho, int Wo, int th,
                                                                    int tw, long P, long Pp, int Kp, int order,
-                                                                   int relu) {
+                                                                   Epilogue ep) {
     const int k = blockIdx.x * blockDim.x + threadIdx.x;
     const long p = (long)blockIdx.y * blockDim.y + threadIdx.y;
     if (k >= K || p >= P) return;
@@ -486,18 +500,7 @@ __global__ __launch_bounds__(256) void output_transform_pk_kernel(const float* _
     output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
     int n, ty, tx;
     decode_tile(p, order, N, th, tw, n, ty, tx);
-    T* yp = y + n * s.n + k * s.c;
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int oh = 2 * ty + a, ow = 2 * tx + b;
-            if (oh < Ho && ow < Wo) {
-                float val = o[a][b];
-                if (relu) val = fmaxf(val, 0.f);
-                yp[oh * s.h + ow * s.w] = from_f32<T>(val);
-            }
-        }
+    output_tile_store<T>(y, s, n, k, ty, tx, Ho, Wo, o, ep);
 }
 
 // ---- plain layout permutation -------------------------------------------------------

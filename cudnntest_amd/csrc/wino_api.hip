@@ -1,10 +1,12 @@
 // C ABI of the gfx950 Winograd F(2x2,3x3) convolution library (see include/wino_amd.h).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
+#include <memory>
 #include <vector>
 
 #include "common.hpp"
@@ -185,21 +187,29 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
     return WINO_OK;
 }
 
+// the epilogue a call asks for, and the strides of the tensor it writes (pooled or not)
+inline Epilogue make_epilogue(unsigned flags, const void* bias) {
+    return Epilogue{bias, (flags & WINO_FLAG_RELU) ? 1 : 0, (flags & WINO_FLAG_POOL2) ? 1 : 0};
+}
+inline ActStrides out_strides(int layout, unsigned flags, int N, int K, int Ho, int Wo) {
+    return (flags & WINO_FLAG_POOL2) ? act_strides(layout, N, K, Ho / 2, Wo / 2) : act_strides(layout, N, K, Ho, Wo);
+}
+
 template <typename T>
-int launch_output_transform(int layout, int order, int porder, unsigned flags, int N, int K, int Ho, int Wo, int Kp,
-                            long P, long Pp, const float* Mo, void* y, hipStream_t st) {
+int launch_output_transform(int layout, int order, int porder, unsigned flags, const void* bias, int N, int K, int Ho,
+                            int Wo, int Kp, long P, long Pp, const float* Mo, void* y, hipStream_t st) {
     const int th = (Ho + 1) / 2, tw = (Wo + 1) / 2;
-    const int relu = (flags & WINO_FLAG_RELU) ? 1 : 0;
+    const Epilogue ep = make_epilogue(flags, bias);
     if (porder == WINO_PRODUCT_PK) {
         int bx = 64;
         while (bx < K && bx < 256) bx *= 2;
         dim3 block(bx, 256 / bx), grid((K + bx - 1) / bx, (unsigned)((P + block.y - 1) / block.y));
         hipLaunchKernelGGL(output_transform_pk_kernel<T>, grid, block, 0, st, Mo, (T*)y,
-                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+                           out_strides(layout, flags, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, ep);
     } else {
         dim3 grid((unsigned)((P + 255) / 256), K), block(256);
         hipLaunchKernelGGL(output_transform_generic_kernel<T>, grid, block, 0, st, Mo, (T*)y,
-                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+                           out_strides(layout, flags, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, ep);
     }
     LAUNCH_CHECK("output_transform");
     return WINO_OK;
@@ -238,61 +248,61 @@ int launch_gemm(int nxi, int dtype, int porder, int Cp, int Kp, long Pp, const v
 }
 
 template <typename T, bool SWAP, int NVG>
-int launch_gemm_rows_t(int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y, int dst,
-                       hipStream_t st) {
+int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geometry& g, const void* U, const void* V,
+                       void* y, int dst, hipStream_t st) {
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
     hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG>), grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
-                       act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
-                       g.Pp, order, (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
+                       out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
+                       g.Pp, order, make_epilogue(flags, bias), kTiles, pTiles);
     LAUNCH_CHECK("gemm_rows");
     return WINO_OK;
 }
 
 template <typename T>
-int launch_gemm_rows_d(int dst, int order, unsigned flags, const Geometry& g, const void* U, const void* V, void* y,
-                       hipStream_t st) {
+int launch_gemm_rows_d(int dst, int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
+                       const void* V, void* y, hipStream_t st) {
     constexpr int CV = ChanVec<T>::n;
     // stages per row must be even: one k-group per stage always is (Cp is a multiple of 4 channel
     // vectors); two k-groups per stage (fewer barriers, measured faster) when Cp allows it
     const bool two = (g.Cp / CV) % 8 == 0 && !getenv("WINO_ROWS_ONE");
     if (dst == WINO_NHWC)
-        return two ? launch_gemm_rows_t<T, true, 2>(order, flags, g, U, V, y, dst, st)
-                   : launch_gemm_rows_t<T, true, 1>(order, flags, g, U, V, y, dst, st);
-    return two ? launch_gemm_rows_t<T, false, 2>(order, flags, g, U, V, y, dst, st)
-               : launch_gemm_rows_t<T, false, 1>(order, flags, g, U, V, y, dst, st);
+        return two ? launch_gemm_rows_t<T, true, 2>(order, flags, bias, g, U, V, y, dst, st)
+                   : launch_gemm_rows_t<T, true, 1>(order, flags, bias, g, U, V, y, dst, st);
+    return two ? launch_gemm_rows_t<T, false, 2>(order, flags, bias, g, U, V, y, dst, st)
+               : launch_gemm_rows_t<T, false, 1>(order, flags, bias, g, U, V, y, dst, st);
 }
 
-int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* U, const void* V,
-                    void* y, hipStream_t st) {
+int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
+                    const void* V, void* y, hipStream_t st) {
     switch (dtype) {
-    case WINO_F32: return launch_gemm_rows_d<float>(dst, order, flags, g, U, V, y, st);
-    case WINO_F16: return launch_gemm_rows_d<f16_t>(dst, order, flags, g, U, V, y, st);
-    case WINO_BF16: return launch_gemm_rows_d<bf16_t>(dst, order, flags, g, U, V, y, st);
+    case WINO_F32: return launch_gemm_rows_d<float>(dst, order, flags, bias, g, U, V, y, st);
+    case WINO_F16: return launch_gemm_rows_d<f16_t>(dst, order, flags, bias, g, U, V, y, st);
+    case WINO_BF16: return launch_gemm_rows_d<bf16_t>(dst, order, flags, bias, g, U, V, y, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
 template <typename T, bool SWAP, int XM, int NVG>
-int launch_fused_rows_t(int src, int dst, int order, unsigned flags, const Geometry& g, const void* x, const void* U,
-                        void* y, hipStream_t st) {
+int launch_fused_rows_t(int src, int dst, int order, unsigned flags, const void* bias, const Geometry& g, const void* x,
+                        const void* U, void* y, hipStream_t st) {
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
     hipLaunchKernelGGL((fused_rows_kernel<T, SWAP, XM, NVG>), grid, block, 0, st, (const T*)x, (const T*)U, (T*)y,
-                       act_strides(src, g.N, g.C, g.H, g.W), act_strides(dst, g.N, g.K, g.Ho, g.Wo), g.N, g.C, g.K,
-                       g.H, g.W, g.pad, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, order,
-                       (flags & WINO_FLAG_RELU) ? 1 : 0, kTiles, pTiles);
+                       act_strides(src, g.N, g.C, g.H, g.W), out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo), g.N, g.C, g.K,
+                       g.H, g.W, g.pad, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, order, make_epilogue(flags, bias),
+                       kTiles, pTiles);
     LAUNCH_CHECK("fused_rows");
     return WINO_OK;
 }
 
 template <typename T>
-int launch_fused_d(int src, int dst, int order, unsigned flags, const Geometry& g, const void* x, const void* U,
-                   void* y, hipStream_t st) {
+int launch_fused_d(int src, int dst, int order, unsigned flags, const void* bias, const Geometry& g, const void* x,
+                   const void* U, void* y, hipStream_t st) {
     if ((long)g.N * g.C * g.H * g.W >= (1L << 31))
         return fail(WINO_ERR_UNSUPPORTED, "fused kernel: input tensor too large for 32-bit element offsets");
     constexpr int CV = ChanVec<T>::n;
@@ -303,7 +313,7 @@ int launch_fused_d(int src, int dst, int order, unsigned flags, const Geometry& 
     if (sizeof(T) == 2 && !(chan_contig && g.C % CV == 0)) two = false;
     const int un = (two ? 2 : 1) * CV / 2;     // channels per thread
     const int xm = (chan_contig && g.C % un == 0) ? XM_CHANVEC : ((src == WINO_NCHW && g.W >= 4) ? XM_ROW : XM_SCALAR);
-#define FR(SW, XM, NG) return launch_fused_rows_t<T, SW, XM, NG>(src, dst, order, flags, g, x, U, y, st)
+#define FR(SW, XM, NG) return launch_fused_rows_t<T, SW, XM, NG>(src, dst, order, flags, bias, g, x, U, y, st)
 #define FR2(SW, NG)                               \
     if (xm == XM_CHANVEC) FR(SW, XM_CHANVEC, NG); \
     if (xm == XM_ROW) FR(SW, XM_ROW, NG);         \
@@ -323,12 +333,12 @@ int launch_fused_d(int src, int dst, int order, unsigned flags, const Geometry& 
 #undef FR
 }
 
-int launch_fused(int src, int dst, int dtype, int order, unsigned flags, const Geometry& g, const void* x,
-                 const void* U, void* y, hipStream_t st) {
+int launch_fused(int src, int dst, int dtype, int order, unsigned flags, const void* bias, const Geometry& g,
+                 const void* x, const void* U, void* y, hipStream_t st) {
     switch (dtype) {
-    case WINO_F32: return launch_fused_d<float>(src, dst, order, flags, g, x, U, y, st);
-    case WINO_F16: return launch_fused_d<f16_t>(src, dst, order, flags, g, x, U, y, st);
-    case WINO_BF16: return launch_fused_d<bf16_t>(src, dst, order, flags, g, x, U, y, st);
+    case WINO_F32: return launch_fused_d<float>(src, dst, order, flags, bias, g, x, U, y, st);
+    case WINO_F16: return launch_fused_d<f16_t>(src, dst, order, flags, bias, g, x, U, y, st);
+    case WINO_BF16: return launch_fused_d<bf16_t>(src, dst, order, flags, bias, g, x, U, y, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -452,7 +462,7 @@ int conv_f4_impl(int src, int dst, int dtype, unsigned flags, int N, int C, int 
 }
 
 int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
-              const void* x, const void* w, const void* Upre, void* y, void* stream) {
+              const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_STAGED_F4) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
@@ -460,7 +470,14 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
+    if (flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)) return fail(WINO_ERR_INVALID, "unknown flags 0x%x", flags);
+    if ((flags & WINO_FLAG_POOL2) && (g.Ho < 2 || g.Wo < 2))
+        return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", g.Ho, g.Wo);
     if (algo == WINO_ALGO_AUTO) algo = pick_algo(src, dtype, g);
+    if (algo == WINO_ALGO_STAGED_F4) {
+        if (bias || (flags & WINO_FLAG_POOL2))
+            return fail(WINO_ERR_UNSUPPORTED, "bias and pooling are not built for the F(4x4,3x3) mode");
+    }
     if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(src, dst, dtype, flags, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
     hipStream_t st = (hipStream_t)stream;
@@ -483,7 +500,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     }
     if (algo == WINO_ALGO_FUSED) {
         StageScope t(WINO_STAGE_GEMM, st);
-        return launch_fused(src, dst, dtype, order, flags, g, x, U, y, st);
+        return launch_fused(src, dst, dtype, order, flags, bias, g, x, U, y, st);
     }
     {
         StageScope t(WINO_STAGE_INPUT, st);
@@ -492,7 +509,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     }
     if (algo == WINO_ALGO_EPILOGUE) {
         StageScope t(WINO_STAGE_GEMM, st);
-        return launch_gemm_out(dst, dtype, order, flags, g, U, V, y, st);
+        return launch_gemm_out(dst, dtype, order, flags, bias, g, U, V, y, st);
     }
     const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
     {
@@ -501,7 +518,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         if (rc) return rc;
     }
     StageScope t(WINO_STAGE_OUTPUT, st);
-    return wino_output_transform(dst, dtype, order, porder, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
+    DISPATCH_DTYPE(dtype, launch_output_transform<T>(dst, order, porder, flags, bias, N, K, g.Ho, g.Wo, g.Kp, g.P, g.Pp, Mo, y, st));
 }
 
 __global__ void warmup_kernel() {}
@@ -513,13 +530,23 @@ extern "C" {
 int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
               const void* x, const void* w, void* y, void* stream) {
     if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
-    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, y, stream);
+    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, nullptr, y, stream);
+}
+int wino_conv_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
+                 const void* x, const void* w, const void* bias, void* y, void* stream) {
+    if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
+    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, bias, y, stream);
 }
 
 int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W,
                        int pad, const void* x, const void* U, void* y, void* stream) {
     if (!U) return fail(WINO_ERR_INVALID, "null transformed-filter pointer");
-    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, y, stream);
+    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, nullptr, y, stream);
+}
+int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W,
+                          int pad, const void* x, const void* U, const void* bias, void* y, void* stream) {
+    if (!U) return fail(WINO_ERR_INVALID, "null transformed-filter pointer");
+    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, bias, y, stream);
 }
 
 int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int pad) {
@@ -607,7 +634,7 @@ int wino_output_transform(int layout, int dtype, int tile_order, int product_ord
     const long P = (long)N * ((Ho + 1) / 2) * ((Wo + 1) / 2);
     const int Kp = (int)round_up(K, kKPad);
     const long Pp = round_up(P, kPPad);
-    DISPATCH_DTYPE(dtype, launch_output_transform<T>(layout, tile_order, product_order, flags, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
+    DISPATCH_DTYPE(dtype, launch_output_transform<T>(layout, tile_order, product_order, flags, nullptr, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
                                                      (hipStream_t)stream));
 }
 
@@ -621,7 +648,7 @@ int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int 
     // geometry from the output size: pad 1 keeps H == Ho
     if (!make_geometry(dtype, N, C, K, Ho, Wo, 1, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d Ho=%d Wo=%d", N, C, K, Ho, Wo);
-    return launch_gemm_out(layout, dtype, tile_order, flags, g, U, V, y, (hipStream_t)stream);
+    return launch_gemm_out(layout, dtype, tile_order, flags, nullptr, g, U, V, y, (hipStream_t)stream);
 }
 
 int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void* in, void* out,
@@ -731,6 +758,129 @@ int wino_stage_times(float* ms, long* calls) {
         (void)hipEventDestroy(sp.b);
     }
     return rc;
+}
+
+// ---- conv stack ------------------------------------------------------------------------------------
+struct wino_stack {
+    int device = 0, dtype = 0, N = 0;
+    struct Layer {
+        int C, K, H, W;            // input of the layer
+        int Ho, Wo;                // what it writes (after pooling)
+        int layout_in, layout_out, algo;
+        unsigned flags;
+        void* U = nullptr;         // cached transformed filters
+        void* bias = nullptr;
+        bool set = false, has_bias = false;
+    };
+    std::vector<Layer> layers;
+    void* act[2] = {nullptr, nullptr};   // activations between layers
+    size_t act_bytes = 0;
+};
+
+int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const wino_stack_layer_t* layers,
+                      wino_stack_t** stack) {
+    if (!stack || !layers) return fail(WINO_ERR_INVALID, "null pointer");
+    *stack = nullptr;
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (nlayers <= 0 || N <= 0 || C <= 0 || H <= 0 || W <= 0)
+        return fail(WINO_ERR_INVALID, "bad stack shape N=%d C=%d H=%d W=%d layers=%d", N, C, H, W, nlayers);
+    std::unique_ptr<wino_stack> s(new wino_stack);
+    s->dtype = dtype;
+    s->N = N;
+    HIP_TRY(hipGetDevice(&s->device));
+    const size_t es = dtype_size(dtype);
+    int c = C, h = H, w = W;
+    for (int l = 0; l < nlayers; ++l) {
+        const wino_stack_layer_t& d = layers[l];
+        if (d.K <= 0 || !valid_layout(d.layout_in) || !valid_layout(d.layout_out) ||
+            d.algo < WINO_ALGO_AUTO || d.algo > WINO_ALGO_FUSED ||
+            (d.flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)))
+            return fail(WINO_ERR_INVALID, "layer %d: bad description", l);
+        if (l > 0 && d.layout_in != layers[l - 1].layout_out)
+            return fail(WINO_ERR_INVALID, "layer %d reads layout %d, layer %d writes %d", l, d.layout_in, l - 1,
+                        layers[l - 1].layout_out);
+        wino_stack::Layer L;
+        L.C = c; L.K = d.K; L.H = h; L.W = w;
+        L.layout_in = d.layout_in; L.layout_out = d.layout_out; L.algo = d.algo; L.flags = d.flags;
+        const bool pool = d.flags & WINO_FLAG_POOL2;
+        if (pool && (h < 2 || w < 2)) return fail(WINO_ERR_INVALID, "layer %d pools a %dx%d image", l, h, w);
+        L.Ho = pool ? h / 2 : h;
+        L.Wo = pool ? w / 2 : w;
+        Geometry g;
+        if (!make_geometry(dtype, N, c, d.K, h, w, 1, &g)) return fail(WINO_ERR_INVALID, "layer %d: bad shape", l);
+        if (l + 1 < nlayers) s->act_bytes = std::max(s->act_bytes, (size_t)N * d.K * L.Ho * L.Wo * es);
+        s->layers.push_back(L);
+        c = d.K; h = L.Ho; w = L.Wo;
+    }
+    // device memory; on failure the destructor path below releases what was taken
+    wino_stack* raw = s.release();
+    auto bail = [&](hipError_t e) {
+        wino_stack_destroy(raw);
+        return fail(WINO_ERR_HIP, "stack allocation: %s", hipGetErrorString(e));
+    };
+    for (auto& L : raw->layers) {
+        Geometry g;
+        make_geometry(dtype, N, L.C, L.K, L.H, L.W, 1, &g);
+        hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
+        if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
+        if (e != hipSuccess) return bail(e);
+    }
+    for (int i = 0; i < 2 && raw->act_bytes; ++i) {
+        hipError_t e = hipMalloc(&raw->act[i], raw->act_bytes);
+        if (e != hipSuccess) return bail(e);
+    }
+    *stack = raw;
+    return WINO_OK;
+}
+
+int wino_stack_set_layer(wino_stack_t* s, int layer, const void* w, const void* bias, void* stream) {
+    if (!s || !w) return fail(WINO_ERR_INVALID, "null pointer");
+    if (layer < 0 || layer >= (int)s->layers.size()) return fail(WINO_ERR_INVALID, "no layer %d", layer);
+    auto& L = s->layers[layer];
+    int rc = wino_filter_transform(L.layout_in, s->dtype, L.K, L.C, w, L.U, stream);
+    if (rc) return rc;
+    L.has_bias = bias != nullptr;
+    if (bias)
+        HIP_TRY(hipMemcpyAsync(L.bias, bias, (size_t)L.K * dtype_size(s->dtype), hipMemcpyDeviceToDevice,
+                               (hipStream_t)stream));
+    L.set = true;
+    return WINO_OK;
+}
+
+int wino_stack_output(const wino_stack_t* s, int* N, int* K, int* H, int* W, int* layout) {
+    if (!s || !N || !K || !H || !W || !layout) return fail(WINO_ERR_INVALID, "null pointer");
+    const auto& L = s->layers.back();
+    *N = s->N; *K = L.K; *H = L.Ho; *W = L.Wo; *layout = L.layout_out;
+    return WINO_OK;
+}
+
+int wino_stack_forward(wino_stack_t* s, const void* x, void* y, void* stream) {
+    if (!s || !x || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    const int n = (int)s->layers.size();
+    for (int l = 0; l < n; ++l)
+        if (!s->layers[l].set) return fail(WINO_ERR_INVALID, "layer %d has no filters yet", l);
+    const void* in = x;
+    for (int l = 0; l < n; ++l) {
+        const auto& L = s->layers[l];
+        void* out = l + 1 == n ? y : s->act[l & 1];
+        int rc = conv_impl(L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
+                           nullptr, L.U, L.has_bias ? L.bias : nullptr, out, stream);
+        if (rc) return rc;
+        in = out;
+    }
+    return WINO_OK;
+}
+
+int wino_stack_destroy(wino_stack_t* s) {
+    if (!s) return WINO_OK;
+    for (auto& L : s->layers) {
+        if (L.U) (void)hipFree(L.U);
+        if (L.bias) (void)hipFree(L.bias);
+    }
+    for (int i = 0; i < 2; ++i)
+        if (s->act[i]) (void)hipFree(s->act[i]);
+    delete s;
+    return WINO_OK;
 }
 
 int wino_warmup(void) {

@@ -27,6 +27,7 @@ ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED, ALGO_STAGED_F4 = 0, 1, 2, 3, 
 TILES_BATCH_MAJOR, TILES_BATCH_MINOR = 0, 1
 PRODUCT_KP, PRODUCT_PK = 0, 1
 FLAG_RELU = 1
+FLAG_POOL2 = 2
 
 
 class DataLayout(enum.IntEnum):
@@ -119,8 +120,27 @@ def stage_times():
 
 # ---- whole layer -------------------------------------------------------------
 
-def conv(x, w, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None):
-    """y = conv3x3(x, w); x, w in `src`'s conventions, y in `dst`'s.  Asynchronous."""
+def _out_for(dst, x, N, K, Ho, Wo, pool, out):
+    if pool:
+        Ho, Wo = Ho // 2, Wo // 2
+    shape = act_shape(dst, N, K, Ho, Wo)
+    if out is None:
+        return torch.empty(shape, dtype=x.dtype, device=x.device)
+    if tuple(out.shape) != tuple(shape):
+        raise ValueError(f"out has shape {tuple(out.shape)}, the layer writes {tuple(shape)}")
+    return out
+
+
+def _check_bias(bias, x, K):
+    if bias is None:
+        return None
+    if bias.dtype != x.dtype or bias.numel() != K or not bias.is_contiguous():
+        raise TypeError("bias must hold K contiguous elements of x's dtype")
+    return bias
+
+
+def conv(x, w, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None, bias=None, pool=False):
+    """y = pool2x2?(relu?(conv3x3(x, w) + bias)); x, w in `src`'s conventions, y in `dst`'s.  Asynchronous."""
     dst = src if dst is None else dst
     N, C, H, W = act_dims(src, x)
     K, C2 = flt_dims(src, w)
@@ -128,24 +148,82 @@ def conv(x, w, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None):
         raise ValueError(f"filter bank has {C2} channels, input has {C}")
     if w.dtype != x.dtype:
         raise TypeError("x and w must share a dtype")
-    if out is None:
-        out = torch.empty(act_shape(dst, N, K, H + 2 * pad - 2, W + 2 * pad - 2), dtype=x.dtype, device=x.device)
-    rc = _lib.load().wino_conv(int(src), int(dst), _dt(x), algo, FLAG_RELU if relu else 0, N, C, K, H, W, pad,
-                               _ptr(x), _ptr(w), _ptr(out), _stream())
-    _lib.check(rc, "wino_conv")
+    bias = _check_bias(bias, x, K)
+    out = _out_for(dst, x, N, K, H + 2 * pad - 2, W + 2 * pad - 2, pool, out)
+    flags = (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0)
+    rc = _lib.load().wino_conv_ex(int(src), int(dst), _dt(x), algo, flags, N, C, K, H, W, pad,
+                                  _ptr(x), _ptr(w), _ptr(bias) if bias is not None else None, _ptr(out), _stream())
+    _lib.check(rc, "wino_conv_ex")
     return out
 
 
-def conv_prepared(x, U, K, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None):
+def conv_prepared(x, U, K, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None, bias=None, pool=False):
     """Same with the filter bank already transformed by filter_transform()."""
     dst = src if dst is None else dst
     N, C, H, W = act_dims(src, x)
-    if out is None:
-        out = torch.empty(act_shape(dst, N, K, H + 2 * pad - 2, W + 2 * pad - 2), dtype=x.dtype, device=x.device)
-    rc = _lib.load().wino_conv_prepared(int(src), int(dst), _dt(x), algo, FLAG_RELU if relu else 0, N, C, K, H, W,
-                                        pad, _ptr(x), _ptr(U), _ptr(out), _stream())
-    _lib.check(rc, "wino_conv_prepared")
+    bias = _check_bias(bias, x, K)
+    out = _out_for(dst, x, N, K, H + 2 * pad - 2, W + 2 * pad - 2, pool, out)
+    flags = (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0)
+    rc = _lib.load().wino_conv_prepared_ex(int(src), int(dst), _dt(x), algo, flags, N, C, K, H, W, pad, _ptr(x),
+                                           _ptr(U), _ptr(bias) if bias is not None else None, _ptr(out), _stream())
+    _lib.check(rc, "wino_conv_prepared_ex")
     return out
+
+
+class ConvStack:
+    """A stack of 3x3 / pad 1 convolution layers with cached filter transforms and bias, ReLU and 2x2
+    pooling in each layer's output stage (wino_stack_*): the convolution part of the reference's
+    classify_example_modified (netTest/cudnn_test_0124/VGG_Batched/Network.h:603-669).
+
+    layers: list of dicts {K, layout_in, layout_out, relu, pool, algo}; `layout_in` of a layer defaults to
+    the previous layer's `layout_out` (the first: NCHW), `layout_out` to its own `layout_in`."""
+
+    def __init__(self, dtype, N, C, H, W, layers):
+        import ctypes
+        descs = (_lib.StackLayer * len(layers))()
+        prev = None
+        for d, L in zip(descs, layers):
+            d.K = int(L["K"])
+            d.layout_in = int(L.get("layout_in", prev if prev is not None else NCHW))
+            d.layout_out = int(L.get("layout_out", d.layout_in))
+            d.flags = (FLAG_RELU if L.get("relu", False) else 0) | (FLAG_POOL2 if L.get("pool", False) else 0)
+            d.algo = int(L.get("algo", ALGO_AUTO))
+            prev = d.layout_out
+        self._descs = descs
+        self._h = ctypes.c_void_p()
+        self.dtype = dtype
+        self.in_shape = act_shape(descs[0].layout_in, N, C, H, W)
+        _lib.check(_lib.load().wino_stack_create(_DTYPES[dtype], N, C, H, W, len(layers), descs, self._h),
+                   "wino_stack_create")
+        n, k, h, w, lay = (ctypes.c_int() for _ in range(5))
+        _lib.check(_lib.load().wino_stack_output(self._h, n, k, h, w, lay), "wino_stack_output")
+        self.out_layout = lay.value
+        self.out_shape = act_shape(lay.value, n.value, k.value, h.value, w.value)
+
+    def set_layer(self, layer, w, bias=None):
+        if w.dtype != self.dtype or (bias is not None and bias.dtype != self.dtype):
+            raise TypeError("filters and bias must have the stack's dtype")
+        _lib.check(_lib.load().wino_stack_set_layer(self._h, layer, _ptr(w), _ptr(bias) if bias is not None else None,
+                                                    _stream()), "wino_stack_set_layer")
+
+    def forward(self, x, out=None):
+        if tuple(x.shape) != tuple(self.in_shape) or x.dtype != self.dtype:
+            raise ValueError(f"input must be {tuple(self.in_shape)} of {self.dtype}")
+        if out is None:
+            out = torch.empty(self.out_shape, dtype=self.dtype, device=x.device)
+        _lib.check(_lib.load().wino_stack_forward(self._h, _ptr(x), _ptr(out), _stream()), "wino_stack_forward")
+        return out
+
+    def close(self):
+        if self._h:
+            _lib.load().wino_stack_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 # ---- stages ------------------------------------------------------------------------
@@ -183,18 +261,21 @@ def batched_gemm(U, V, C, K, P, product_order=PRODUCT_KP):
 
 
 def output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False, dtype=torch.float32,
-                     product_order=PRODUCT_KP):
-    y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=dtype, device=Mo.device)
+                     product_order=PRODUCT_KP, pool=False):
+    y = torch.empty(act_shape(layout, N, K, Ho // 2, Wo // 2) if pool else act_shape(layout, N, K, Ho, Wo),
+                    dtype=dtype, device=Mo.device)
     _lib.check(_lib.load().wino_output_transform(int(layout), _DTYPES[dtype], tile_order, product_order,
-                                                 FLAG_RELU if relu else 0,
+                                                 (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0),
                                                  N, K, Ho, Wo, _ptr(Mo), _ptr(y), _stream()),
                "wino_output_transform")
     return y
 
 
-def gemm_output(U, V, N, C, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False):
-    y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=U.dtype, device=U.device)
-    _lib.check(_lib.load().wino_gemm_output(int(layout), _dt(U), tile_order, FLAG_RELU if relu else 0, N, C, K, Ho,
+def gemm_output(U, V, N, C, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False, pool=False):
+    y = torch.empty(act_shape(layout, N, K, Ho // 2, Wo // 2) if pool else act_shape(layout, N, K, Ho, Wo),
+                    dtype=U.dtype, device=U.device)
+    _lib.check(_lib.load().wino_gemm_output(int(layout), _dt(U), tile_order,
+                                            (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0), N, C, K, Ho,
                                             Wo, _ptr(U), _ptr(V), _ptr(y), _stream()), "wino_gemm_output")
     return y
 

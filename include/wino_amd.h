@@ -62,8 +62,10 @@ typedef enum {
     WINO_ERR_WORKSPACE = -4    /* caller-provided workspace too small */
 } wino_status_t;
 
-/* flags for wino_conv */
-#define WINO_FLAG_RELU 1u /* clamp negatives in the output transform */
+/* flags for wino_conv and the output-side stage functions */
+#define WINO_FLAG_RELU 1u  /* clamp negatives in the output stage */
+#define WINO_FLAG_POOL2 2u /* 2x2 / stride-2 max pooling in the output stage: y has floor(Ho/2) x floor(Wo/2)
+                              outputs per image and filter (the 2x2 outputs of a tile are one window) */
 
 /*
  * Whole layer: y = conv3x3(x, w).  x and w are in `src`'s conventions, y in
@@ -85,6 +87,20 @@ int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
  */
 int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K,
                        int H, int W, int pad, const void *x, const void *U, void *y, void *stream);
+
+/*
+ * The two calls above with a per-filter bias (K elements of the tensor's element type, or NULL):
+ *   y = pool2x2?( relu?( conv3x3(x, w) + bias[k] ) )
+ * in the output stage of whichever algorithm runs, instead of the separate passes over y of
+ *   addBias_CHWN / relu_CHWN / maxPool_CHWN
+ *   netTest/cudnn_test_0124/VGG_Batched/CHWN_support.cuh:107,512,248
+ * (the fused form is what fusedTest/winotrans.cuh:380-400 sketches).  Not built for WINO_ALGO_STAGED_F4.
+ */
+int wino_conv_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
+                 int W, int pad, const void *x, const void *w, const void *bias, void *y, void *stream);
+int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K,
+                          int H, int W, int pad, const void *x, const void *U, const void *bias, void *y,
+                          void *stream);
 
 /* the algorithm WINO_ALGO_AUTO resolves to for this problem (a wino_algo_t), or a negative status;
  * layout is that of the input tensor */
@@ -165,6 +181,34 @@ typedef enum {
 } wino_stage_t;
 int wino_stage_timing(int enable);
 int wino_stage_times(float *ms, long *calls);
+
+/* ---- a stack of 3x3 convolution layers with cached filter transforms -------------------------
+ * The convolution part of the reference's network driver, classify_example_modified
+ * (netTest/cudnn_test_0124/VGG_Batched/Network.h:603-669): per layer convMethodChoose (:456-519:
+ * layoutManager with the layer's own layout_in / layout_out, then addBias), activationForward, and
+ * poolForward after some layers -- here one wino_conv_prepared_ex call per layer, with bias, ReLU and
+ * pooling in its output stage, the filter bank of every layer transformed once when it is set (the
+ * reference transforms it again on every call), and the activations between layers in two buffers the
+ * stack owns.  The fully connected layers and the softmax of the reference driver are cuBLAS/cuDNN
+ * code and not part of this library.  Every layer is 3x3, stride 1, pad 1. */
+typedef struct wino_stack wino_stack_t;
+typedef struct {
+    int K;                     /* filters of the layer; its channels are the previous layer's K */
+    int layout_in, layout_out; /* wino_layout_t; layout_in must equal the previous layer's layout_out */
+    unsigned flags;            /* WINO_FLAG_RELU | WINO_FLAG_POOL2 */
+    int algo;                  /* wino_algo_t, normally WINO_ALGO_AUTO */
+} wino_stack_layer_t;
+/* the stack for inputs of N x C x H x W in layers[0].layout_in; allocates device memory */
+int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const wino_stack_layer_t *layers,
+                      wino_stack_t **stack);
+/* filter bank (in the layer's layout_in convention) and bias (K elements or NULL) of one layer, both device
+ * pointers; the bank is transformed and the bias copied before the call returns control to the stream */
+int wino_stack_set_layer(wino_stack_t *stack, int layer, const void *w, const void *bias, void *stream);
+/* shape and layout of what wino_stack_forward writes */
+int wino_stack_output(const wino_stack_t *stack, int *N, int *K, int *H, int *W, int *layout);
+/* all layers on `stream`; x and y are caller tensors; fails if a layer has not been set */
+int wino_stack_forward(wino_stack_t *stack, const void *x, void *y, void *stream);
+int wino_stack_destroy(wino_stack_t *stack);
 
 /* ---- housekeeping ----------------------------------------------------------- */
 int wino_warmup(void);                 /* empty kernel; replaces warmup<<<1,1>>> (wrapedConv_NCHW.cuh:4-7) */

@@ -1,0 +1,92 @@
+"""The conv-stack driver (wino_stack_*): the convolution part of the reference's network driver
+classify_example_modified (netTest/cudnn_test_0124/VGG_Batched/Network.h:603-669) -- per layer a
+3x3 convolution in the layer's own layout pair, bias, ReLU, and 2x2 pooling after some layers --
+with the filter transforms cached.  Oracle: the CPU direct convolution layer by layer, bias / ReLU /
+pooling in NumPy."""
+import numpy as np
+import pytest
+import torch
+
+from cudnntest_amd import _lib, ops, synth
+from gpu_util import TOL, TORCH_DT, dev, host, rounded
+
+pytestmark = pytest.mark.gpu
+
+
+def reference_chain(oracle, x_nchw, params, layers):
+    """fp32 chain in NCHW: conv + bias -> relu -> pool, per layer."""
+    a = x_nchw
+    for (w, b), L in zip(params, layers):
+        a = oracle.direct_conv_f32(a, w, 1)
+        a = a + b[None, :, None, None]
+        if L.get("relu"):
+            a = np.maximum(a, 0)
+        if L.get("pool"):
+            N, K, H, W = a.shape
+            a = a[:, :, :H // 2 * 2, :W // 2 * 2].reshape(N, K, H // 2, 2, W // 2, 2).max(axis=(3, 5))
+        a = np.ascontiguousarray(a.astype(np.float32))
+    return a
+
+
+def make_params(oracle, C, layers, dtype):
+    params = []
+    for i, L in enumerate(layers):
+        K = L["K"]
+        w = rounded(synth.normal(K * C * 9, 0x300 + i, float(np.sqrt(2.0 / (9.0 * C)))).reshape(K, C, 3, 3), dtype, oracle)
+        b = rounded(synth.normal(K, 0x400 + i, 0.1).astype(np.float32), dtype, oracle)
+        params.append((w, b))
+        C = K
+    return params
+
+
+VGG_LIKE = [dict(K=16, relu=True), dict(K=16, relu=True, pool=True), dict(K=32, relu=True),
+            dict(K=32, relu=True, pool=True), dict(K=64, relu=True), dict(K=64, relu=True, pool=True)]
+
+
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16, ops.BF16])
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
+def test_stack_matches_the_layerwise_oracle(oracle, layout, dtype):
+    N, C, H = 3, 3, 36
+    layers = [dict(L, layout_in=layout, layout_out=layout) for L in VGG_LIKE]
+    # the reference hands the activations over to NCHW at its last convolution (vggCUDNN.cu:173-176)
+    layers[-1]["layout_out"] = ops.NCHW
+    params = make_params(oracle, C, layers, dtype)
+    x = rounded(synth.uniform_pm1(N * C * H * H, 0xA1).reshape(N, C, H, H), dtype, oracle)
+    want = reference_chain(oracle, x, params, layers)
+
+    st = ops.ConvStack(TORCH_DT[dtype], N, C, H, H, layers)
+    assert tuple(st.out_shape) == want.shape and st.out_layout == ops.NCHW
+    for i, (w, b) in enumerate(params):
+        st.set_layer(i, dev(synth.flt_to_layout(w, layout), dtype), dev(b, dtype))
+    xd = dev(synth.act_to_layout(x, layout), dtype)
+    got = st.forward(xd)
+    assert oracle.rel_l2(host(got), want) <= TOL[dtype]
+
+    # the same layers one wino_conv_ex call at a time give the same bits
+    a = xd
+    for (w, b), L in zip(params, layers):
+        a = ops.conv(a, dev(synth.flt_to_layout(w, layout), dtype), 1, L["layout_in"], L["layout_out"],
+                     relu=L.get("relu", False), pool=L.get("pool", False), bias=dev(b, dtype))
+    assert torch.equal(a, got)
+    # a second pass over the cached transforms gives the same bits again
+    assert torch.equal(st.forward(xd), got)
+    st.close()
+
+
+def test_stack_rejects_bad_requests():
+    with pytest.raises(_lib.WinoError):          # layer 1 reads what layer 0 does not write
+        ops.ConvStack(torch.float32, 1, 3, 8, 8, [dict(K=4, layout_in=ops.NCHW, layout_out=ops.NHWC),
+                                                   dict(K=4, layout_in=ops.CHWN)])
+    st = ops.ConvStack(torch.float32, 1, 3, 8, 8, [dict(K=4), dict(K=4, pool=True)])
+    assert tuple(st.out_shape) == (1, 4, 4, 4)
+    x = torch.zeros((1, 3, 8, 8), device="cuda")
+    with pytest.raises(_lib.WinoError):          # no filters yet
+        st.forward(x)
+    st.set_layer(0, torch.zeros((4, 3, 3, 3), device="cuda"))
+    with pytest.raises(_lib.WinoError):          # layer 1 still missing
+        st.forward(x)
+    with pytest.raises(_lib.WinoError):
+        st.set_layer(2, torch.zeros((4, 4, 3, 3), device="cuda"))
+    st.set_layer(1, torch.zeros((4, 4, 3, 3), device="cuda"), torch.ones(4, device="cuda"))
+    assert torch.equal(st.forward(x), torch.ones((1, 4, 4, 4), device="cuda"))
+    st.close()
