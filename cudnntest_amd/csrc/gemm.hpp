@@ -398,6 +398,11 @@ __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restric
     }
 }
 
+// f(integral_constant<int, S>) for every S of the sequence, in order
+template <int... S, class F> __device__ __forceinline__ void for_each_const(std::integer_sequence<int, S...>, F&& f) {
+    (f(std::integral_constant<int, S>{}), ...);
+}
+
 // =============================================================================
 // GEMM with the output transform in its epilogue, one Winograd ROW at a time.
 //
@@ -407,7 +412,7 @@ __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restric
 // planes y00, y01, y10, y11 of its (filter, tile) pairs.  When the channel
 // reduction of row i ends, the row is folded into the outputs,
 //     T_b = (A^T-column transform of m_i0..m_i3)_b,   y_ab += (A^T)_{a i} * T_b,
-// and the accumulators restart for row i+1.  A wave needs ~170 registers instead
+// and the accumulators restart for row i+1.  A wave needs ~160 registers instead
 // of 512, so three workgroups share a CU: their barriers and load latencies
 // overlap, and three times as many waves pull operands from L2 (one 4-wave
 // workgroup per CU cannot draw more than ~38 B/clk, which is what a kernel that
@@ -415,19 +420,37 @@ __device__ __forceinline__ void rows_store(const floatx16 (&yo)[4], T* __restric
 // peak; that variant measured 8-14 % slower on every shape).
 //
 // A stage is NVG k-groups of one row: [4][2*NVG][64] channel vectors of U and of V,
-// moved HBM -> LDS by global_load_lds_dwordx4, two static stages.  The 4 * nst
-// stages of a patch form one pipeline that runs across the row boundaries.
+// moved HBM -> LDS by global_load_lds_dwordx4.  The 4 * nst stages of a patch form
+// one pipeline that runs across the row boundaries, through a ring of RING LDS
+// stages with RING-1 of them in flight: the operands of a stage come from HBM or a
+// remote L2 slice and need longer than one stage of MFMAs to arrive (a 3-deep ring
+// measured 7-17 % faster than double buffering with 2-byte operands, a 4-deep one
+// 2-4 % with fp32).  The ring slot is a compile-time index (loop unrolled RING
+// times, remainder peeled) and every slot is an array of its own, so the compiler
+// can tell the slot being filled from the one being read.  The stage barrier is a
+// bare s_barrier: __syncthreads() carries a release fence for which the compiler
+// drains every pending direct-to-LDS load.
 // =============================================================================
-template <typename T, bool SWAP, int NVG>
+template <typename T, bool SWAP, int NVG, int RING>
 __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__ U, const T* __restrict__ V,
-                                                           T* __restrict__ y, ActStrides ys, int N, int K, int Ho,
-                                                           int Wo, int th, int tw, long P, int Cp, int Kp, long Pp,
-                                                           int order, Epilogue ep, int kTiles, int pTiles) {
+                                                                T* __restrict__ y, ActStrides ys, int N, int K,
+                                                                int Ho, int Wo, int th, int tw, long P, int Cp,
+                                                                int Kp, long Pp, int order, Epilogue ep, int kTiles,
+                                                                int pTiles) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
-    constexpr int NV = 2 * NVG;                     // channel vectors per stage and coordinate
-    __shared__ vec Us0[4][NV][GO_T], Us1[4][NV][GO_T];
-    __shared__ vec Vs0[4][NV][GO_T], Vs1[4][NV][GO_T];
+    constexpr int NV = 2 * NVG;
+    static_assert(RING == 3 || RING == 4, "ring depth");
+    __shared__ vec Us0[4][NV][GO_T], Us1[4][NV][GO_T], Us2[4][NV][GO_T], Us3[RING > 3 ? 4 : 1][NV][GO_T];
+    __shared__ vec Vs0[4][NV][GO_T], Vs1[4][NV][GO_T], Vs2[4][NV][GO_T], Vs3[RING > 3 ? 4 : 1][NV][GO_T];
+    auto uslot = [&](auto sl) -> vec(*)[NV][GO_T] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return Us0; else if constexpr (S == 1) return Us1; else if constexpr (S == 2) return Us2; else return Us3;
+    };
+    auto vslot = [&](auto sl) -> vec(*)[NV][GO_T] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return Vs0; else if constexpr (S == 1) return Vs1; else if constexpr (S == 2) return Vs2; else return Vs3;
+    };
 
     const int b = blockIdx.x;
     const int xcd = b & 7, jb = b >> 3;
@@ -437,46 +460,39 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     const int k0 = ktile * GO_T;
     const long p0 = (long)ptile * GO_T;
     const int CQ = Cp / CV;
-    const int nst = CQ / NV;                        // stages per row (even)
+    const int nst = CQ / NV;
+    const int total = 4 * nst;
     const vec* Ug = reinterpret_cast<const vec*>(U);
     const vec* Vg = reinterpret_cast<const vec*>(V);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    floatx16 acc[4];
-    floatx16 yo[4];                                  // y00, y01, y10, y11
+    floatx16 acc[4], yo[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { acc[j][r] = 0.f; yo[j][r] = 0.f; }
 
-    typedef std::integral_constant<int, 0> par0_t;
-    typedef std::integral_constant<int, 1> par1_t;
-    // a stage is 8*NV rows of 64 vectors (4 coordinates x NV vectors, U and V); wave w issues rows w, w+4, ...
-    // Row r of a stage is (operand, coordinate j of the row, vector v); its address advances by NV
-    // vectors per stage and by NV + 3*CQ vectors when the Winograd row changes.
     const unsigned lane_off = lane * 16;
     uint64_t sptr[2 * NV];
     const uint64_t stepU = (uint64_t)NV * Kp * 16, wrapU = (uint64_t)(NV + 3 * CQ) * Kp * 16;
     const uint64_t stepV = (uint64_t)NV * Pp * 16, wrapV = (uint64_t)(NV + 3 * CQ) * Pp * 16;
 #pragma unroll
     for (int q = 0; q < 2 * NV; ++q) {
-        const int r = wave + 4 * q;                  // 0 .. 8*NV-1, wave-uniform
-        const int opnd = q / NV;                     // 0: U, 1: V  (= r / (4*NV), known at compile time)
+        const int r = wave + 4 * q;
+        const int opnd = q / NV;
         const int j = (r / NV) & 3, v = r % NV;
         const size_t cvec = (size_t)j * CQ + v;
         sptr[q] = opnd ? reinterpret_cast<uint64_t>(Vg + cvec * Pp + p0) : reinterpret_cast<uint64_t>(Ug + cvec * Kp + k0);
     }
-    const int total = 4 * nst;
-    int issued = 0, in_row = 0;                      // stages requested so far, and of the current row
-    auto stage_load = [&](auto par) {
-        constexpr int S = decltype(par)::value;
+    int issued = 0, in_row = 0;
+    auto stage_load = [&](auto sl) {
         ++issued;
-        const bool wrap = ++in_row == nst, last = issued >= total;   // past the end: the last stage again (never read)
+        const bool wrap = ++in_row == nst, last = issued >= total;
         if (wrap) in_row = 0;
         const uint64_t incU = last ? 0 : (wrap ? wrapU : stepU), incV = last ? 0 : (wrap ? wrapV : stepV);
 #pragma unroll
@@ -484,52 +500,47 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
             const int r = wave + 4 * q;
             const int opnd = q / NV;
             const int j = (r / NV) & 3, v = r % NV;
-            vec* dst = opnd ? (S ? &Vs1[j][v][0] : &Vs0[j][v][0]) : (S ? &Us1[j][v][0] : &Us0[j][v][0]);
-            dma_row(sptr[q], lane_off, dst);
+            dma_row(sptr[q], lane_off, opnd ? &vslot(sl)[j][v][0] : &uslot(sl)[j][v][0]);
             sptr[q] += opnd ? incV : incU;
         }
     };
-    // first: the stage opens a row, its MFMAs start from a zero accumulator (an inline constant,
-    // instead of 64 register clears per row)
-    auto iteration = [&](auto par, auto first) {
-        constexpr int S = decltype(par)::value;
-        constexpr bool FIRST = decltype(first)::value;
-        stage_load(std::integral_constant<int, 1 - S>{});
+    constexpr int LPW = 2 * NV;                       // loads per wave and stage
+    constexpr int WV = (RING - 2) * LPW;              // the newest RING-2 stages may still be in flight
+    constexpr int WAIT_IMM = (WV & 0xF) | (0x7 << 4) | (0xF << 8) | ((WV >> 4) << 14);
+    int row = 0, cst = 0;                             // Winograd row and stage of it being multiplied
+    auto iteration = [&](auto sl) {
+        constexpr int S = decltype(sl)::value;
+        __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+        __builtin_amdgcn_s_barrier();                 // stage S landed for every wave; slot S-1 is free
+        asm volatile("" ::: "memory");
+        stage_load(std::integral_constant<int, (S + RING - 1) % RING>{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < NVG; ++g)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const vec fu = S ? Us1[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32] : Us0[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32];
-                const vec fv = S ? Vs1[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32] : Vs0[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32];
-                if (FIRST && g == 0) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
-                }
+                const vec fu = uslot(sl)[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32];
+                const vec fv = vslot(sl)[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32];
                 if (SWAP) Mma<T>::run(fv, fu, acc[j]);
                 else Mma<T>::run(fu, fv, acc[j]);
             }
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's rows of the next stage are in LDS
-        __syncthreads();
+        if (++cst == nst) {
+            cst = 0;
+            rows_fold<true>(acc, yo, row);
+            ++row;
+        }
     };
 
-    stage_load(par0_t{});
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-
-    for (int i = 0; i < 4; ++i) {
-        iteration(par0_t{}, std::true_type{});
-        iteration(par1_t{}, std::false_type{});
-        for (int st = 2; st < nst; st += 2) {
-            iteration(par0_t{}, std::false_type{});
-            iteration(par1_t{}, std::false_type{});
-        }
-        rows_fold<false>(acc, yo, i);
-    }
-
+    for_each_const(std::make_integer_sequence<int, RING - 1>{}, stage_load);
+    int s = 0;
+    for (; s + RING <= total; s += RING) for_each_const(std::make_integer_sequence<int, RING>{}, iteration);
+    // total = 4*nst is even; with RING = 3 up to two stages remain, in slots 0 and 1; with RING = 4 none or two
+    if (s < total) iteration(std::integral_constant<int, 0>{});
+    if (s + 1 < total) iteration(std::integral_constant<int, 1>{});
+    if (RING == 4 && s + 2 < total) iteration(std::integral_constant<int, 2>{});
+    __builtin_amdgcn_s_waitcnt(0x0F70);               // the surplus requests of the last stages
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);
 }
-
 
 }  // namespace wino

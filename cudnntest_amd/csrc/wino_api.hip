@@ -247,14 +247,14 @@ int launch_gemm(int nxi, int dtype, int porder, int Cp, int Kp, long Pp, const v
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
-template <typename T, bool SWAP, int NVG>
-int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geometry& g, const void* U, const void* V,
-                       void* y, int dst, hipStream_t st) {
+template <typename T, bool SWAP, int NVG, int RING>
+int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
+                            const void* V, void* y, int dst, hipStream_t st) {
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
     dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
-    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG>), grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
+    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING>), grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
                        out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
                        g.Pp, order, make_epilogue(flags, bias), kTiles, pTiles);
     LAUNCH_CHECK("gemm_rows");
@@ -264,15 +264,10 @@ int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geomet
 template <typename T>
 int launch_gemm_rows_d(int dst, int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
                        const void* V, void* y, hipStream_t st) {
-    constexpr int CV = ChanVec<T>::n;
-    // stages per row must be even: one k-group per stage always is (Cp is a multiple of 4 channel
-    // vectors); two k-groups per stage (fewer barriers, measured faster) when Cp allows it
-    const bool two = (g.Cp / CV) % 8 == 0 && !getenv("WINO_ROWS_ONE");
-    if (dst == WINO_NHWC)
-        return two ? launch_gemm_rows_t<T, true, 2>(order, flags, bias, g, U, V, y, dst, st)
-                   : launch_gemm_rows_t<T, true, 1>(order, flags, bias, g, U, V, y, dst, st);
-    return two ? launch_gemm_rows_t<T, false, 2>(order, flags, bias, g, U, V, y, dst, st)
-               : launch_gemm_rows_t<T, false, 1>(order, flags, bias, g, U, V, y, dst, st);
+    // one k-group per stage; ring depth from measurements: 3 for 2-byte operands, 4 for fp32
+    constexpr int RING = sizeof(T) == 2 ? 3 : 4;
+    if (dst == WINO_NHWC) return launch_gemm_rows_t<T, true, 1, RING>(order, flags, bias, g, U, V, y, dst, st);
+    return launch_gemm_rows_t<T, false, 1, RING>(order, flags, bias, g, U, V, y, dst, st);
 }
 
 int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
@@ -403,21 +398,21 @@ int tile_order_for(int src, int /*dst*/) {
 // Chosen from sweeps of the VGG-16 shapes over the three algorithms, per layout and element type.
 int pick_algo(int layout, int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
-    if (patches < 512) return WINO_ALGO_STAGED;          // too few 64x64 patches to fill 256 CUs
     const bool nhwc = layout == WINO_NHWC;
     if (dtype == WINO_F32) {
+        if (patches < 512) return WINO_ALGO_STAGED;      // too few 64x64 patches to fill 256 CUs
         // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
         if (g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
-        if (g.C <= 256 && g.K <= 256) return nhwc ? WINO_ALGO_FUSED : WINO_ALGO_EPILOGUE;
-        return WINO_ALGO_STAGED;      // the 128x128 GEMM's lower L2 traffic per flop wins
+        if (g.C <= 256) return WINO_ALGO_EPILOGUE;
+        // many channels: the 128x128 GEMM's lower L2 traffic per flop wins unless there are few tiles
+        return g.P <= 4096 ? WINO_ALGO_EPILOGUE : WINO_ALGO_STAGED;
     }
-    // 16-bit operands: the fp32 product tensor is the largest HBM stream, so never STAGED; the in-kernel
-    // input transform is VALU work repeated per filter tile and pays only with few filter tiles and
-    // cheap loads (channel vectors for NHWC, which need C % 8 == 0; coalesced elements for CHWN)
+    // 16-bit operands: the fp32 product tensor is the largest HBM stream, so STAGED only for tiny problems;
+    // the in-kernel input transform is VALU work repeated per filter tile and pays only with few filter
+    // tiles and cheap loads (channel vectors for NHWC, which need C % 8 == 0)
+    if (patches < 64) return WINO_ALGO_STAGED;
     if (nhwc) {
-        if (g.C >= 16 && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
-    } else if (layout == WINO_CHWN) {
-        if (g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
+        if (g.C >= 16 && g.C <= 128 && g.K <= 128 && (g.K <= 64 || g.C >= 128)) return WINO_ALGO_FUSED;
     } else if (g.C <= 64 && g.K <= 64) {
         return WINO_ALGO_FUSED;
     }
