@@ -59,252 +59,8 @@ __device__ __forceinline__ void dma_row(uint64_t sbase, unsigned lane_off, void*
                                      (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
 }
 
-// =============================================================================
-// Plain batched GEMM, product written to HBM as Mo[xi][Kp][Pp] (fp32).
-//
-// Block tile 128 filters x 128 tiles, 4 waves in a 2x2 arrangement, each wave
-// 64x64 = 2x2 MFMA tiles.  The reduction is consumed NV channel vectors at a
-// time from two LDS stages; the next slab travels HBM -> LDS directly
-// (global_load_lds_dwordx4: one instruction moves 64 channel vectors = 1 KB,
-// lane l to LDS row base + 16*l) while the current one feeds the MFMAs.  No
-// staging registers, no LDS store instructions; one wait + barrier per slab.
-// =============================================================================
 constexpr int GEMM_BM = 128, GEMM_BN = 128;
 
-// PK = false: product stored as Mo[xi][Kp][Pp] (MFMA rows = filters, lanes = tiles)
-// PK = true : product stored as Mo[xi][Pp][Kp] (MFMA rows = tiles, lanes = filters), for
-//             destinations whose contiguous axis is K (NHWC)
-template <typename T, int NV, bool PK>
-__global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__ U, const T* __restrict__ V,
-                                                            float* __restrict__ Mo, int Cp, int Kp, long Pp,
-                                                            int kTiles, int pTiles) {
-    typedef typename Mma<T>::vec vec;
-    constexpr int CV = ChanVec<T>::n;
-    // separate arrays per stage so the compiler can tell the stage being filled from the one being read
-    __shared__ vec As0[NV][GEMM_BM], As1[NV][GEMM_BM];
-    __shared__ vec Bs0[NV][GEMM_BN], Bs1[NV][GEMM_BN];
-
-    // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so the
-    // ids that share an XCD walk the filter tiles of one tile column first and the V slab
-    // they share is fetched from HBM once, into that XCD's L2.
-    const int xi = blockIdx.y;
-    const int b = blockIdx.x;
-    const int xcd = b & 7, jj = b >> 3;
-    const int ktile = jj % kTiles;
-    const int ptile = (jj / kTiles) * 8 + xcd;
-    if (ptile >= pTiles) return;
-    const long p0 = (long)ptile * GEMM_BN;
-    const int k0 = ktile * GEMM_BM;
-    const int CQ = Cp / CV;
-    const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
-    const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
-    const int wm = wave >> 1, wn = wave & 1;
-    const int l32 = lane & 31, lh = lane >> 5;
-
-    floatx16 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    typedef std::integral_constant<int, 0> par0_t;
-    typedef std::integral_constant<int, 1> par1_t;
-    // a stage is 2*NV rows of 128 vectors = 4*NV pieces of 64 vectors; wave w issues pieces w, w+4, ...
-    auto stage_load = [&](auto par, int ch) {
-        constexpr int S = decltype(par)::value;
-        const int q0 = ch * NV;
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int piece = wave + 4 * i;              // 0 .. 4*NV-1, wave-uniform
-            const int opnd = piece / (2 * NV);           // 0: U, 1: V
-            const int row = (piece >> 1) % NV, half = piece & 1;
-            const vec* src = opnd ? Vb + (size_t)(q0 + row) * Pp + half * 64 + lane
-                                  : Ub + (size_t)(q0 + row) * Kp + half * 64 + lane;
-            vec* dst = opnd ? (S ? &Bs1[row][half * 64] : &Bs0[row][half * 64])
-                            : (S ? &As1[row][half * 64] : &As0[row][half * 64]);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-        }
-    };
-    const int nch = CQ / NV;
-    auto iteration = [&](auto par, int ch) {
-        constexpr int S = decltype(par)::value;
-        stage_load(std::integral_constant<int, 1 - S>{}, ch + 1 < nch ? ch + 1 : ch);   // surplus load never read
-        // fence: without it the compiler sinks the loads to the end of the slab, right before the wait
-        __builtin_amdgcn_sched_barrier(0);
-        vec a[2][2], b[2][2];                      // fragments of k-group g live in set g&1, fetched one group ahead
-        auto frag_load = [&](int g) {
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const vec fa = S ? As1[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32]
-                                 : As0[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32];
-                const vec fb = S ? Bs1[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32]
-                                 : Bs0[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32];
-                a[g & 1][q] = PK ? fb : fa;
-                b[g & 1][q] = PK ? fa : fb;
-            }
-        };
-        frag_load(0);
-#pragma unroll
-        for (int g = 0; g < NV / 2; ++g) {
-            if (g + 1 < NV / 2) frag_load(g + 1);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) Mma<T>::run(a[g & 1][i], b[g & 1][j], acc[i][j]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's pieces of the next stage are in LDS
-        __syncthreads();
-    };
-
-    stage_load(par0_t{}, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    int ch = 0;
-    for (; ch + 1 < nch; ch += 2) {
-        iteration(par0_t{}, ch);
-        iteration(par1_t{}, ch + 1);
-    }
-    if (ch < nch) iteration(par0_t{}, ch);
-
-    float* Mb = Mo + (size_t)xi * Kp * Pp;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ri = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);   // MFMA row
-                const int ci = wn * 64 + j * 32 + l32;                               // MFMA column (lane)
-                if (PK) Mb[(size_t)(p0 + ri) * Kp + k0 + ci] = acc[i][j][r];
-                else Mb[(size_t)(k0 + ri) * Pp + p0 + ci] = acc[i][j][r];
-            }
-}
-
-// Register-staged variant of the same tile: the next slab travels HBM -> registers while the
-// current one feeds the MFMAs, then registers -> the other LDS buffer.  Measured faster than the
-// direct-to-LDS version for fp32 (115 vs 106 TFLOP/s on N=32, C=K=256, H=56: LDS writes of the
-// in-flight DMA compete with the fragment reads of the long fp32 MFMAs), slower for 16-bit
-// operands (257 vs 355 TFLOP/s), so fp32 uses this one.
-template <typename T, int NV, bool PK>
-__global__ __launch_bounds__(256) void gemm_128x128_reg_kernel(const T* __restrict__ U, const T* __restrict__ V,
-                                                            float* __restrict__ Mo, int Cp, int Kp, long Pp,
-                                                            int kTiles, int pTiles) {
-    typedef typename Mma<T>::vec vec;
-    constexpr int CV = ChanVec<T>::n;
-    __shared__ vec As[2][NV][GEMM_BM];
-    __shared__ vec Bs[2][NV][GEMM_BN];
-
-    // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so the
-    // ids that share an XCD walk the filter tiles of one tile column first and the V slab
-    // they share is fetched from HBM once, into that XCD's L2.
-    const int xi = blockIdx.y;
-    const int b = blockIdx.x;
-    const int xcd = b & 7, jj = b >> 3;
-    const int ktile = jj % kTiles;
-    const int ptile = (jj / kTiles) * 8 + xcd;
-    if (ptile >= pTiles) return;
-    const long p0 = (long)ptile * GEMM_BN;
-    const int k0 = ktile * GEMM_BM;
-    const int CQ = Cp / CV;
-    const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
-    const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so addresses built from it stay on the scalar unit
-    const int wm = wave >> 1, wn = wave & 1;
-    const int l32 = lane & 31, lh = lane >> 5;
-    const int lrow = tid >> 7, lcol = tid & 127;   // rows lrow + 2*h
-
-    floatx16 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    vec ra[NV / 2], rb[NV / 2];
-    auto gload = [&](int ch) {
-        const int q0 = ch * NV;
-#pragma unroll
-        for (int h = 0; h < NV / 2; ++h) {
-            ra[h] = Ub[(size_t)(q0 + lrow + 2 * h) * Kp + lcol];
-            rb[h] = Vb[(size_t)(q0 + lrow + 2 * h) * Pp + lcol];
-        }
-    };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int h = 0; h < NV / 2; ++h) {
-            As[buf][lrow + 2 * h][lcol] = ra[h];
-            Bs[buf][lrow + 2 * h][lcol] = rb[h];
-        }
-    };
-
-    const int nch = CQ / NV;
-    gload(0);
-    lstore(0);
-    __syncthreads();
-
-    for (int ch = 0; ch < nch; ++ch) {
-        const int buf = ch & 1;
-        if (ch + 1 < nch) gload(ch + 1);
-#pragma unroll
-        for (int g = 0; g < NV / 2; ++g) {
-            vec a[2], b[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (PK) {
-                    a[t] = Bs[buf][2 * g + lh][wm * 64 + t * 32 + l32];
-                    b[t] = As[buf][2 * g + lh][wn * 64 + t * 32 + l32];
-                } else {
-                    a[t] = As[buf][2 * g + lh][wm * 64 + t * 32 + l32];
-                    b[t] = Bs[buf][2 * g + lh][wn * 64 + t * 32 + l32];
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) Mma<T>::run(a[i], b[j], acc[i][j]);
-        }
-        if (ch + 1 < nch) lstore(buf ^ 1);
-        __syncthreads();
-    }
-
-    float* Mb = Mo + (size_t)xi * Kp * Pp;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ri = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);   // MFMA row
-                const int ci = wn * 64 + j * 32 + l32;                               // MFMA column (lane)
-                if (PK) Mb[(size_t)(p0 + ri) * Kp + k0 + ci] = acc[i][j][r];
-                else Mb[(size_t)(k0 + ri) * Pp + p0 + ci] = acc[i][j][r];
-            }
-}
-
-// =============================================================================
-// Shared pieces of the kernels that apply the output transform in registers
-// (patch = 64 filters x 64 tiles per workgroup, 4 waves of 32x32 MFMA tiles).
-//
-// SWAP = false: MFMA rows = filters, lanes = tiles  (stores contiguous along the
-//               tile axis: NCHW, or CHWN with batch-minor tiles)
-// SWAP = true : MFMA rows = tiles, lanes = filters  (stores contiguous along K: NHWC)
-//
-// Workgroup -> patch mapping is XCD-aware: consecutive workgroup ids go to the
-// 8 XCDs round-robin, so the ids that land on one XCD walk the filter tiles of
-// one tile patch first; the V slab they share then stays in that XCD's L2.
-// =============================================================================
 constexpr int GO_T = 64;   // patch edge (filters and tiles)
 
 // The 2x2 outputs of tile (n, ty, tx), filter k.  pair: the destination is W-contiguous with even
@@ -541,6 +297,146 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     if (RING == 4 && s + 2 < total) iteration(std::integral_constant<int, 2>{});
     __builtin_amdgcn_s_waitcnt(0x0F70);               // the surplus requests of the last stages
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);
+}
+
+// =============================================================================
+// Plain batched GEMM, product written to HBM as Mo[xi][Kp][Pp] (fp32).
+//
+// Block tile 128 filters x 128 tiles, 4 waves in a 2x2 arrangement, each wave
+// 64x64 = 2x2 MFMA tiles.  The reduction is consumed NV channel vectors at a
+// time from a ring of RING LDS stages; the stages travel HBM -> LDS directly
+// (global_load_lds_dwordx4: one instruction moves 64 channel vectors = 1 KB,
+// lane l to LDS row base + 16*l), RING-1 of them in flight, from running scalar
+// addresses; no staging registers, no LDS store instructions; one wait and one
+// bare s_barrier per stage (the pipeline of gemm_rows_kernel).  Measured: 4 deep
+// for fp32 (1-5 % faster than register-staged double buffering), 2 deep for 2-byte
+// operands (deeper rings are slower there: the fp32 product store bounds the kernel).
+//
+// XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so
+// the ids that share an XCD walk the filter tiles of one tile column first and the
+// V slab they share is fetched from HBM once, into that XCD's L2.
+//
+// PK = false: product stored as Mo[xi][Kp][Pp] (MFMA rows = filters, lanes = tiles)
+// PK = true : product stored as Mo[xi][Pp][Kp] (MFMA rows = tiles, lanes = filters), for
+//             destinations whose contiguous axis is K (NHWC)
+// =============================================================================
+template <typename T, int NV, bool PK, int RING>
+__global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                                float* __restrict__ Mo, int Cp, int Kp, long Pp,
+                                                                int kTiles, int pTiles) {
+    typedef typename Mma<T>::vec vec;
+    constexpr int CV = ChanVec<T>::n;
+    static_assert(RING >= 2 && RING <= 4, "ring depth");
+    __shared__ vec As0[NV][GEMM_BM], As1[NV][GEMM_BM], As2[RING > 2 ? NV : 1][GEMM_BM], As3[RING > 3 ? NV : 1][GEMM_BM];
+    __shared__ vec Bs0[NV][GEMM_BN], Bs1[NV][GEMM_BN], Bs2[RING > 2 ? NV : 1][GEMM_BN], Bs3[RING > 3 ? NV : 1][GEMM_BN];
+    auto aslot = [&](auto sl) -> vec(*)[GEMM_BM] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return As0; else if constexpr (S == 1) return As1; else if constexpr (S == 2) return As2; else return As3;
+    };
+    auto bslot = [&](auto sl) -> vec(*)[GEMM_BN] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return Bs0; else if constexpr (S == 1) return Bs1; else if constexpr (S == 2) return Bs2; else return Bs3;
+    };
+    const int xi = blockIdx.y;
+    const int b = blockIdx.x;
+    const int xcd = b & 7, jj = b >> 3;
+    const int ktile = jj % kTiles;
+    const int ptile = (jj / kTiles) * 8 + xcd;
+    if (ptile >= pTiles) return;
+    const long p0 = (long)ptile * GEMM_BN;
+    const int k0 = ktile * GEMM_BM;
+    const int CQ = Cp / CV;
+    const int nch = CQ / NV;
+    const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
+    const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // a stage is 2*NV rows of 128 vectors = 4*NV pieces of 64 vectors; wave w issues pieces w, w+4, ...
+    const unsigned lane_off = lane * 16;
+    uint64_t sptr[NV];
+    const uint64_t stepU = (uint64_t)NV * Kp * 16, stepV = (uint64_t)NV * Pp * 16;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int piece = wave + 4 * i;
+        const int opnd = i / (NV / 2);               // = piece / (2*NV), known at compile time
+        const int row = (piece >> 1) % NV, half = piece & 1;
+        sptr[i] = opnd ? reinterpret_cast<uint64_t>(Vb + (size_t)row * Pp + half * 64)
+                       : reinterpret_cast<uint64_t>(Ub + (size_t)row * Kp + half * 64);
+    }
+    int issued = 0;
+    auto stage_load = [&](auto sl) {
+        const bool last = ++issued >= nch;           // past the end: the last stage again (never read)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int piece = wave + 4 * i;
+            const int opnd = i / (NV / 2);
+            const int row = (piece >> 1) % NV, half = piece & 1;
+            dma_row(sptr[i], lane_off, opnd ? &bslot(sl)[row][half * 64] : &aslot(sl)[row][half * 64]);
+            sptr[i] += last ? 0 : (opnd ? stepV : stepU);
+        }
+    };
+    constexpr int WV = (RING - 2) * NV;
+    constexpr int WAIT_IMM = (WV & 0xF) | (0x7 << 4) | (0xF << 8) | ((WV >> 4) << 14);
+    auto iteration = [&](auto sl) {
+        __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        stage_load(std::integral_constant<int, (decltype(sl)::value + RING - 1) % RING>{});
+        __builtin_amdgcn_sched_barrier(0);
+        vec a[2][2], bq[2][2];
+        auto frag_load = [&](int g) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const vec fa = aslot(sl)[2 * g + lh][(PK ? wn : wm) * 64 + q * 32 + l32];
+                const vec fb = bslot(sl)[2 * g + lh][(PK ? wm : wn) * 64 + q * 32 + l32];
+                a[g & 1][q] = PK ? fb : fa;
+                bq[g & 1][q] = PK ? fa : fb;
+            }
+        };
+        frag_load(0);
+#pragma unroll
+        for (int g = 0; g < NV / 2; ++g) {
+            if (g + 1 < NV / 2) frag_load(g + 1);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) Mma<T>::run(a[g & 1][i], bq[g & 1][j], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for_each_const(std::make_integer_sequence<int, RING - 1>{}, stage_load);
+    int s = 0;
+    for (; s + RING <= nch; s += RING) for_each_const(std::make_integer_sequence<int, RING>{}, iteration);
+    if (s < nch) iteration(std::integral_constant<int, 0>{});
+    if (s + 1 < nch) iteration(std::integral_constant<int, 1>{});
+    if (RING > 3 && s + 2 < nch) iteration(std::integral_constant<int, 2>{});
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+    float* Mb = Mo + (size_t)xi * Kp * Pp;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ri = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);   // MFMA row
+                const int ci = wn * 64 + j * 32 + l32;                               // MFMA column (lane)
+                if (PK) Mb[(size_t)(p0 + ri) * Kp + k0 + ci] = acc[i][j][r];
+                else Mb[(size_t)(k0 + ri) * Pp + p0 + ci] = acc[i][j][r];
+            }
 }
 
 }  // namespace wino

@@ -219,12 +219,9 @@ template <typename T, int NV, bool PK>
 int launch_gemm_t(int nxi, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
     const int kTiles = Kp / GEMM_BM, pTiles = (int)(Pp / GEMM_BN);
     dim3 grid((unsigned)((pTiles + 7) / 8 * 8 * kTiles), nxi), block(256);
-    if (sizeof(T) == 4)
-        hipLaunchKernelGGL((gemm_128x128_reg_kernel<T, NV, PK>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp,
-                           Kp, Pp, kTiles, pTiles);
-    else
-        hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp, Kp,
-                           Pp, kTiles, pTiles);
+    constexpr int RING = sizeof(T) == 4 ? 4 : 2;     // from measurements, see gemm.hpp
+    hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK, RING>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp,
+                       Kp, Pp, kTiles, pTiles);
     LAUNCH_CHECK("batched_gemm");
     return WINO_OK;
 }
