@@ -186,13 +186,19 @@ template <int... S, class F> __device__ __forceinline__ void for_each_const(std:
 // can tell the slot being filled from the one being read.  The stage barrier is a
 // bare s_barrier: __syncthreads() carries a release fence for which the compiler
 // drains every pending direct-to-LDS load.
+//
+// A workgroup alone on its CU needs the MFMA time of a whole patch (55 us for C = 256 in fp32),
+// and that is what a last round of a few workgroups costs while the other CUs idle.  The host
+// therefore launches the patches of a small last round through the TAIL variant: four workgroups
+// per patch, one Winograd row each, combined by the last one to arrive.
 // =============================================================================
-template <typename T, bool SWAP, int NVG, int RING>
+template <typename T, bool SWAP, int NVG, int RING, bool TAIL>
 __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__ U, const T* __restrict__ V,
-                                                                T* __restrict__ y, ActStrides ys, int N, int K,
-                                                                int Ho, int Wo, int th, int tw, long P, int Cp,
-                                                                int Kp, long Pp, int order, Epilogue ep, int kTiles,
-                                                                int pTiles) {
+                                                           T* __restrict__ y, ActStrides ys, int N, int K,
+                                                           int Ho, int Wo, int th, int tw, long P, int Cp,
+                                                           int Kp, long Pp, int order, Epilogue ep, int kTiles,
+                                                           int pTiles, int first_id, float* __restrict__ tail_part,
+                                                           int* __restrict__ tail_cnt) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     constexpr int NV = 2 * NVG;
@@ -208,7 +214,13 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         if constexpr (S == 0) return Vs0; else if constexpr (S == 1) return Vs1; else if constexpr (S == 2) return Vs2; else return Vs3;
     };
 
-    const int b = blockIdx.x;
+    // TAIL: the patches of the last, partly filled round of workgroups are cut four ways -- one
+    // Winograd row per workgroup (a quarter of the reduction) -- so the whole chip works on them
+    // instead of a few CUs; tq = patch of the tail, trow = its row.  The four workgroups of a patch
+    // have ids 8 apart: the same XCD.
+    const int tq = TAIL ? ((int)blockIdx.x >> 5) * 8 + ((int)blockIdx.x & 7) : 0;
+    const int trow = TAIL ? ((int)blockIdx.x >> 3) & 3 : 0;
+    const int b = TAIL ? first_id + tq : (int)blockIdx.x;
     const int xcd = b & 7, jb = b >> 3;
     const int ktile = jb % kTiles;
     const int ptile = (jb / kTiles) * 8 + xcd;
@@ -217,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     const long p0 = (long)ptile * GO_T;
     const int CQ = Cp / CV;
     const int nst = CQ / NV;
-    const int total = 4 * nst;
+    const int total = TAIL ? nst : 4 * nst;
     const vec* Ug = reinterpret_cast<const vec*>(U);
     const vec* Vg = reinterpret_cast<const vec*>(V);
 
@@ -242,7 +254,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         const int r = wave + 4 * q;
         const int opnd = q / NV;
         const int j = (r / NV) & 3, v = r % NV;
-        const size_t cvec = (size_t)j * CQ + v;
+        const size_t cvec = (size_t)(4 * trow + j) * CQ + v;
         sptr[q] = opnd ? reinterpret_cast<uint64_t>(Vg + cvec * Pp + p0) : reinterpret_cast<uint64_t>(Ug + cvec * Kp + k0);
     }
     int issued = 0, in_row = 0;
@@ -263,7 +275,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     constexpr int LPW = 2 * NV;                       // loads per wave and stage
     constexpr int WV = (RING - 2) * LPW;              // the newest RING-2 stages may still be in flight
     constexpr int WAIT_IMM = (WV & 0xF) | (0x7 << 4) | (0xF << 8) | ((WV >> 4) << 14);
-    int row = 0, cst = 0;                             // Winograd row and stage of it being multiplied
+    int row = trow, cst = 0;                          // Winograd row and stage of it being multiplied
     auto iteration = [&](auto sl) {
         constexpr int S = decltype(sl)::value;
         __builtin_amdgcn_s_waitcnt(WAIT_IMM);
@@ -296,6 +308,35 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     if (s + 1 < total) iteration(std::integral_constant<int, 1>{});
     if (RING == 4 && s + 2 < total) iteration(std::integral_constant<int, 2>{});
     __builtin_amdgcn_s_waitcnt(0x0F70);               // the surplus requests of the last stages
+    if (TAIL) {
+        // Every workgroup leaves its row's contribution in tail_part[patch][row][register][thread]; the
+        // one that arrives last (a counter per patch, returned to zero for the next launch) adds the four
+        // rows in the order 0..3 -- so the result does not depend on who was last -- and stores the patch.
+        float* mine = tail_part + ((size_t)(tq * 4 + trow) * 64) * 256 + tid;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mine[(a * 16 + r) * 256] = yo[a][r];
+        __shared__ int s_last;
+        __threadfence();                              // this workgroup's partial sums, visible to the device
+        __syncthreads();
+        if (tid == 0) {
+            const int old = atomicAdd(&tail_cnt[tq], 1);
+            s_last = old == 3;
+            if (old == 3) tail_cnt[tq] = 0;
+        }
+        __syncthreads();
+        if (!s_last) return;
+        __threadfence();                              // the other workgroups' partial sums
+        const float* all = tail_part + ((size_t)(tq * 4) * 64) * 256 + tid;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float* e = all + (a * 16 + r) * 256;
+                yo[a][r] = ((e[0] + e[64 * 256]) + e[2 * 64 * 256]) + e[3 * 64 * 256];
+            }
+    }
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);
 }
 

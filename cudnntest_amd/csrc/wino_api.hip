@@ -54,6 +54,7 @@ struct Arena {
     void* ext = nullptr;
     size_t ext_bytes = 0;
 };
+constexpr size_t kCounterBytes = 4096;     // 1024 arrival counters at the head of every arena
 Arena g_arena[kMaxDevices];
 std::mutex g_arena_mu;
 
@@ -78,6 +79,7 @@ int arena_get(size_t bytes, void** out) {
         }
         HIP_TRY(hipMalloc(&a.own, bytes));
         a.own_bytes = bytes;
+        HIP_TRY(hipMemset(a.own, 0, kCounterBytes));       // arrival counters: zero between launches
     }
     *out = a.own;
     return WINO_OK;
@@ -115,13 +117,16 @@ struct Scratch {
     size_t u_off, v_off, m_off, total;
 };
 
+// The arena opens with the arrival counters of the epilogue GEMM's tail workgroups (zero whenever no
+// kernel is running); U, V and the product follow.  The product region doubles as the tail workgroups'
+// partial sums: the epilogue path has no product tensor.
 Scratch scratch_layout(const Geometry& g, int dtype) {
     const size_t es = dtype_size(dtype);
     const size_t nxi = (size_t)(g.m + 2) * (g.m + 2);
     auto al = [](size_t v) { return (v + 255) / 256 * 256; };
     Scratch s;
-    s.u_off = 0;
-    s.v_off = al(nxi * (size_t)g.Cp * g.Kp * es);
+    s.u_off = kCounterBytes;
+    s.v_off = s.u_off + al(nxi * (size_t)g.Cp * g.Kp * es);
     s.m_off = s.v_off + al(nxi * (size_t)g.Cp * g.Pp * es);
     s.total = s.m_off + al(nxi * (size_t)g.Kp * g.Pp * sizeof(float));
     return s;
@@ -244,35 +249,64 @@ int launch_gemm(int nxi, int dtype, int porder, int Cp, int Kp, long Pp, const v
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
+// tail: scratch for the cut-up last round (partial sums, arrival counters), or null to launch every patch whole
+struct TailScratch {
+    float* part = nullptr;
+    size_t part_bytes = 0;
+    int* cnt = nullptr;
+};
+
 template <typename T, bool SWAP, int NVG, int RING>
 int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
-                            const void* V, void* y, int dst, hipStream_t st) {
+                       const void* V, void* y, int dst, const TailScratch& ts, hipStream_t st) {
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
-    dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
-    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING>), grid, block, 0, st, (const T*)U, (const T*)V, (T*)y,
-                       out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo), g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp,
-                       g.Pp, order, make_epilogue(flags, bias), kTiles, pTiles);
+    const int group = 8 * kTiles;                         // workgroup ids per group of 8 tile patches
+    const ActStrides ys = out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo);
+    const Epilogue ep = make_epilogue(flags, bias);
+    // Workgroups resident at once: 256 CUs x 2 (64 KB of LDS, fp32) or x 3 (48 KB, 2-byte operands).  If the
+    // last round would occupy at most a quarter of them, its patches go to the TAIL variant.
+    const long slots = 256L * (sizeof(T) == 2 ? 3 : 2);
+    const long real = (long)pTiles * kTiles;
+    int tail_groups = 0;
+    if (ts.part && real > slots && real % slots != 0 && 4 * (real % slots) <= slots) {
+        tail_groups = (int)((real % slots + group - 1) / group);
+        const long tail_ids = (long)tail_groups * group;
+        if (tail_groups >= pGroups || 4 * tail_ids > slots || tail_ids > (long)(kCounterBytes / sizeof(int)) ||
+            (size_t)tail_ids * 4 * 64 * 256 * sizeof(float) > ts.part_bytes)
+            tail_groups = 0;
+    }
+    const int main_ids = (pGroups - tail_groups) * group;
+    dim3 block(256);
+    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING, false>), dim3((unsigned)main_ids), block, 0, st,
+                       (const T*)U, (const T*)V, (T*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, g.Pp,
+                       order, ep, kTiles, pTiles, 0, (float*)nullptr, (int*)nullptr);
     LAUNCH_CHECK("gemm_rows");
+    if (tail_groups) {
+        hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING, true>), dim3((unsigned)(tail_groups * group * 4)),
+                           block, 0, st, (const T*)U, (const T*)V, (T*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P,
+                           g.Cp, g.Kp, g.Pp, order, ep, kTiles, pTiles, main_ids, ts.part, ts.cnt);
+        LAUNCH_CHECK("gemm_rows tail");
+    }
     return WINO_OK;
 }
 
 template <typename T>
 int launch_gemm_rows_d(int dst, int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
-                       const void* V, void* y, hipStream_t st) {
+                       const void* V, void* y, const TailScratch& ts, hipStream_t st) {
     // one k-group per stage; ring depth from measurements: 3 for 2-byte operands, 4 for fp32
     constexpr int RING = sizeof(T) == 2 ? 3 : 4;
-    if (dst == WINO_NHWC) return launch_gemm_rows_t<T, true, 1, RING>(order, flags, bias, g, U, V, y, dst, st);
-    return launch_gemm_rows_t<T, false, 1, RING>(order, flags, bias, g, U, V, y, dst, st);
+    if (dst == WINO_NHWC) return launch_gemm_rows_t<T, true, 1, RING>(order, flags, bias, g, U, V, y, dst, ts, st);
+    return launch_gemm_rows_t<T, false, 1, RING>(order, flags, bias, g, U, V, y, dst, ts, st);
 }
 
 int launch_gemm_out(int dst, int dtype, int order, unsigned flags, const void* bias, const Geometry& g, const void* U,
-                    const void* V, void* y, hipStream_t st) {
+                    const void* V, void* y, const TailScratch& ts, hipStream_t st) {
     switch (dtype) {
-    case WINO_F32: return launch_gemm_rows_d<float>(dst, order, flags, bias, g, U, V, y, st);
-    case WINO_F16: return launch_gemm_rows_d<f16_t>(dst, order, flags, bias, g, U, V, y, st);
-    case WINO_BF16: return launch_gemm_rows_d<bf16_t>(dst, order, flags, bias, g, U, V, y, st);
+    case WINO_F32: return launch_gemm_rows_d<float>(dst, order, flags, bias, g, U, V, y, ts, st);
+    case WINO_F16: return launch_gemm_rows_d<f16_t>(dst, order, flags, bias, g, U, V, y, ts, st);
+    case WINO_BF16: return launch_gemm_rows_d<bf16_t>(dst, order, flags, bias, g, U, V, y, ts, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -501,7 +535,11 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     }
     if (algo == WINO_ALGO_EPILOGUE) {
         StageScope t(WINO_STAGE_GEMM, st);
-        return launch_gemm_out(dst, dtype, order, flags, bias, g, U, V, y, st);
+        TailScratch ts;
+        ts.part = Mo;                                 // the product region is free in this pipeline
+        ts.part_bytes = sc.total - sc.m_off;
+        ts.cnt = (int*)base;
+        return launch_gemm_out(dst, dtype, order, flags, bias, g, U, V, y, ts, st);
     }
     const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
     {
@@ -579,6 +617,8 @@ int wino_set_workspace(void* ptr, size_t bytes) {
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return fail(WINO_ERR_UNSUPPORTED, "device index %d out of range", dev);
     if (ptr && bytes == 0) return fail(WINO_ERR_INVALID, "workspace pointer with zero size");
+    if (ptr && bytes < kCounterBytes) return fail(WINO_ERR_WORKSPACE, "workspace smaller than %zu bytes", kCounterBytes);
+    if (ptr) HIP_TRY(hipMemset(ptr, 0, kCounterBytes));   // arrival counters (blocking, like every allocation)
     std::lock_guard<std::mutex> lk(g_arena_mu);
     g_arena[dev].ext = ptr;
     g_arena[dev].ext_bytes = ptr ? bytes : 0;
@@ -640,7 +680,7 @@ int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int 
     // geometry from the output size: pad 1 keeps H == Ho
     if (!make_geometry(dtype, N, C, K, Ho, Wo, 1, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d Ho=%d Wo=%d", N, C, K, Ho, Wo);
-    return launch_gemm_out(layout, dtype, tile_order, flags, nullptr, g, U, V, y, (hipStream_t)stream);
+    return launch_gemm_out(layout, dtype, tile_order, flags, nullptr, g, U, V, y, TailScratch{}, (hipStream_t)stream);
 }
 
 int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void* in, void* out,

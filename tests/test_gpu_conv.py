@@ -121,9 +121,10 @@ def test_caller_owned_workspace(oracle):
     xd, wd = dev(x), dev(w)
     want = oracle.direct_conv(x, w, 1)
     need = ops.workspace_bytes(ops.F32, N, C, K, H, W, 1)
-    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    small = torch.empty(8192, dtype=torch.uint8, device="cuda")
     big = torch.empty(need, dtype=torch.uint8, device="cuda")
     try:
+        assert L.wino_set_workspace(small.data_ptr(), 1024) == -4      # not even room for the arrival counters
         assert L.wino_set_workspace(small.data_ptr(), small.numel()) == 0
         with pytest.raises(_lib.WinoError) as e:
             ops.conv(xd, wd, algo=ops.ALGO_STAGED)
@@ -134,3 +135,27 @@ def test_caller_owned_workspace(oracle):
     finally:
         assert L.wino_set_workspace(None, 0) == 0
     assert np.array_equal(host(ops.conv(xd, wd)), want)
+
+
+@pytest.mark.parametrize("dtype,N", [(ops.F32, 65), (ops.BF16, 97)])
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_epilogue_gemm_with_a_cut_up_last_round(oracle, layout, dtype, N):
+    """Patch counts just above a whole number of rounds of resident workgroups (512 for fp32, 768 for
+    2-byte operands): the last patches are computed by four workgroups each, one Winograd row per
+    workgroup, combined by the last to arrive.  Exact on integers, and the same bits on every run."""
+    from gpu_util import TORCH_DT
+    C, K, H, W = 8, 64, 32, 64                      # 512 tiles per image, one filter tile: N*8 patches
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=5150 + N, layout=layout, integer=True)
+    bias = synth.small_ints(K, seed=3, lo=-2, hi=2).astype(np.float32)
+    want = oracle.direct_conv(x, w, 1, layout)
+    want = np.maximum(synth.act_from_layout(want, layout) + bias[None, :, None, None], 0)
+    want = synth.act_to_layout(np.ascontiguousarray(want.astype(np.float32)), layout)
+    xd, wd, bd = dev(x, dtype), dev(w, dtype), dev(bias, dtype)
+    got = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_EPILOGUE, relu=True, bias=bd)
+    assert np.array_equal(host(got), want)
+    xf, wf = synth.conv_inputs(N, C, K, H, W, seed=77, layout=layout)
+    xfd, wfd = dev(xf, dtype), dev(wf, dtype)
+    first = ops.conv(xfd, wfd, 1, layout, algo=ops.ALGO_EPILOGUE)
+    for _ in range(3):
+        assert torch.equal(ops.conv(xfd, wfd, 1, layout, algo=ops.ALGO_EPILOGUE), first)
+    assert torch.equal(ops.conv(xd, wd, 1, layout, algo=ops.ALGO_EPILOGUE, relu=True, bias=bd), got)
