@@ -312,29 +312,36 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         // Every workgroup leaves its row's contribution in tail_part[patch][row][register][thread]; the
         // one that arrives last (a counter per patch, returned to zero for the next launch) adds the four
         // rows in the order 0..3 -- so the result does not depend on who was last -- and stores the patch.
+        // The partial sums travel as device-scope relaxed atomic stores and loads (coherent across the
+        // chip's L2 slices without flushing them: a device-scope fence writes the whole L2 back); the
+        // stores have completed (vmcnt) before the workgroup's arrival is counted.
         float* mine = tail_part + ((size_t)(tq * 4 + trow) * 64) * 256 + tid;
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) mine[(a * 16 + r) * 256] = yo[a][r];
+            for (int r = 0; r < 16; ++r)
+                __hip_atomic_store(mine + (a * 16 + r) * 256, yo[a][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __shared__ int s_last;
-        __threadfence();                              // this workgroup's partial sums, visible to the device
+        __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's partial sums are in memory
         __syncthreads();
         if (tid == 0) {
-            const int old = atomicAdd(&tail_cnt[tq], 1);
+            const int old = __hip_atomic_fetch_add(&tail_cnt[tq], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = old == 3;
-            if (old == 3) tail_cnt[tq] = 0;
+            if (old == 3) __hip_atomic_store(&tail_cnt[tq], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
         if (!s_last) return;
-        __threadfence();                              // the other workgroups' partial sums
         const float* all = tail_part + ((size_t)(tq * 4) * 64) * 256 + tid;
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float* e = all + (a * 16 + r) * 256;
-                yo[a][r] = ((e[0] + e[64 * 256]) + e[2 * 64 * 256]) + e[3 * 64 * 256];
+                const float e0 = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const float e1 = __hip_atomic_load(e + 64 * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const float e2 = __hip_atomic_load(e + 2 * 64 * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const float e3 = __hip_atomic_load(e + 3 * 64 * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                yo[a][r] = ((e0 + e1) + e2) + e3;
             }
     }
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);

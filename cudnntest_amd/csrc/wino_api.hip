@@ -270,7 +270,8 @@ int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geomet
     const long slots = 256L * (sizeof(T) == 2 ? 3 : 2);
     const long real = (long)pTiles * kTiles;
     int tail_groups = 0;
-    if (ts.part && real > slots && real % slots != 0 && 4 * (real % slots) <= slots) {
+    // (fp32 only: with 2-byte operands a patch is short and the cut costs more than the idle CUs, measured)
+    if (sizeof(T) == 4 && ts.part && real > slots && real % slots != 0 && 4 * (real % slots) <= slots) {
         tail_groups = (int)((real % slots + group - 1) / group);
         const long tail_ids = (long)tail_groups * group;
         if (tail_groups >= pGroups || 4 * tail_ids > slots || tail_ids > (long)(kCounterBytes / sizeof(int)) ||
