@@ -274,8 +274,10 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
         if (ni > 3) { ni = 3; nstg = nst - 1; }      // past the end: repeat the last stage (never read)
     };
     vec fu[2], fv[2];
-    auto iteration = [&](auto par) {
+    // first: the stage opens a Winograd row, its MFMAs start from a zero accumulator
+    auto iteration = [&](auto par, auto first) {
         constexpr int S = decltype(par)::value;
+        constexpr bool FIRST = decltype(first)::value;
         typedef std::integral_constant<int, 1 - S> other_t;
         auto frag_load = [&](int r) {
             const int j = r & 3, v = 2 * (r >> 2) + lh;
@@ -293,12 +295,17 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
         for (int r = 0; r < NR; ++r) {
             if (r + 1 < NR) frag_load(r + 1);
             if (r >= NR - 1 - WP) v_piece(other_t{}, r - (NR - 1 - WP));
+            if (FIRST && r < 4) {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) acc[r][q] = 0.f;
+            }
             if (SWAP) Mma<T>::run(fv[r & 1], fu[r & 1], acc[r & 3]);
             else Mma<T>::run(fu[r & 1], fv[r & 1], acc[r & 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0) lgkmcnt(0)
-        __syncthreads();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");               // no LDS access moves across the barrier
     };
 
     // prologue: stage (0, 0) of both operands in LDS
@@ -313,11 +320,13 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     __syncthreads();
 
     for (int i = 0; i < 4; ++i) {
-        for (int st = 0; st < nst; st += 2) {
-            iteration(par0_t{});
-            iteration(par1_t{});
+        iteration(par0_t{}, std::true_type{});
+        iteration(par1_t{}, std::false_type{});
+        for (int st = 2; st < nst; st += 2) {
+            iteration(par0_t{}, std::false_type{});
+            iteration(par1_t{}, std::false_type{});
         }
-        rows_fold<true>(acc, yo, i);
+        rows_fold<false>(acc, yo, i);
     }
     rows_store<T, SWAP>(yo, y, ys, N, K, Ho, Wo, th, tw, P, order, ep, k0, p0, wm, wn, l32, lh);
 }
