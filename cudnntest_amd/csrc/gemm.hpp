@@ -189,15 +189,15 @@ template <int... S, class F> __device__ __forceinline__ void for_each_const(std:
 //
 // A workgroup alone on its CU needs the MFMA time of a whole patch (55 us for C = 256 in fp32),
 // and that is what a last round of a few workgroups costs while the other CUs idle.  The host
-// therefore launches the patches of a small last round through the TAIL variant: four workgroups
-// per patch, one Winograd row each, combined by the last one to arrive.
+// therefore appends the patches of a small last round as TAIL workgroups: four per patch, one
+// Winograd row each, combined by the last one to arrive.
 // =============================================================================
-template <typename T, bool SWAP, int NVG, int RING, bool TAIL>
+template <typename T, bool SWAP, int NVG, int RING>
 __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__ U, const T* __restrict__ V,
                                                            T* __restrict__ y, ActStrides ys, int N, int K,
                                                            int Ho, int Wo, int th, int tw, long P, int Cp,
                                                            int Kp, long Pp, int order, Epilogue ep, int kTiles,
-                                                           int pTiles, int first_id, float* __restrict__ tail_part,
+                                                           int pTiles, int main_ids, float* __restrict__ tail_part,
                                                            int* __restrict__ tail_cnt) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
@@ -214,13 +214,16 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         if constexpr (S == 0) return Vs0; else if constexpr (S == 1) return Vs1; else if constexpr (S == 2) return Vs2; else return Vs3;
     };
 
-    // TAIL: the patches of the last, partly filled round of workgroups are cut four ways -- one
-    // Winograd row per workgroup (a quarter of the reduction) -- so the whole chip works on them
-    // instead of a few CUs; tq = patch of the tail, trow = its row.  The four workgroups of a patch
-    // have ids 8 apart: the same XCD.
-    const int tq = TAIL ? ((int)blockIdx.x >> 5) * 8 + ((int)blockIdx.x & 7) : 0;
-    const int trow = TAIL ? ((int)blockIdx.x >> 3) & 3 : 0;
-    const int b = TAIL ? first_id + tq : (int)blockIdx.x;
+    // Workgroup ids >= main_ids are TAIL workgroups: the patches of the last, partly filled round are
+    // cut four ways -- one Winograd row per workgroup (a quarter of the reduction) -- so the whole chip
+    // works on them instead of a few CUs; tq = patch of the tail, trow = its row.  The four workgroups
+    // of a patch have ids 8 apart (the same XCD); they follow the whole patches in the same launch, so
+    // they start as soon as CUs run out of whole patches.
+    const bool TAIL = (int)blockIdx.x >= main_ids;
+    const int tb = (int)blockIdx.x - main_ids;
+    const int tq = TAIL ? (tb >> 5) * 8 + (tb & 7) : 0;
+    const int trow = TAIL ? (tb >> 3) & 3 : 0;
+    const int b = TAIL ? main_ids + tq : (int)blockIdx.x;
     const int xcd = b & 7, jb = b >> 3;
     const int ktile = jb % kTiles;
     const int ptile = (jb / kTiles) * 8 + xcd;

@@ -279,17 +279,11 @@ int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geomet
             tail_groups = 0;
     }
     const int main_ids = (pGroups - tail_groups) * group;
-    dim3 block(256);
-    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING, false>), dim3((unsigned)main_ids), block, 0, st,
-                       (const T*)U, (const T*)V, (T*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, g.Pp,
-                       order, ep, kTiles, pTiles, 0, (float*)nullptr, (int*)nullptr);
+    hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING>), dim3((unsigned)(main_ids + tail_groups * group * 4)),
+                       dim3(256), 0, st, (const T*)U, (const T*)V, (T*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P,
+                       g.Cp, g.Kp, g.Pp, order, ep, kTiles, pTiles, main_ids, tail_groups ? ts.part : nullptr,
+                       tail_groups ? ts.cnt : nullptr);
     LAUNCH_CHECK("gemm_rows");
-    if (tail_groups) {
-        hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING, true>), dim3((unsigned)(tail_groups * group * 4)),
-                           block, 0, st, (const T*)U, (const T*)V, (T*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P,
-                           g.Cp, g.Kp, g.Pp, order, ep, kTiles, pTiles, main_ids, ts.part, ts.cnt);
-        LAUNCH_CHECK("gemm_rows tail");
-    }
     return WINO_OK;
 }
 
@@ -436,8 +430,12 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
         // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
         if (g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
         if (g.C <= 256) return WINO_ALGO_EPILOGUE;
-        // many channels: the 128x128 GEMM's lower L2 traffic per flop wins unless there are few tiles
-        return g.P <= 4096 ? WINO_ALGO_EPILOGUE : WINO_ALGO_STAGED;
+        // many channels: the 128x128 GEMM's lower L2 traffic per flop wins, unless there are few tiles or the
+        // 64x64 patches fill their rounds of 512 resident workgroups (a small last round is cut up, see
+        // launch_gemm_rows_t)
+        const long rem = patches % 512;
+        const bool full_rounds = patches > 512 && (rem == 0 || 4 * rem <= 512);
+        return (g.P <= 4096 || full_rounds) ? WINO_ALGO_EPILOGUE : WINO_ALGO_STAGED;
     }
     // 16-bit operands: the fp32 product tensor is the largest HBM stream, so STAGED only for tiny problems;
     // the in-kernel input transform is VALU work repeated per filter tile and pays only with few filter
