@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
 
     // ---- this thread's tile and channels: fixed for the whole kernel --------------------
     const int tile = XM == XM_CHANVEC ? tid >> 2 : tid & 63;
-    const int ch0 = (XM == XM_CHANVEC ? tid & 3 : tid >> 6) * UN;   // first of its UN channels inside a stage
+    const int ch0 = (XM == XM_CHANVEC ? tid & 3 : wave) * UN;       // first of its UN channels inside a stage (wave-uniform unless XM_CHANVEC)
     unsigned u_col[4];                         // XM_ROW: [0] = offset of the clamped first column; else the 4 clamped columns
     unsigned cw[4];                            // all ones when column j of the patch lies inside the image (and the tile exists)
     unsigned img_off;                          // element offset of the tile's image
@@ -112,13 +112,19 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
             u_col[i] = (unsigned)(iwc * xs.w);                       // value is discarded through the masks
         }
         if (XM == XM_ROW) {
-            const int s0 = min(max(iw0, 0), W - 4);
-            dcol = iw0 - s0;                   // -1 at the left edge, 1 or 2 at the right edge, else 0
+            // The quadruple starts at column iw0 even where that lies outside the row: the elements it
+            // then takes from the neighbouring row are zeroed through cw.  Only where it could leave
+            // the TENSOR (first image at its left edge, last image at its right edge) is it moved
+            // inside the row, and the columns are put back in place with lane selects.
+            const bool fix = (n == 0 && iw0 < 0) || (n == N - 1 && iw0 + 3 > W - 1);
+            const int s0 = fix ? min(max(iw0, 0), W - 4) : iw0;
+            dcol = iw0 - s0;                   // fix lanes: -1 at the left edge, 1 or 2 at the right edge; else 0
             u_col[0] = (unsigned)s0;
         }
     }
     // lane masks of the edge tiles (wave-uniform 64-bit values, fixed for the whole kernel)
     const unsigned long laneL = __ballot(dcol == -1), laneR1 = __ballot(dcol == 1), laneR2 = __ballot(dcol == 2);
+    const bool any_fix = (laneL | laneR1 | laneR2) != 0;     // wave-uniform; false for all but a few waves of the grid
 
     floatx16 acc[4];
     floatx16 yo[4];                            // y00, y01, y10, y11
@@ -137,18 +143,24 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     T xa[4][UN], xb[4][UN];                    // [column][channel]; XM_ROW: [element of the quadruple][channel]
     unsigned ma_c = 0, mb_c = 0, cok_c = 0;    // all ones when patch row ra / rb lies inside the image; bit u: channel u is real
     float sg_c = 0.f;
-    unsigned ma_n, mb_n, cok_n, ra_off, rb_off;
-    float sg_n;
+    unsigned ma_n = 0, mb_n = 0, cok_n, ra_off = 0, rb_off = 0;
+    float sg_n = 0.f;
     int c_n;
     auto x_prep = [&](int row_i, int st) {
-        const int ra = row_i == 0 ? 0 : (row_i == 2 ? 2 : 1);
-        const int rb = row_i < 2 ? 2 : (row_i == 2 ? 1 : 3);
-        const int iha = ih0 + ra, ihb = ih0 + rb;
-        ma_n = (iha >= 0 && iha < H) ? 0xFFFFFFFFu : 0u;
-        mb_n = (ihb >= 0 && ihb < H) ? 0xFFFFFFFFu : 0u;
-        ra_off = img_off + (unsigned)(min(max(iha, 0), H - 1) * xs.h);
-        rb_off = img_off + (unsigned)(min(max(ihb, 0), H - 1) * xs.h);
-        sg_n = row_i == 1 ? 1.f : -1.f;
+        if (st == 0) {                             // the raw rows, their masks and the sign change with the Winograd row only
+            const int ra = row_i == 0 ? 0 : (row_i == 2 ? 2 : 1);
+            const int rb = row_i < 2 ? 2 : (row_i == 2 ? 1 : 3);
+            const int iha = ih0 + ra, ihb = ih0 + rb;
+            ma_n = (iha >= 0 && iha < H) ? 0xFFFFFFFFu : 0u;
+            mb_n = (ihb >= 0 && ihb < H) ? 0xFFFFFFFFu : 0u;
+            ra_off = img_off + (unsigned)(min(max(iha, 0), H - 1) * xs.h);
+            rb_off = img_off + (unsigned)(min(max(ihb, 0), H - 1) * xs.h);
+            if (XM == XM_ROW) {                    // byte offsets of the two quadruples inside a channel plane
+                ra_off = (ra_off + u_col[0]) * (unsigned)sizeof(T);
+                rb_off = (rb_off + u_col[0]) * (unsigned)sizeof(T);
+            }
+            sg_n = row_i == 1 ? 1.f : -1.f;
+        }
         c_n = st * NC + ch0;
         cok_n = 0;
 #pragma unroll
@@ -157,8 +169,10 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     auto x_load_unit = [&](int u) {            // XM_SCALAR, XM_ROW
         const unsigned coff = ((cok_n >> u) & 1u) ? (unsigned)((c_n + u) * xs.c) : 0u;
         if (XM == XM_ROW) {
-            const Quad<T> qa = *reinterpret_cast<const Quad<T>*>(x + (ra_off + coff + u_col[0]));
-            const Quad<T> qb = *reinterpret_cast<const Quad<T>*>(x + (rb_off + coff + u_col[0]));
+            // channel plane: a wave-uniform (scalar) base; the lane adds its 32-bit byte offset
+            const char* plane = reinterpret_cast<const char*>(x) + (size_t)coff * sizeof(T);
+            const Quad<T> qa = *reinterpret_cast<const Quad<T>*>(plane + ra_off);
+            const Quad<T> qb = *reinterpret_cast<const Quad<T>*>(plane + rb_off);
 #pragma unroll
             for (int jj = 0; jj < 4; ++jj) { xa[jj][u] = qa.v[jj]; xb[jj][u] = qb.v[jj]; }
         } else {
@@ -197,8 +211,10 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
                 const float e3 = lane_select(d[3], d[2], laneL);
                 d[0] = e0; d[1] = e1; d[2] = e2; d[3] = e3;
             };
-            pick(da);
-            pick(db);
+            if (any_fix) {
+                pick(da);
+                pick(db);
+            }
         }
         float r[4];
 #pragma unroll

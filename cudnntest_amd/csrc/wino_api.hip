@@ -324,8 +324,8 @@ int launch_fused_rows_t(int src, int dst, int order, unsigned flags, const void*
 template <typename T>
 int launch_fused_d(int src, int dst, int order, unsigned flags, const void* bias, const Geometry& g, const void* x,
                    const void* U, void* y, hipStream_t st) {
-    if ((long)g.N * g.C * g.H * g.W >= (1L << 31))
-        return fail(WINO_ERR_UNSUPPORTED, "fused kernel: input tensor too large for 32-bit element offsets");
+    if ((long)g.N * g.C * g.H * g.W * (long)sizeof(T) >= (1L << 32))
+        return fail(WINO_ERR_UNSUPPORTED, "fused kernel: input tensor too large for 32-bit byte offsets");
     constexpr int CV = ChanVec<T>::n;
     const bool swap = dst == WINO_NHWC, chan_contig = src == WINO_NHWC;
     // two k-groups per stage when Cp allows an even stage count; a 2-byte source without
@@ -425,10 +425,12 @@ int tile_order_for(int src, int /*dst*/) {
 int pick_algo(int layout, int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
     const bool nhwc = layout == WINO_NHWC;
+    // the single-kernel path addresses the input with 32-bit byte offsets
+    const bool fused_ok = (long)g.N * g.C * g.H * g.W * (long)dtype_size(dtype) < (1L << 32);
     if (dtype == WINO_F32) {
         if (patches < 512) return WINO_ALGO_STAGED;      // too few 64x64 patches to fill 256 CUs
         // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
-        if (g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
+        if (g.C <= 128 && g.K <= 128 && fused_ok) return WINO_ALGO_FUSED;
         if (g.C <= 256) return WINO_ALGO_EPILOGUE;
         // many channels: the 128x128 GEMM's lower L2 traffic per flop wins, unless there are few tiles or the
         // 64x64 patches fill their rounds of 512 resident workgroups (a small last round is cut up, see
@@ -441,6 +443,7 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     // the in-kernel input transform is VALU work repeated per filter tile and pays only with few filter
     // tiles and cheap loads (channel vectors for NHWC, which need C % 8 == 0)
     if (patches < 64) return WINO_ALGO_STAGED;
+    if (!fused_ok) return WINO_ALGO_EPILOGUE;
     if (nhwc) {
         if (g.C >= 16 && g.C <= 128 && g.K <= 128 && (g.K <= 64 || g.C >= 128)) return WINO_ALGO_FUSED;
     } else if (g.C <= 64 && g.K <= 64) {
