@@ -284,16 +284,25 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
         __builtin_amdgcn_s_waitcnt(WAIT_IMM);
         __builtin_amdgcn_s_barrier();                 // stage S landed for every wave; slot S-1 is free
         asm volatile("" ::: "memory");
+        // the stage's fragments are requested first, all of them, and the loads of the stage RING-1 ahead
+        // are issued while they travel: a wave's own LDS latency is not covered by its own MFMAs otherwise
+        vec fu[NVG][4], fv[NVG][4];
+#pragma unroll
+        for (int g = 0; g < NVG; ++g)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                fu[g][j] = uslot(sl)[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32];
+                fv[g][j] = vslot(sl)[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32];
+            }
+        __builtin_amdgcn_sched_barrier(0);
         stage_load(std::integral_constant<int, (S + RING - 1) % RING>{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < NVG; ++g)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const vec fu = uslot(sl)[j][2 * g + lh][(SWAP ? wn : wm) * 32 + l32];
-                const vec fv = vslot(sl)[j][2 * g + lh][(SWAP ? wm : wn) * 32 + l32];
-                if (SWAP) Mma<T>::run(fv, fu, acc[j]);
-                else Mma<T>::run(fu, fv, acc[j]);
+                if (SWAP) Mma<T>::run(fv[g][j], fu[g][j], acc[j]);
+                else Mma<T>::run(fu[g][j], fv[g][j], acc[j]);
             }
         __builtin_amdgcn_sched_barrier(0);
         if (++cst == nst) {
