@@ -428,7 +428,7 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     // the single-kernel path addresses the input with 32-bit byte offsets
     const bool fused_ok = (long)g.N * g.C * g.H * g.W * (long)dtype_size(dtype) < (1L << 32);
     if (dtype == WINO_F32) {
-        if (patches < 512) return WINO_ALGO_STAGED;      // too few 64x64 patches to fill 256 CUs
+        if (patches < 256) return WINO_ALGO_STAGED;      // not even one 64x64 patch per CU
         // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
         if (g.C <= 128 && g.K <= 128 && fused_ok) return WINO_ALGO_FUSED;
         if (g.C <= 256) return WINO_ALGO_EPILOGUE;
@@ -445,7 +445,7 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     if (patches < 64) return WINO_ALGO_STAGED;
     if (!fused_ok) return WINO_ALGO_EPILOGUE;
     if (nhwc) {
-        if (g.C >= 16 && g.C <= 128 && g.K <= 128 && (g.K <= 64 || g.C >= 128)) return WINO_ALGO_FUSED;
+        if (g.C >= 16 && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
     } else if (g.C <= 64 && g.K <= 64) {
         return WINO_ALGO_FUSED;
     }
