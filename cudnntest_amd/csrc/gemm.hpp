@@ -189,8 +189,8 @@ template <int... S, class F> __device__ __forceinline__ void for_each_const(std:
 //
 // A workgroup alone on its CU needs the MFMA time of a whole patch (55 us for C = 256 in fp32),
 // and that is what a last round of a few workgroups costs while the other CUs idle.  The host
-// therefore appends the patches of a small last round as TAIL workgroups: four per patch, one
-// Winograd row each, combined by the last one to arrive.
+// therefore appends the patches of a last round that fills at most 60 % of the resident workgroups
+// as TAIL workgroups: four per patch, one Winograd row each, combined by the last one to arrive.
 // =============================================================================
 template <typename T, bool SWAP, int NVG, int RING>
 __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__ U, const T* __restrict__ V,

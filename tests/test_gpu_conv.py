@@ -137,12 +137,13 @@ def test_caller_owned_workspace(oracle):
     assert np.array_equal(host(ops.conv(xd, wd)), want)
 
 
-@pytest.mark.parametrize("dtype,N", [(ops.F32, 65), (ops.F32, 66)])
+@pytest.mark.parametrize("dtype,N", [(ops.F32, 65), (ops.F32, 66), (ops.F32, 96)])
 @pytest.mark.parametrize("layout", LAYOUTS)
 def test_epilogue_gemm_with_a_cut_up_last_round(oracle, layout, dtype, N):
     """Patch counts just above a whole number of rounds of resident workgroups (512 for fp32): the
-    last patches are computed by four workgroups each, one Winograd row per workgroup, combined by the
-    last to arrive.  Exact on integers, and the same bits on every run."""
+    last patches (8, 16, and with N=96 a last round of 256) are computed by four workgroups each, one
+    Winograd row per workgroup, combined by the last to arrive.  Exact on integers, and the same bits on
+    every run."""
     from gpu_util import TORCH_DT
     C, K, H, W = 8, 64, 32, 64                      # 512 tiles per image, one filter tile: N*8 patches
     x, w = synth.conv_inputs(N, C, K, H, W, seed=5150 + N, layout=layout, integer=True)
