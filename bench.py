@@ -70,6 +70,9 @@ def main():
     ap.add_argument("--layout", default="NCHW", choices=["NCHW", "NHWC", "CHWN"])
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4"])
+    ap.add_argument("--batch", type=int, default=32, help="N of the vgg16_all13 / vgg16_stack workloads")
+    ap.add_argument("--graph", action="store_true",
+                    help="vgg16_stack: replay the pass from a HIP graph (one submission instead of ~30 launches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain copy kernel of the first layer's input (known size) three times, so a "
@@ -90,7 +93,10 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
 
-    layers = WORKLOADS[args.workload] or [(32, C, K, H) for (C, K, H) in synth.VGG16_CONV]   # (N, C, K, H)
+    if args.graph and args.workload != "vgg16_stack":
+        print("bench.py: --graph applies to --workload vgg16_stack", file=sys.stderr)
+        sys.exit(2)
+    layers = WORKLOADS[args.workload] or [(args.batch, C, K, H) for (C, K, H) in synth.VGG16_CONV]   # (N, C, K, H)
     multi = len(layers) > 1
     layout = {"NCHW": ops.NCHW, "NHWC": ops.NHWC, "CHWN": ops.CHWN}[args.layout]
     tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
@@ -107,7 +113,7 @@ def main():
         pools = {1, 3, 6, 9, 12}
         descs = [dict(K=K, layout_in=layout, layout_out=layout, relu=True, pool=i in pools, algo=algo)
                  for i, (N, C, K, H) in enumerate(layers)]
-        stack = ops.ConvStack(tdt, 32, 3, 224, 224, descs)
+        stack = ops.ConvStack(tdt, args.batch, 3, 224, 224, descs)
         for i, (N, C, K, H) in enumerate(layers):
             _, w_h = synth.conv_inputs(1, C, K, 4, 4, seed=0x5EED + i, layout=layout)
             b_h = synth.normal(K, 0xB1A5 + i, 0.05)
@@ -128,7 +134,7 @@ def main():
 
     def step():
         if stack is not None:
-            stack.forward(tensors[0][0], out=stack_out)
+            stack.forward(tensors[0][0], out=stack_out, graph=args.graph)
             return
         for (x, w, y) in tensors:
             ops.conv(x, w, 1, layout, algo=algo, relu=multi, out=y)
@@ -205,7 +211,7 @@ def main():
                    "pad": 1, "layout": args.layout, "algo": args.algo, "resolved_algo": resolved,
                    "winograd": "F(4x4,3x3)" if algo_label == "staged_f4" else "F(2x2,3x3)",
                    "filter_transform_in_step": stack is None, "relu": multi,
-                   "bias_and_pooling_in_step": stack is not None},
+                   "bias_and_pooling_in_step": stack is not None, "hip_graph": args.graph},
         "roofline": roofline,
         "stages": stages,
     }

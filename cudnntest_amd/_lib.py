@@ -32,6 +32,7 @@ SYMBOLS = {
     "wino_stack_set_layer": (_i, [_vp, _i, _vp, _vp, _vp]),
     "wino_stack_output": (_i, [_vp, _ip, _ip, _ip, _ip, _ip]),
     "wino_stack_forward": (_i, [_vp, _vp, _vp, _vp]),
+    "wino_stack_forward_graph": (_i, [_vp, _vp, _vp, _vp]),
     "wino_stack_destroy": (_i, [_vp]),
     "wino_conv": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
     "wino_conv_prepared": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),

@@ -53,6 +53,7 @@ struct Arena {
     size_t own_bytes = 0;
     void* ext = nullptr;
     size_t ext_bytes = 0;
+    unsigned long generation = 0;          // bumped whenever the arena's address may have changed
 };
 constexpr size_t kCounterBytes = 4096;     // 1024 arrival counters at the head of every arena
 Arena g_arena[kMaxDevices];
@@ -79,10 +80,16 @@ int arena_get(size_t bytes, void** out) {
         }
         HIP_TRY(hipMalloc(&a.own, bytes));
         a.own_bytes = bytes;
+        ++a.generation;
         HIP_TRY(hipMemset(a.own, 0, kCounterBytes));       // arrival counters: zero between launches
     }
     *out = a.own;
     return WINO_OK;
+}
+
+unsigned long arena_generation(int dev) {
+    std::lock_guard<std::mutex> lk(g_arena_mu);
+    return g_arena[dev].generation;
 }
 
 // ---- optional per-stage timing: HIP events recorded on the launch stream ---------
@@ -429,9 +436,10 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     // the single-kernel path addresses the input with 32-bit byte offsets
     const bool fused_ok = (long)g.N * g.C * g.H * g.W * (long)dtype_size(dtype) < (1L << 32);
     if (dtype == WINO_F32) {
-        if (patches < 256) return WINO_ALGO_STAGED;      // not even one 64x64 patch per CU
+        if (patches < 128) return WINO_ALGO_STAGED;      // a 64x64 patch for every other CU at most
         // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
         if (g.C <= 128 && g.K <= 128 && fused_ok) return WINO_ALGO_FUSED;
+        if (patches < 256) return WINO_ALGO_STAGED;      // not even one 64x64 patch per CU
         if (g.C <= 256) return WINO_ALGO_EPILOGUE;
         // many channels: the 128x128 GEMM's lower L2 traffic per flop wins, unless there are few tiles or the
         // 64x64 patches fill their rounds of 512 resident workgroups (a small last round is cut up, see
@@ -443,7 +451,7 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     // 16-bit operands: the fp32 product tensor is the largest HBM stream, so STAGED only for tiny problems;
     // the in-kernel input transform is VALU work repeated per filter tile and pays only with few filter
     // tiles and cheap loads (channel vectors for NHWC, which need C % 8 == 0)
-    if (patches < 64) return WINO_ALGO_STAGED;
+    if (patches < 64 || (g.C >= 256 && patches < 128) || (g.C >= 512 && patches < 256)) return WINO_ALGO_STAGED;
     if (!fused_ok) return WINO_ALGO_EPILOGUE;
     if (nhwc) {
         if (g.C >= 16 && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
@@ -625,6 +633,7 @@ int wino_set_workspace(void* ptr, size_t bytes) {
     std::lock_guard<std::mutex> lk(g_arena_mu);
     g_arena[dev].ext = ptr;
     g_arena[dev].ext_bytes = ptr ? bytes : 0;
+    ++g_arena[dev].generation;
     return WINO_OK;
 }
 
@@ -810,7 +819,35 @@ struct wino_stack {
     std::vector<Layer> layers;
     void* act[2] = {nullptr, nullptr};   // activations between layers
     size_t act_bytes = 0;
+    // the captured forward pass (wino_stack_forward_graph) and what it was captured for
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipStream_t capture_stream = nullptr;
+    const void* gx = nullptr;
+    void* gy = nullptr;
+    unsigned long garena = 0;
 };
+
+static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
+    const int n = (int)s->layers.size();
+    const void* in = x;
+    for (int l = 0; l < n; ++l) {
+        const auto& L = s->layers[l];
+        void* out = l + 1 == n ? y : s->act[l & 1];
+        int rc = conv_impl(L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
+                           nullptr, L.U, L.has_bias ? L.bias : nullptr, out, stream);
+        if (rc) return rc;
+        in = out;
+    }
+    return WINO_OK;
+}
+
+static void stack_drop_graph(wino_stack* s) {
+    if (s->exec) (void)hipGraphExecDestroy(s->exec);
+    if (s->graph) (void)hipGraphDestroy(s->graph);
+    s->exec = nullptr;
+    s->graph = nullptr;
+}
 
 int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const wino_stack_layer_t* layers,
                       wino_stack_t** stack) {
@@ -894,15 +931,45 @@ int wino_stack_forward(wino_stack_t* s, const void* x, void* y, void* stream) {
     const int n = (int)s->layers.size();
     for (int l = 0; l < n; ++l)
         if (!s->layers[l].set) return fail(WINO_ERR_INVALID, "layer %d has no filters yet", l);
-    const void* in = x;
-    for (int l = 0; l < n; ++l) {
-        const auto& L = s->layers[l];
-        void* out = l + 1 == n ? y : s->act[l & 1];
-        int rc = conv_impl(L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
-                           nullptr, L.U, L.has_bias ? L.bias : nullptr, out, stream);
-        if (rc) return rc;
-        in = out;
+    return stack_run(s, x, y, stream);
+}
+
+int wino_stack_forward_graph(wino_stack_t* s, const void* x, void* y, void* stream) {
+    if (!s || !x || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    for (size_t l = 0; l < s->layers.size(); ++l)
+        if (!s->layers[l].set) return fail(WINO_ERR_INVALID, "layer %zu has no filters yet", l);
+    if (g_timing) return stack_run(s, x, y, stream);          // stage timing brackets eager launches
+    // the arena must not grow while the pass is being captured: size it for the largest layer first
+    size_t need = 0;
+    for (const auto& L : s->layers) {
+        Geometry g;
+        if (!make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g)) return fail(WINO_ERR_INVALID, "bad layer shape");
+        need = std::max(need, scratch_layout(g, s->dtype).total);
     }
+    void* base = nullptr;
+    int rc = arena_get(need, &base);
+    if (rc) return rc;
+    const unsigned long gen = arena_generation(s->device);
+    if (!s->exec || s->gx != x || s->gy != y || s->garena != gen) {
+        stack_drop_graph(s);
+        if (!s->capture_stream) HIP_TRY(hipStreamCreateWithFlags(&s->capture_stream, hipStreamNonBlocking));
+        HIP_TRY(hipStreamBeginCapture(s->capture_stream, hipStreamCaptureModeThreadLocal));
+        rc = stack_run(s, x, y, s->capture_stream);
+        const hipError_t e = hipStreamEndCapture(s->capture_stream, &s->graph);
+        if (rc || e != hipSuccess) {
+            stack_drop_graph(s);
+            return rc ? rc : fail(WINO_ERR_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+        }
+        const hipError_t ei = hipGraphInstantiate(&s->exec, s->graph, nullptr, nullptr, 0);
+        if (ei != hipSuccess) {
+            stack_drop_graph(s);
+            return fail(WINO_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(ei));
+        }
+        s->gx = x;
+        s->gy = y;
+        s->garena = gen;
+    }
+    HIP_TRY(hipGraphLaunch(s->exec, (hipStream_t)stream));
     return WINO_OK;
 }
 
@@ -914,6 +981,8 @@ int wino_stack_destroy(wino_stack_t* s) {
     }
     for (int i = 0; i < 2; ++i)
         if (s->act[i]) (void)hipFree(s->act[i]);
+    stack_drop_graph(s);
+    if (s->capture_stream) (void)hipStreamDestroy(s->capture_stream);
     delete s;
     return WINO_OK;
 }

@@ -206,12 +206,18 @@ class ConvStack:
         _lib.check(_lib.load().wino_stack_set_layer(self._h, layer, _ptr(w), _ptr(bias) if bias is not None else None,
                                                     _stream()), "wino_stack_set_layer")
 
-    def forward(self, x, out=None):
+    def forward(self, x, out=None, graph=False):
+        """All layers on the current stream.  graph=True replays the pass from a HIP graph recorded on the
+        first call for this (x, out) pair: pass the same tensors again to benefit."""
         if tuple(x.shape) != tuple(self.in_shape) or x.dtype != self.dtype:
             raise ValueError(f"input must be {tuple(self.in_shape)} of {self.dtype}")
         if out is None:
             out = torch.empty(self.out_shape, dtype=self.dtype, device=x.device)
-        _lib.check(_lib.load().wino_stack_forward(self._h, _ptr(x), _ptr(out), _stream()), "wino_stack_forward")
+        if graph:
+            _lib.check(_lib.load().wino_stack_forward_graph(self._h, _ptr(x), _ptr(out), _stream()),
+                       "wino_stack_forward_graph")
+        else:
+            _lib.check(_lib.load().wino_stack_forward(self._h, _ptr(x), _ptr(out), _stream()), "wino_stack_forward")
         return out
 
     def close(self):

@@ -208,6 +208,13 @@ int wino_stack_set_layer(wino_stack_t *stack, int layer, const void *w, const vo
 int wino_stack_output(const wino_stack_t *stack, int *N, int *K, int *H, int *W, int *layout);
 /* all layers on `stream`; x and y are caller tensors; fails if a layer has not been set */
 int wino_stack_forward(wino_stack_t *stack, const void *x, void *y, void *stream);
+/* The same pass replayed from a HIP graph: the first call for a pair (x, y) records the launches of all layers
+ * (on a stream of the stack's own) and instantiates the graph, later calls with the same pointers launch it on
+ * `stream` -- one submission instead of two or three kernel launches per layer, which is what small batches are
+ * bound by.  Recorded again by itself when x, y or the scratch arena's address change.  Not for concurrent use
+ * with calls that may grow the arena from other threads.  The reference launches layer by layer
+ * (VGG_Batched/Network.h:603-669) and has no counterpart. */
+int wino_stack_forward_graph(wino_stack_t *stack, const void *x, void *y, void *stream);
 int wino_stack_destroy(wino_stack_t *stack);
 
 /* ---- housekeeping ----------------------------------------------------------- */

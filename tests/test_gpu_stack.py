@@ -90,3 +90,40 @@ def test_stack_rejects_bad_requests():
     st.set_layer(1, torch.zeros((4, 4, 3, 3), device="cuda"), torch.ones(4, device="cuda"))
     assert torch.equal(st.forward(x), torch.ones((1, 4, 4, 4), device="cuda"))
     st.close()
+
+
+def test_stack_replayed_from_a_graph_matches_eager_launches(oracle):
+    """wino_stack_forward_graph: every replay -- with eager work of the library and synchronisations in
+    between, after the input changed in place, after a change of tensors and after the scratch arena moved --
+    gives the bits of the eager pass."""
+    N, C, H = 2, 3, 20
+    layers = [dict(L, layout_in=ops.NCHW, layout_out=ops.NCHW) for L in VGG_LIKE[:4]]
+    params = make_params(oracle, C, layers, ops.F32)
+    st = ops.ConvStack(torch.float32, N, C, H, H, layers)
+    for i, (w, b) in enumerate(params):
+        st.set_layer(i, dev(w), dev(b))
+    x = dev(synth.uniform_pm1(N * C * H * H, 0xC1).reshape(N, C, H, H))
+    other_x, other_w = synth.conv_inputs(2, 8, 8, 12, 12, seed=5)
+    other_x, other_w = dev(other_x), dev(other_w)
+    out = torch.empty(st.out_shape, device="cuda")
+    want = st.forward(x).clone()
+    for rep in range(4):
+        out.zero_()
+        st.forward(x, out=out, graph=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+        ops.conv(other_x, other_w)                    # eager work between the replays
+        torch.cuda.synchronize()
+    x.mul_(-0.5)                                      # new values behind the same pointer
+    want2 = st.forward(x).clone()
+    assert not torch.equal(want2, want)
+    assert torch.equal(st.forward(x, out=out, graph=True), want2)
+    x2, out2 = x.clone(), torch.empty_like(out)       # other tensors: recorded again
+    assert torch.equal(st.forward(x2, out=out2, graph=True), want2)
+    big_x, big_w = synth.conv_inputs(4, 64, 64, 40, 40, seed=6)
+    ops.conv(dev(big_x), dev(big_w), algo=ops.ALGO_STAGED)   # grows the arena: its address may change
+    torch.cuda.synchronize()
+    for rep in range(2):
+        out2.zero_()
+        assert torch.equal(st.forward(x2, out=out2, graph=True), want2), rep
+    st.close()
