@@ -127,24 +127,29 @@ __host__ inline bool make_geometry(int dtype, int N, int C, int K, int H, int W,
     g->th = (g->Ho + m - 1) / m;
     g->tw = (g->Wo + m - 1) / m;
     g->P = (long)N * g->th * g->tw;
+    if (g->P >= (1L << 31)) return false;          // the kernels decode tile indices with 32-bit arithmetic
     g->Cp = (int)round_up(C, c_pad(dtype));
     g->Kp = (int)round_up(K, kKPad);
     g->Pp = round_up(g->P, kPPad);
     return true;
 }
 
-// tile index -> (n, ty, tx)
+// tile index -> (n, ty, tx); p < 2^31 (make_geometry), so 32-bit unsigned divisions (a quarter of the
+// instructions of 64-bit ones: the stores of the GEMM epilogues decode up to 16 tiles per lane)
 __device__ __forceinline__ void decode_tile(long p, int order, int N, int th, int tw, int& n, int& ty, int& tx) {
+    const unsigned pu = (unsigned)p;
     if (order == WINO_TILES_BATCH_MAJOR) {
-        tx = (int)(p % tw);
-        long q = p / tw;
-        ty = (int)(q % th);
-        n = (int)(q / th);
+        const unsigned q = pu / (unsigned)tw;
+        tx = (int)(pu - q * (unsigned)tw);
+        const unsigned nn = q / (unsigned)th;
+        ty = (int)(q - nn * (unsigned)th);
+        n = (int)nn;
     } else {
-        n = (int)(p % N);
-        long q = p / N;
-        tx = (int)(q % tw);
-        ty = (int)(q / tw);
+        const unsigned q = pu / (unsigned)N;
+        n = (int)(pu - q * (unsigned)N);
+        const unsigned yy = q / (unsigned)tw;
+        tx = (int)(q - yy * (unsigned)tw);
+        ty = (int)yy;
     }
 }
 
