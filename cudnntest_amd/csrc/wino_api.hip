@@ -142,7 +142,9 @@ Scratch scratch_layout(const Geometry& g, int dtype) {
 // ---- stage launchers (typed) -------------------------------------------------------
 template <typename T>
 int launch_filter_transform(int layout, int K, int C, int Kp, int Cp, const void* w, void* U, hipStream_t st) {
-    dim3 grid((Kp + 255) / 256, Cp / ChanVec<T>::n), block(256);
+    // one wave per workgroup: the kernel is all latency, and K*C/CV threads in workgroups of 256 would leave
+    // most CUs of the chip without a wave
+    dim3 grid((Kp + 63) / 64, Cp / ChanVec<T>::n), block(64);
     hipLaunchKernelGGL(filter_transform_kernel<T>, grid, block, 0, st, (const T*)w, (T*)U, flt_strides(layout, K, C),
                        K, C, Kp, Cp);
     LAUNCH_CHECK("filter_transform");
