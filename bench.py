@@ -52,12 +52,12 @@ WORKLOADS = {
 # script (summaries and the copy-kernel scale factor under profiles/), keyed by
 # (workload, layout, dtype, resolved algo).
 MEASURED_TRAFFIC = {
-    # profiles/epilogue_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 589.3 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
-    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"): 700.5e6,
-    # profiles/staged_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 449.4 MB fetched + 411.0 MB written
-    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"): 860.4e6,
-    # profiles/fused_fp32_nchw_vgg16_conv1_2_N32_hbm_traffic.txt: 593.9 MB fetched + 411.0 MB written
-    ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"): 1004.9e6,
+    # profiles/epilogue_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 594.9 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"): 706.0e6,
+    # profiles/staged_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 449.5 MB fetched + 411.0 MB written
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"): 860.5e6,
+    # profiles/fused_fp32_nchw_vgg16_conv1_2_N32_hbm_traffic.txt: 596.1 MB fetched + 411.0 MB written
+    ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"): 1007.2e6,
 }
 
 
@@ -69,7 +69,7 @@ def main():
     ap.add_argument("--workload", default="vgg16_conv3_N32_C256_K256_H56", choices=sorted(WORKLOADS))
     ap.add_argument("--layout", default="NCHW", choices=["NCHW", "NHWC", "CHWN"])
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
-    ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4", "direct"])
     ap.add_argument("--batch", type=int, default=32, help="N of the vgg16_all13 / vgg16_stack workloads")
     ap.add_argument("--graph", action="store_true",
                     help="vgg16_stack: replay the pass from a HIP graph (one submission instead of ~30 launches)")
@@ -102,7 +102,7 @@ def main():
     tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
     dt = {"f32": ops.F32, "f16": ops.F16, "bf16": ops.BF16}[args.dtype]
     algo = {"auto": ops.ALGO_AUTO, "staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE,
-            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4}[args.algo]
+            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4, "direct": ops.ALGO_DIRECT}[args.algo]
     es = 4 if args.dtype == "f32" else 2
 
     stack = None
@@ -174,6 +174,9 @@ def main():
         g = ops.f4_geometry(dt, N, C, K, H, H, 1) if f4 else ops.geometry(dt, N, C, K, H, H, 1)
         P, nxi = g["P"], (36 if f4 else 16)
         resolved.append(ops.ALGO_NAMES[a])
+        if a == ops.ALGO_DIRECT:                  # no Winograd: the direct-convolution flops, no transforms
+            gemm_flops += 2.0 * N * K * C * H * H * 9
+            continue
         gemm_flops += 2.0 * nxi * P * K * C
         if stack is None:
             alg_flt += (9 + nxi) * K * C * es
@@ -193,7 +196,7 @@ def main():
     peak = MFMA_PEAK_TFLOPS[args.dtype]
     stages["gemm"] = {"ms": round(gemm_ms, 4), "TFLOPs": round(achieved, 2)}
     kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
-              "staged_f4": "gemm_128x128_kernel"}
+              "staged_f4": "gemm_128x128_kernel", "direct": "direct_small_c_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"
     traffic = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label))
     roofline = {"bound": "mfma", "kernel": kernel.get(algo_label, "per-layer choice"),

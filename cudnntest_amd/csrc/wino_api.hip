@@ -11,6 +11,7 @@
 
 #include "common.hpp"
 #include "fused.hpp"
+#include "direct.hpp"
 #include "gemm.hpp"
 #include "transforms.hpp"
 #include "transforms_f4.hpp"
@@ -432,6 +433,52 @@ int tile_order_for(int src, int /*dst*/) {
 // Measured on MI355X over the VGG-16 layer shapes: the fewer the channels, the more
 // the transformed tensors cost relative to the multiplies, and the more fusion pays.
 // Chosen from sweeps of the VGG-16 shapes over the three algorithms, per layout and element type.
+// ---- direct convolution of layers with C <= 4 ----------------------------------------
+// lanes along the contiguous axis of y (w for NCHW, n for CHWN, k for NHWC); pooled outputs stay on the
+// Winograd path
+bool direct_ok(int dst, unsigned flags, const Geometry& g) {
+    const size_t lds = direct_lds_bytes(g.C, g.K);
+    return lds != 0 && lds <= 64 * 1024 && !(flags & WINO_FLAG_POOL2) &&
+           (long)g.N * g.C * g.H * g.W < (1L << 30) && (long)g.N * g.K * g.Ho * g.Wo < (1L << 30);   // 32-bit byte offsets
+}
+
+template <typename T>
+int launch_direct_t(int src, int dst, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
+                    void* y, hipStream_t st) {
+    const long Q = (long)g.N * g.Ho * g.Wo;
+    // 32-pixel groups per wave: as many as leave about eight workgroups for every CU (the filter bank is staged
+    // per workgroup, so more pixels per workgroup are cheaper, fewer workgroups fill the chip worse)
+    int groups = (int)std::min<long>(DIRECT_MAX_GROUPS, std::max<long>(1, Q / (128L * 2048)));
+    const long per_wg = 128L * groups;
+    const dim3 grid((unsigned)((Q + per_wg - 1) / per_wg)), block(256);
+    const size_t lds = direct_lds_bytes(g.C, g.K);
+    const ActStrides xs = act_strides(src, g.N, g.C, g.H, g.W), ys = act_strides(dst, g.N, g.K, g.Ho, g.Wo);
+    const FltStrides fs = flt_strides(src, g.K, g.C);
+    const Epilogue ep = make_epilogue(flags, bias);
+    const int minor = dst == WINO_CHWN;
+#define DIRECT_LAUNCH(NE)                                                                                           \
+    if (dst == WINO_NHWC)                                                                                           \
+        hipLaunchKernelGGL((direct_small_c_kernel<T, NE, true>), grid, block, lds, st, (const T*)x, (const T*)w, (T*)y, \
+                           xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, minor, Q, groups, ep);            \
+    else                                                                                                            \
+        hipLaunchKernelGGL((direct_small_c_kernel<T, NE, false>), grid, block, lds, st, (const T*)x, (const T*)w, (T*)y, \
+                           xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, minor, Q, groups, ep)
+    switch (g.C) {
+    case 1: DIRECT_LAUNCH(5); break;
+    case 2: DIRECT_LAUNCH(9); break;
+    case 3: DIRECT_LAUNCH(14); break;
+    default: DIRECT_LAUNCH(18); break;
+    }
+#undef DIRECT_LAUNCH
+    LAUNCH_CHECK("direct_small_c");
+    return WINO_OK;
+}
+
+int launch_direct(int src, int dst, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x,
+                  const void* w, void* y, hipStream_t st) {
+    DISPATCH_DTYPE(dtype, launch_direct_t<T>(src, dst, flags, bias, g, x, w, y, st));
+}
+
 int pick_algo(int layout, int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
     const bool nhwc = layout == WINO_NHWC;
@@ -504,7 +551,7 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
               const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
-    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_STAGED_F4) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
+    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_DIRECT) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
     if (!x || (!w && !Upre) || !y) return fail(WINO_ERR_INVALID, "null tensor pointer");
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
@@ -512,7 +559,14 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     if (flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)) return fail(WINO_ERR_INVALID, "unknown flags 0x%x", flags);
     if ((flags & WINO_FLAG_POOL2) && (g.Ho < 2 || g.Wo < 2))
         return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", g.Ho, g.Wo);
-    if (algo == WINO_ALGO_AUTO) algo = pick_algo(src, dtype, g);
+    if (algo == WINO_ALGO_AUTO) algo = (w && direct_ok(dst, flags, g)) ? WINO_ALGO_DIRECT : pick_algo(src, dtype, g);
+    if (algo == WINO_ALGO_DIRECT) {
+        if (!w) return fail(WINO_ERR_INVALID, "the direct path needs the filter bank, not its Winograd transform");
+        if (!direct_ok(dst, flags, g))
+            return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for C <= 4 without pooling");
+        StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
+        return launch_direct(src, dst, dtype, flags, bias, g, x, w, y, (hipStream_t)stream);
+    }
     if (algo == WINO_ALGO_STAGED_F4) {
         if (bias || (flags & WINO_FLAG_POOL2))
             return fail(WINO_ERR_UNSUPPORTED, "bias and pooling are not built for the F(4x4,3x3) mode");
@@ -598,7 +652,7 @@ int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
-    return pick_algo(layout, dtype, g);
+    return direct_ok(layout, 0, g) ? WINO_ALGO_DIRECT : pick_algo(layout, dtype, g);
 }
 
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp, int* Kp,
@@ -815,6 +869,7 @@ struct wino_stack {
         int layout_in, layout_out, algo;
         unsigned flags;
         void* U = nullptr;         // cached transformed filters
+        void* wraw = nullptr;      // layers with C <= 4: a copy of the filter bank itself, for the direct path
         void* bias = nullptr;
         bool set = false, has_bias = false;
     };
@@ -837,7 +892,7 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
         const auto& L = s->layers[l];
         void* out = l + 1 == n ? y : s->act[l & 1];
         int rc = conv_impl(L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
-                           nullptr, L.U, L.has_bias ? L.bias : nullptr, out, stream);
+                           L.wraw, L.U, L.has_bias ? L.bias : nullptr, out, stream);
         if (rc) return rc;
         in = out;
     }
@@ -897,6 +952,7 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         make_geometry(dtype, N, L.C, L.K, L.H, L.W, 1, &g);
         hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
+        if (e == hipSuccess && L.C <= 4) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         if (e != hipSuccess) return bail(e);
     }
     for (int i = 0; i < 2 && raw->act_bytes; ++i) {
@@ -913,6 +969,9 @@ int wino_stack_set_layer(wino_stack_t* s, int layer, const void* w, const void* 
     auto& L = s->layers[layer];
     int rc = wino_filter_transform(L.layout_in, s->dtype, L.K, L.C, w, L.U, stream);
     if (rc) return rc;
+    if (L.wraw)
+        HIP_TRY(hipMemcpyAsync(L.wraw, w, (size_t)9 * L.K * L.C * dtype_size(s->dtype), hipMemcpyDeviceToDevice,
+                               (hipStream_t)stream));
     L.has_bias = bias != nullptr;
     if (bias)
         HIP_TRY(hipMemcpyAsync(L.bias, bias, (size_t)L.K * dtype_size(s->dtype), hipMemcpyDeviceToDevice,
@@ -979,6 +1038,7 @@ int wino_stack_destroy(wino_stack_t* s) {
     if (!s) return WINO_OK;
     for (auto& L : s->layers) {
         if (L.U) (void)hipFree(L.U);
+        if (L.wraw) (void)hipFree(L.wraw);
         if (L.bias) (void)hipFree(L.bias);
     }
     for (int i = 0; i < 2; ++i)

@@ -23,7 +23,7 @@ from . import _lib
 
 NCHW, NHWC, CHWN = 0, 1, 2
 F32, F16, BF16 = 0, 1, 2
-ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED, ALGO_STAGED_F4 = 0, 1, 2, 3, 4
+ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED, ALGO_STAGED_F4, ALGO_DIRECT = 0, 1, 2, 3, 4, 5
 TILES_BATCH_MAJOR, TILES_BATCH_MINOR = 0, 1
 PRODUCT_KP, PRODUCT_PK = 0, 1
 FLAG_RELU = 1
@@ -83,7 +83,7 @@ def geometry(dtype, N, C, K, H, W, pad):
 
 
 ALGO_NAMES = {ALGO_AUTO: "auto", ALGO_STAGED: "staged", ALGO_EPILOGUE: "epilogue", ALGO_FUSED: "fused",
-              ALGO_STAGED_F4: "staged_f4"}
+              ALGO_STAGED_F4: "staged_f4", ALGO_DIRECT: "direct"}
 
 
 def pick_algo(layout, dtype, N, C, K, H, W, pad=1):

@@ -37,9 +37,14 @@ typedef enum {
     WINO_ALGO_EPILOGUE = 2, /* output transform applied in the GEMM epilogue (no product tensor in HBM) */
     WINO_ALGO_FUSED = 3,    /* one kernel: input transform, multiply-accumulate and output transform
                                (the structure of fusedTest/winotrans.cuh:1452 Winofuse4433) */
-    WINO_ALGO_STAGED_F4 = 4 /* the staged pipeline in F(4x4,3x3) -- 6x6 tiles, 36 coordinates, the reference's
+    WINO_ALGO_STAGED_F4 = 4, /* the staged pipeline in F(4x4,3x3) -- 6x6 tiles, 36 coordinates, the reference's
                                own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101).
                                Never chosen by WINO_ALGO_AUTO. */
+    WINO_ALGO_DIRECT = 5     /* no Winograd at all: the 9*C <= 36 products of an output as one short MFMA
+                               reduction, for layers with C <= 4 (the network's first layer, which the
+                               reference runs through the same wrappers: comparison/layoutCompare.cu:38-46).
+                               Bias and ReLU, no pooling; needs the filter bank itself (not
+                               wino_conv_prepared).  What WINO_ALGO_AUTO picks for such layers. */
 } wino_algo_t;
 
 /* order of the tile index p inside the transformed operands */
