@@ -10,6 +10,9 @@ convolutions (ReLU fused into the output stage) on synthetic activations of each
 layer's shape; `--workload vgg16_stack` chains them through the conv-stack driver
 (bias, ReLU and the five 2x2 poolings in the output stages, cached filter transforms).
 
+Before the W warm-up steps the step runs untimed for --ramp-ms (200 ms): the GPU's clock governor needs
+tens of milliseconds of load to reach its working frequency, and W steps of a 0.5 ms layer do not give it that.
+
 Prints ONE JSON line:
   value        effective TFLOP/s = direct-convolution FLOPs (2*N*K*C*H*W*9) / time
   ms_per_step  ms per layer (per 13-layer pass for vgg16_all13)
@@ -73,6 +76,9 @@ def main():
     ap.add_argument("--batch", type=int, default=32, help="N of the vgg16_all13 / vgg16_stack workloads")
     ap.add_argument("--graph", action="store_true",
                     help="vgg16_stack: replay the pass from a HIP graph (one submission instead of ~30 launches)")
+    ap.add_argument("--ramp-ms", type=float, default=200.0,
+                    help="untimed steps before the warm-up, for this long: the shader clock needs tens of ms of "
+                         "sustained load to leave its idle level (2.1 -> 2.4 GHz measured), more than W short steps give")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain copy kernel of the first layer's input (known size) three times, so a "
@@ -143,6 +149,11 @@ def main():
     if args.copy_probe:
         for _ in range(3):
             ops.layout_transform(tensors[0][0], layout, layout)   # same layout both sides: a plain copy
+    t_ramp = time.perf_counter()
+    while (time.perf_counter() - t_ramp) * 1e3 < args.ramp_ms:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
