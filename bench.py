@@ -21,6 +21,8 @@ Prints ONE JSON line:
                algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4)
   cpu_baseline the oracle's fp32 OpenMP direct convolution on this host's cores (reported, not a target)
   stages       per-stage ms and achieved GB/s (algorithmic bytes) or TFLOP/s
+  layout_transforms   the stand-alone permutations of the layer's input between its layout and the other two
+               (wino_layout_transform; bytes = read + write), timed apart from the convolution
 """
 import argparse
 import json
@@ -229,6 +231,31 @@ def main():
         "roofline": roofline,
         "stages": stages,
     }
+
+    # ---- the stand-alone layout permutations of the layer's input, timed separately ------------
+    if not multi and stack is None:
+        names = {ops.NCHW: "NCHW", ops.NHWC: "NHWC", ops.CHWN: "CHWN"}
+        x0 = tensors[0][0]
+        perms = {}
+        for dst_l in (ops.NCHW, ops.NHWC, ops.CHWN):
+            if dst_l == layout:
+                continue
+            x1 = ops.layout_transform(x0, layout, dst_l)
+            for (a, la, lb) in ((x0, layout, dst_l), (x1, dst_l, layout)):
+                for _ in range(3):
+                    ops.layout_transform(a, la, lb)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(20):
+                    ops.layout_transform(a, la, lb)
+                e1.record()
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / 20
+                gbs = 2.0 * x0.numel() * es / (ms * 1e-3) / 1e9
+                perms[f"{names[la]}->{names[lb]}"] = {"ms": round(ms, 4), "GBps": round(gbs, 1),
+                                                      "frac_hbm": round(gbs / HBM_PEAK_GBS, 3)}
+            del x1
+        out["layout_transforms"] = perms
 
     if not args.no_cpu_baseline:
         import oracle

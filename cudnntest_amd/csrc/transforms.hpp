@@ -521,4 +521,47 @@ __global__ __launch_bounds__(256) void permute_gather_kernel(const T* __restrict
     out[e] = in[n * a.n + c * a.c + h * a.h + w * a.w];
 }
 
+// Layout permutation through an LDS tile: a tensor seen as [R][A][B] with the source contiguous along A and the
+// destination contiguous along B (the six layout pairs all have this shape: e.g. NCHW -> NHWC is R = n,
+// A = h*w, B = c).  A workgroup moves a TA x TB (A x B) tile of 4096 elements -- 64 x 64, or 32 x 128 / 128 x 32
+// when one of the axes is the batch of 32 or fewer: lanes read along A, write along B, in runs of up to 512 bytes;
+// the tile is padded by one column so that neither side has bank conflicts.
+struct PermuteDims {
+    long nA, nB, nR;          // extents
+    long sB, sR;              // source strides of B and R (A has stride 1)
+    long dA, dR;              // destination strides of A and R (B has stride 1)
+};
+
+template <typename T, int TA, int TB>
+__global__ __launch_bounds__(256) void permute_tiled_kernel(const T* __restrict__ in, T* __restrict__ out, PermuteDims d,
+                                                             int tilesA, int tilesB) {
+    static_assert(TA * TB == 4096 && TA >= 32 && TB >= 32, "tile shape");
+    __shared__ T tile[TB][TA + 1];
+    long t = blockIdx.x;
+    const int ta = (int)(t % tilesA);
+    t /= tilesA;
+    const int tb = (int)(t % tilesB);
+    const long r = t / tilesB;
+    const long a0 = (long)ta * TA, b0 = (long)tb * TB;
+    const T* src = in + r * d.sR;
+    T* dst = out + r * d.dR;
+    {
+        const int lx = threadIdx.x % TA, ly = threadIdx.x / TA;      // lanes along A
+#pragma unroll 4
+        for (int i = ly; i < TB; i += 256 / TA) {
+            const long a = a0 + lx, b = b0 + i;
+            if (a < d.nA && b < d.nB) tile[i][lx] = src[b * d.sB + a];
+        }
+    }
+    __syncthreads();
+    {
+        const int lx = threadIdx.x % TB, ly = threadIdx.x / TB;      // lanes along B
+#pragma unroll 4
+        for (int i = ly; i < TA; i += 256 / TB) {
+            const long a = a0 + i, b = b0 + lx;
+            if (a < d.nA && b < d.nB) dst[a * d.dA + b] = tile[lx][i];
+        }
+    }
+}
+
 }  // namespace wino

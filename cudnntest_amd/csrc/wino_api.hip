@@ -758,9 +758,36 @@ int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int 
     if (!in || !out) return fail(WINO_ERR_INVALID, "null pointer");
     if (N <= 0 || C <= 0 || H <= 0 || W <= 0) return fail(WINO_ERR_INVALID, "bad shape");
     const long total = (long)N * C * H * W;
+    hipStream_t st = (hipStream_t)stream;
+    if (src != dst) {
+        // [R][A][B]: A = the source's contiguous axis, B = the destination's (see permute_tiled_kernel)
+        const long HW = (long)H * W;
+        PermuteDims d;
+        if (src == WINO_NCHW && dst == WINO_NHWC) d = {HW, C, N, HW, C * HW, C, HW * C};
+        else if (src == WINO_NHWC && dst == WINO_NCHW) d = {C, HW, N, C, HW * C, HW, C * HW};
+        else if (src == WINO_NCHW && dst == WINO_CHWN) d = {C * HW, N, 1, C * HW, 0, N, 0};
+        else if (src == WINO_CHWN && dst == WINO_NCHW) d = {N, C * HW, 1, N, 0, C * HW, 0};
+        else if (src == WINO_NHWC && dst == WINO_CHWN) d = {C, N, HW, HW * C, C, HW * N, N};
+        else d = {N, C, HW, HW * N, N, HW * C, C};               // CHWN -> NHWC
+        const int TA = d.nA <= 32 ? 32 : (d.nB <= 32 ? 128 : 64), TB = 4096 / TA;
+        const long tilesA = (d.nA + TA - 1) / TA, tilesB = (d.nB + TB - 1) / TB;
+        const long blocks = tilesA * tilesB * d.nR;
+        if (blocks >= (1L << 31)) return fail(WINO_ERR_UNSUPPORTED, "layout transform: tensor too large");
+#define PERMUTE(T, A, B)                                                                                      \
+    hipLaunchKernelGGL((permute_tiled_kernel<T, A, B>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)in, \
+                       (T*)out, d, (int)tilesA, (int)tilesB)
+        if (dtype == WINO_F32) {
+            if (TA == 32) PERMUTE(float, 32, 128); else if (TA == 128) PERMUTE(float, 128, 32); else PERMUTE(float, 64, 64);
+        } else {
+            if (TA == 32) PERMUTE(uint16_t, 32, 128); else if (TA == 128) PERMUTE(uint16_t, 128, 32); else PERMUTE(uint16_t, 64, 64);
+        }
+#undef PERMUTE
+        LAUNCH_CHECK("layout_transform");
+        return WINO_OK;
+    }
+    // same layout on both sides: a plain copy
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     const ActStrides a = act_strides(src, N, C, H, W);
-    hipStream_t st = (hipStream_t)stream;
     if (dtype == WINO_F32)
         hipLaunchKernelGGL(permute_gather_kernel<float>, grid, block, 0, st, (const float*)in, (float*)out, a, dst, N,
                            C, H, W);
