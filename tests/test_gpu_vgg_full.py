@@ -1,4 +1,4 @@
-"""Every VGG-16 3x3 layer at its full size (N=32), in all three layouts, fp32 and bf16, with the
+"""Every VGG-16 3x3 layer at its full size (N=32), in all three layouts, fp32, f16 and bf16, with the
 algorithm AUTO picks: the configuration list of the reference's layer driver
 (comparison/layoutCompare.cu:38-148, one case per (C, K, H) of the network) at the batch the
 headline numbers are quoted on.
@@ -8,7 +8,7 @@ The CPU oracle cannot convolve whole layers of this size in test time, so the ch
     of that image with those filters (the oracle sees exactly the values the device was given);
   * the NHWC and CHWN results must agree with the NCHW result of the same values over the whole tensor
     (different input kernels, tile orders, store paths; the same arithmetic up to summation order).
-Tolerances: relative L2 1e-4 (fp32), 2e-2 (bf16)."""
+Tolerances: relative L2 1e-4 (fp32), 2e-2 (f16, bf16)."""
 import numpy as np
 import pytest
 import torch
@@ -36,7 +36,7 @@ def from_layout(t, layout):
     return t.permute(3, 0, 1, 2)
 
 
-@pytest.mark.parametrize("dtype", [ops.F32, ops.BF16])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16, ops.BF16])
 @pytest.mark.parametrize("layer", range(len(synth.VGG16_CONV)))
 def test_full_size_layer_all_layouts(oracle, layer, dtype):
     C, K, H = synth.VGG16_CONV[layer]
