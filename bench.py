@@ -175,7 +175,7 @@ def main():
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    st = ops.stage_times()
+    st = ops.stage_stats()
     ops.stage_timing(False)
 
     per_step = {k: (v[0] / args.steps) for k, v in st.items()}        # ms per step, summed over layers
@@ -204,10 +204,14 @@ def main():
             gbs = nbytes / (per_step[name] * 1e-3) / 1e9
             stages[name] = {"ms": round(per_step[name], 4), "GBps": round(gbs, 1),
                             "frac_hbm": round(gbs / HBM_PEAK_GBS, 3)}
+            if not multi:                          # one span per step: shortest and longest of the K steps
+                stages[name].update(min_ms=round(st[name][1], 4), max_ms=round(st[name][2], 4))
     gemm_ms = per_step["gemm"]
     achieved = gemm_flops / (gemm_ms * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[args.dtype]
     stages["gemm"] = {"ms": round(gemm_ms, 4), "TFLOPs": round(achieved, 2)}
+    if not multi:
+        stages["gemm"].update(min_ms=round(st["gemm"][1], 4), max_ms=round(st["gemm"][2], 4))
     kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
               "staged_f4": "gemm_128x128_kernel", "direct": "direct_small_c_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"

@@ -57,6 +57,7 @@ SYMBOLS = {
     "wino_layout_transform": (_i, [_i] * 7 + [_vp, _vp, _vp]),
     "wino_stage_timing": (_i, [_i]),
     "wino_stage_times": (_i, [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(_l)]),
+    "wino_stage_stats": (_i, [ctypes.POINTER(ctypes.c_float)] * 3 + [ctypes.POINTER(_l)]),
     "wino_warmup": (_i, []),
     "wino_sync": (_i, [_vp]),
     "wino_last_error": (ctypes.c_char_p, []),

@@ -866,26 +866,39 @@ int wino_stage_timing(int enable) {
     return WINO_OK;
 }
 
-int wino_stage_times(float* ms, long* calls) {
-    if (!ms || !calls) return fail(WINO_ERR_INVALID, "null pointer");
+int wino_stage_stats(float* sum_ms, float* min_ms, float* max_ms, long* calls) {
+    if (!sum_ms || !calls) return fail(WINO_ERR_INVALID, "null pointer");
     std::vector<StageSpan> spans;
     {
         std::lock_guard<std::mutex> lk(g_spans_mu);
         spans.swap(g_spans);
     }
-    for (int i = 0; i < WINO_NUM_STAGES; ++i) { ms[i] = 0.f; calls[i] = 0; }
+    for (int i = 0; i < WINO_NUM_STAGES; ++i) {
+        sum_ms[i] = 0.f;
+        calls[i] = 0;
+        if (min_ms) min_ms[i] = 0.f;
+        if (max_ms) max_ms[i] = 0.f;
+    }
     int rc = WINO_OK;
     for (auto& sp : spans) {
         float t = 0.f;
         hipError_t e = hipEventSynchronize(sp.b);
         if (e == hipSuccess) e = hipEventElapsedTime(&t, sp.a, sp.b);
         if (e != hipSuccess) rc = fail(WINO_ERR_HIP, "stage timing: %s", hipGetErrorString(e));
-        else { ms[sp.stage] += t; calls[sp.stage] += 1; }
+        else {
+            const int s = sp.stage;
+            if (min_ms) min_ms[s] = calls[s] == 0 ? t : std::min(min_ms[s], t);
+            if (max_ms) max_ms[s] = calls[s] == 0 ? t : std::max(max_ms[s], t);
+            sum_ms[s] += t;
+            calls[s] += 1;
+        }
         (void)hipEventDestroy(sp.a);
         (void)hipEventDestroy(sp.b);
     }
     return rc;
 }
+
+int wino_stage_times(float* ms, long* calls) { return wino_stage_stats(ms, nullptr, nullptr, calls); }
 
 // ---- conv stack ------------------------------------------------------------------------------------
 struct wino_stack {

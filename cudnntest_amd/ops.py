@@ -118,6 +118,16 @@ def stage_times():
     return {name: (float(ms[i]), int(calls[i])) for i, name in enumerate(STAGES)}
 
 
+def stage_stats():
+    """{stage: (total_ms, min_ms, max_ms, spans)} since the last call: the average / minimum / maximum of the
+    reference's per-stage harness (delayTest/testbench/src/M1/M1Test.h:100-151) from the library's own events."""
+    import ctypes
+    tot, lo, hi = ((ctypes.c_float * 4)() for _ in range(3))
+    calls = (ctypes.c_long * 4)()
+    _lib.check(_lib.load().wino_stage_stats(tot, lo, hi, calls), "wino_stage_stats")
+    return {name: (float(tot[i]), float(lo[i]), float(hi[i]), int(calls[i])) for i, name in enumerate(STAGES)}
+
+
 # ---- whole layer -------------------------------------------------------------
 
 def _out_for(dst, x, N, K, Ho, Wo, pool, out):

@@ -176,7 +176,10 @@ int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int 
  * While enabled, wino_conv / wino_conv_prepared bracket every stage they launch
  * with a pair of HIP events on the launch stream.  wino_stage_times() waits for
  * the recorded events, returns the accumulated milliseconds and number of spans
- * per stage (arrays of WINO_NUM_STAGES) and forgets them. */
+ * per stage (arrays of WINO_NUM_STAGES) and forgets them; wino_stage_stats() does
+ * the same and also returns the shortest and longest span of every stage (the
+ * average / minimum / maximum line that the reference's timing harness prints per
+ * configuration, delayTest/testbench/src/M1/M1Test.h:100-151); min_ms and max_ms may be null. */
 typedef enum {
     WINO_STAGE_FILTER = 0,
     WINO_STAGE_INPUT = 1,
@@ -186,6 +189,7 @@ typedef enum {
 } wino_stage_t;
 int wino_stage_timing(int enable);
 int wino_stage_times(float *ms, long *calls);
+int wino_stage_stats(float *sum_ms, float *min_ms, float *max_ms, long *calls);
 
 /* ---- a stack of 3x3 convolution layers with cached filter transforms -------------------------
  * The convolution part of the reference's network driver, classify_example_modified
