@@ -45,6 +45,10 @@ int fail(int code, const char* fmt, ...) {
 bool valid_layout(int l) { return l == WINO_NCHW || l == WINO_NHWC || l == WINO_CHWN; }
 bool valid_dtype(int d) { return d == WINO_F32 || d == WINO_F16 || d == WINO_BF16; }
 bool valid_porder(int o) { return o == WINO_PRODUCT_KP || o == WINO_PRODUCT_PK; }
+// Winograd-domain operands (U, V, M) move as 16-byte vectors, partly by direct-to-LDS loads: their addresses
+// must be 16-byte aligned (every hipMalloc'ed buffer is); plain tensors need their element's alignment only.
+bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+size_t elem_bytes(int dtype) { return dtype == WINO_F32 ? 4 : 2; }
 bool valid_order(int o) { return o == WINO_TILES_BATCH_MAJOR || o == WINO_TILES_BATCH_MINOR; }
 
 // ---- scratch arena: one grow-only allocation per device ------------------------
@@ -553,6 +557,10 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_DIRECT) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
     if (!x || (!w && !Upre) || !y) return fail(WINO_ERR_INVALID, "null tensor pointer");
+    if (misaligned(x, elem_bytes(dtype)) || misaligned(w, elem_bytes(dtype)) || misaligned(y, elem_bytes(dtype)) ||
+        misaligned(bias, elem_bytes(dtype)))
+        return fail(WINO_ERR_INVALID, "tensor pointer not aligned to its element size");
+    if (misaligned(Upre, 16)) return fail(WINO_ERR_INVALID, "transformed filters must be 16-byte aligned");
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
@@ -684,6 +692,7 @@ int wino_set_workspace(void* ptr, size_t bytes) {
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return fail(WINO_ERR_UNSUPPORTED, "device index %d out of range", dev);
     if (ptr && bytes == 0) return fail(WINO_ERR_INVALID, "workspace pointer with zero size");
+    if (misaligned(ptr, 256)) return fail(WINO_ERR_INVALID, "workspace must be 256-byte aligned");
     if (ptr && bytes < kCounterBytes) return fail(WINO_ERR_WORKSPACE, "workspace smaller than %zu bytes", kCounterBytes);
     if (ptr) HIP_TRY(hipMemset(ptr, 0, kCounterBytes));   // arrival counters (blocking, like every allocation)
     std::lock_guard<std::mutex> lk(g_arena_mu);
@@ -696,6 +705,7 @@ int wino_set_workspace(void* ptr, size_t bytes) {
 int wino_filter_transform(int layout, int dtype, int K, int C, const void* w, void* U, void* stream) {
     if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
     if (!w || !U) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(U, 16)) return fail(WINO_ERR_INVALID, "transformed filters must be 16-byte aligned");
     if (K <= 0 || C <= 0) return fail(WINO_ERR_INVALID, "bad filter bank K=%d C=%d", K, C);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     const int Kp = (int)round_up(K, kKPad), Cp = (int)round_up(C, c_pad(dtype));
@@ -707,6 +717,7 @@ int wino_input_transform(int layout, int dtype, int tile_order, int N, int C, in
     if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!x || !V) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(V, 16)) return fail(WINO_ERR_INVALID, "transformed input must be 16-byte aligned");
     Geometry g;
     if (!make_geometry(dtype, N, C, 1, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d H=%d W=%d pad=%d", N, C, H, W, pad);
@@ -718,6 +729,8 @@ int wino_batched_gemm(int dtype, int product_order, int C, int K, long P, const 
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(U, 16) || misaligned(V, 16) || misaligned(Mo, 16))
+        return fail(WINO_ERR_INVALID, "GEMM operands must be 16-byte aligned");
     if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
     return launch_gemm(16, dtype, product_order, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad), round_up(P, kPPad), U, V, Mo,
                        (hipStream_t)stream);
@@ -729,6 +742,7 @@ int wino_output_transform(int layout, int dtype, int tile_order, int product_ord
     if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!Mo || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(Mo, 16)) return fail(WINO_ERR_INVALID, "the product tensor must be 16-byte aligned");
     if (N <= 0 || K <= 0 || Ho <= 0 || Wo <= 0)
         return fail(WINO_ERR_INVALID, "bad shape N=%d K=%d Ho=%d Wo=%d", N, K, Ho, Wo);
     const long P = (long)N * ((Ho + 1) / 2) * ((Wo + 1) / 2);
@@ -744,6 +758,7 @@ int wino_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int 
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!U || !V || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(U, 16) || misaligned(V, 16)) return fail(WINO_ERR_INVALID, "GEMM operands must be 16-byte aligned");
     Geometry g;
     // geometry from the output size: pad 1 keeps H == Ho
     if (!make_geometry(dtype, N, C, K, Ho, Wo, 1, &g))
@@ -817,6 +832,7 @@ int wino_f4_filter_transform(int layout, int dtype, int K, int C, const void* w,
     if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (!w || !U) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(U, 16)) return fail(WINO_ERR_INVALID, "transformed filters must be 16-byte aligned");
     if (K <= 0 || C <= 0) return fail(WINO_ERR_INVALID, "bad filter bank K=%d C=%d", K, C);
     const int Kp = (int)round_up(K, kKPad), Cp = (int)round_up(C, c_pad(dtype));
     DISPATCH_DTYPE(dtype, launch_f4_filter<T>(layout, K, C, Kp, Cp, w, U, (hipStream_t)stream));
@@ -828,6 +844,7 @@ int wino_f4_input_transform(int layout, int dtype, int tile_order, int N, int C,
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!x || !V) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(V, 16)) return fail(WINO_ERR_INVALID, "transformed input must be 16-byte aligned");
     Geometry g;
     if (!make_geometry(dtype, N, C, 1, H, W, pad, &g, 4))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d H=%d W=%d pad=%d", N, C, H, W, pad);
@@ -839,6 +856,8 @@ int wino_f4_batched_gemm(int dtype, int product_order, int C, int K, long P, con
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!U || !V || !Mo) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(U, 16) || misaligned(V, 16) || misaligned(Mo, 16))
+        return fail(WINO_ERR_INVALID, "GEMM operands must be 16-byte aligned");
     if (C <= 0 || K <= 0 || P <= 0) return fail(WINO_ERR_INVALID, "bad GEMM shape C=%d K=%d P=%ld", C, K, P);
     return launch_gemm(36, dtype, product_order, (int)round_up(C, c_pad(dtype)), (int)round_up(K, kKPad),
                        round_up(P, kPPad), U, V, Mo, (hipStream_t)stream);
@@ -851,6 +870,7 @@ int wino_f4_output_transform(int layout, int dtype, int tile_order, int product_
     if (!valid_porder(product_order)) return fail(WINO_ERR_INVALID, "unknown product order %d", product_order);
     if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
     if (!Mo || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(Mo, 16)) return fail(WINO_ERR_INVALID, "the product tensor must be 16-byte aligned");
     if (N <= 0 || K <= 0 || Ho <= 0 || Wo <= 0)
         return fail(WINO_ERR_INVALID, "bad shape N=%d K=%d Ho=%d Wo=%d", N, K, Ho, Wo);
     const long P = (long)N * ((Ho + 3) / 4) * ((Wo + 3) / 4);

@@ -14,6 +14,11 @@
  *   CHWN     [C][H][W][N]                [C][3][3][K]   comparison/wrapedConv_CHWN.cuh:288
  * The convolution is a stride-1 cross-correlation with `pad` rows/columns of
  * zeros on every side; the output is Ho x Wo = (H+2*pad-2) x (W+2*pad-2).
+ *
+ * Alignment: x, w, bias and y need only the alignment of their element type (any
+ * view of a device allocation works).  The Winograd-domain operands U, V and the
+ * product tensor move as 16-byte vectors and must be 16-byte aligned, a caller's
+ * workspace 256-byte aligned; anything else is refused with WINO_ERR_INVALID.
  */
 #ifndef WINO_AMD_H
 #define WINO_AMD_H

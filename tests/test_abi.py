@@ -76,6 +76,18 @@ def test_invalid_arguments_are_rejected_without_a_gpu():
     assert L.wino_output_transform(3, 0, 0, 0, 0, 1, 1, 4, 4, one, one, None) == -1
     assert L.wino_layout_transform(0, 1, 0, 1, 1, 0, 4, one, one, None) == -1
     assert L.wino_workspace_bytes(0, 0, 1, 1, 4, 4, 1) == 0
+    # alignment: tensors to their element size, Winograd-domain operands to 16 bytes
+    odd, off8 = ctypes.c_void_p(18), ctypes.c_void_p(24)
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1, odd, one, one, None) == -1
+    assert b"aligned" in L.wino_last_error()
+    assert L.wino_conv(0, 0, 1, 0, 0, 1, 1, 1, 4, 4, 1, one, one, ctypes.c_void_p(17), None) == -1
+    assert L.wino_conv_prepared(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1, one, off8, one, None) == -1
+    assert b"16-byte" in L.wino_last_error()
+    assert L.wino_filter_transform(0, 0, 4, 4, one, off8, None) == -1
+    assert L.wino_input_transform(0, 0, 0, 1, 1, 4, 4, 1, one, off8, None) == -1
+    assert L.wino_batched_gemm(0, 0, 4, 4, 4, one, off8, one, None) == -1
+    assert L.wino_output_transform(0, 0, 0, 0, 0, 1, 1, 4, 4, off8, one, None) == -1
+    assert L.wino_gemm_output(0, 0, 0, 0, 1, 4, 4, 4, 4, off8, one, one, None) == -1
 
 
 def test_operator_layer_refuses_cpu_tensors():

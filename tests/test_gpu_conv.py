@@ -160,3 +160,35 @@ def test_epilogue_gemm_with_a_cut_up_last_round(oracle, layout, dtype, N):
     for _ in range(3):
         assert torch.equal(ops.conv(xfd, wfd, 1, layout, algo=ops.ALGO_EPILOGUE), first)
     assert torch.equal(ops.conv(xd, wd, 1, layout, algo=ops.ALGO_EPILOGUE, relu=True, bias=bd), got)
+
+
+def _view_at(t, shift):
+    """A contiguous copy of `t` that starts `shift` elements into its allocation (element-aligned only)."""
+    flat = torch.empty(t.numel() + shift, dtype=t.dtype, device=t.device)
+    v = flat[shift:].view(t.shape)
+    v.copy_(t)
+    return v
+
+
+@pytest.mark.parametrize("algo", [ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_AUTO])
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16])
+@pytest.mark.parametrize("C", [32, 3])
+def test_tensors_that_are_only_element_aligned(C, dtype, layout, algo):
+    """x, w, bias and y may be any view of an allocation: only the alignment of the element type is
+    required.  The vector paths either test the address or use loads that need no alignment; the result
+    must be bit-identical with that of 256-byte aligned tensors."""
+    from gpu_util import TORCH_DT
+    N, K, H = 2, 64, 16
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = (torch.rand(ops.act_shape(layout, N, C, H, H), device="cuda", generator=g) - 0.5).to(TORCH_DT[dtype])
+    wshape = {ops.NCHW: (K, C, 3, 3), ops.NHWC: (K, 3, 3, C), ops.CHWN: (C, 3, 3, K)}[layout]
+    w = (torch.randn(wshape, device="cuda", generator=g) * 0.1).to(TORCH_DT[dtype])
+    b = torch.randn(K, device="cuda", generator=g).to(TORCH_DT[dtype])
+    want = ops.conv(x, w, 1, layout, algo=algo, bias=b, relu=True)
+    for shift in (1, 3):
+        out = _view_at(torch.zeros_like(want), shift)
+        got = ops.conv(_view_at(x, shift), _view_at(w, shift), 1, layout, algo=algo, bias=_view_at(b, shift),
+                       relu=True, out=out)
+        assert got.data_ptr() % 16 != 0
+        assert torch.equal(got, want), (shift, (got.float() - want.float()).abs().max().item())
