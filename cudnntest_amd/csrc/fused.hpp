@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
                                                             T* __restrict__ y, ActStrides xs, ActStrides ys, int N,
                                                             int C, int K, int H, int W, int pad, int Ho, int Wo,
                                                             int th, int tw, long P, int Cp, int Kp, int order,
-                                                            Epilogue ep, int kTiles, int pTiles) {
+                                                            Epilogue ep, int kTiles, int pTiles, int xcd_map) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     constexpr int NV = 2 * NVG;                // channel vectors per stage and coordinate
@@ -72,7 +72,8 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     // Workgroup ids go round-robin to the 8 XCDs.  The ids of one XCD walk the filter tiles of a
     // tile patch first (they share its raw input), then CONSECUTIVE tile patches: neighbouring
     // patches are neighbouring tile rows, whose raw input rows overlap, and an XCD has its own L2.
-    const int xcd = b & 7, jb = b >> 3;
+    // (With few tile patches that order would leave XCDs idle: the host then asks for the plain one.)
+    const int xcd = xcd_map ? b & 7 : 0, jb = xcd_map ? b >> 3 : b;
     const int ktile = jb % kTiles;
     const int ptile = xcd * ((pTiles + 7) / 8) + jb / kTiles;
     if (ptile >= pTiles) return;

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
                                                            int Ho, int Wo, int th, int tw, long P, int Cp,
                                                            int Kp, long Pp, int order, Epilogue ep, int kTiles,
                                                            int pTiles, int main_ids, float* __restrict__ tail_part,
-                                                           int* __restrict__ tail_cnt) {
+                                                           int* __restrict__ tail_cnt, int xcd_map) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     constexpr int NV = 2 * NVG;
@@ -224,9 +224,12 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
     const int tq = TAIL ? (tb >> 5) * 8 + (tb & 7) : 0;
     const int trow = TAIL ? (tb >> 3) & 3 : 0;
     const int b = TAIL ? main_ids + tq : (int)blockIdx.x;
-    const int xcd = b & 7, jb = b >> 3;
+    // xcd_map: ids go round-robin to the 8 XCDs, and the ids of one XCD walk the filter tiles of a tile patch
+    // before the next patch (one XCD's L2 serves the patch's V to all of them).  With few tile patches that
+    // would leave XCDs idle (one patch: seven of eight), so the host then asks for the plain order.
+    const int xcd = xcd_map ? b & 7 : 0, jb = xcd_map ? b >> 3 : b;
     const int ktile = jb % kTiles;
-    const int ptile = (jb / kTiles) * 8 + xcd;
+    const int ptile = (jb / kTiles) * (xcd_map ? 8 : 1) + xcd;
     if (ptile >= pTiles) return;
     const int k0 = ktile * GO_T;
     const long p0 = (long)ptile * GO_T;
@@ -383,7 +386,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rows_kernel(const T* __restrict__
 template <typename T, int NV, bool PK, int RING>
 __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__ U, const T* __restrict__ V,
                                                                 float* __restrict__ Mo, int Cp, int Kp, long Pp,
-                                                                int kTiles, int pTiles) {
+                                                                int kTiles, int pTiles, int split_chunks, int xcd_map) {
     typedef typename Mma<T>::vec vec;
     constexpr int CV = ChanVec<T>::n;
     static_assert(RING >= 2 && RING <= 4, "ring depth");
@@ -399,16 +402,19 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
     };
     const int xi = blockIdx.y;
     const int b = blockIdx.x;
-    const int xcd = b & 7, jj = b >> 3;
+    const int xcd = xcd_map ? b & 7 : 0, jj = xcd_map ? b >> 3 : b;     // as in gemm_rows_kernel
     const int ktile = jj % kTiles;
-    const int ptile = (jj / kTiles) * 8 + xcd;
+    const int ptile = (jj / kTiles) * (xcd_map ? 8 : 1) + xcd;
     if (ptile >= pTiles) return;
     const long p0 = (long)ptile * GEMM_BN;
     const int k0 = ktile * GEMM_BM;
     const int CQ = Cp / CV;
-    const int nch = CQ / NV;
-    const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
-    const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + p0;
+    // blockIdx.z: which run of split_chunks stages (NV channel vectors each) of the reduction this workgroup
+    // sums; its product goes to copy blockIdx.z of Mo (the host makes every run non-empty)
+    const int c_first = blockIdx.z * split_chunks;
+    const int nch = min(split_chunks, CQ / NV - c_first);
+    const vec* Ub = reinterpret_cast<const vec*>(U) + ((size_t)xi * CQ + (size_t)c_first * NV) * Kp + k0;
+    const vec* Vb = reinterpret_cast<const vec*>(V) + ((size_t)xi * CQ + (size_t)c_first * NV) * Pp + p0;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -485,7 +491,7 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
     if (RING > 3 && s + 2 < nch) iteration(std::integral_constant<int, 2>{});
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
-    float* Mb = Mo + (size_t)xi * Kp * Pp;
+    float* Mb = Mo + ((size_t)blockIdx.z * gridDim.y + xi) * Kp * Pp;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll

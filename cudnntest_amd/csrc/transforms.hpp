@@ -464,7 +464,7 @@ __global__ __launch_bounds__(256) void output_transform_generic_kernel(const flo
                                                                         T* __restrict__ y, ActStrides s, int N,
                                                                         int K, int Ho, int Wo, int th, int tw,
                                                                         long P, long Pp, int Kp, int order,
-                                                                        Epilogue ep) {
+                                                                        Epilogue ep, int splits) {
     const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const int k = blockIdx.y;
     if (p >= P || k >= K) return;
@@ -473,6 +473,9 @@ __global__ __launch_bounds__(256) void output_transform_generic_kernel(const flo
     float m[16];
 #pragma unroll
     for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];
+    for (int sp = 1; sp < splits; ++sp)          // partial products of a reduction cut into runs, in a fixed order
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi) m[xi] += mp[((size_t)sp * 16 + xi) * plane];
     float o[2][2];
     output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
     int n, ty, tx;
@@ -487,7 +490,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void output_transform_pk_kernel(const float* __restrict__ Mo, T* __restrict__ y,
                                                                    ActStrides s, int N, int K, int Ho, int Wo, int th,
                                                                    int tw, long P, long Pp, int Kp, int order,
-                                                                   Epilogue ep) {
+                                                                   Epilogue ep, int splits) {
     const int k = blockIdx.x * blockDim.x + threadIdx.x;
     const long p = (long)blockIdx.y * blockDim.y + threadIdx.y;
     if (k >= K || p >= P) return;
@@ -496,6 +499,9 @@ __global__ __launch_bounds__(256) void output_transform_pk_kernel(const float* _
     float m[16];
 #pragma unroll
     for (int xi = 0; xi < 16; ++xi) m[xi] = mp[xi * plane];
+    for (int sp = 1; sp < splits; ++sp)
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi) m[xi] += mp[((size_t)sp * 16 + xi) * plane];
     float o[2][2];
     output_tile_transform(m, o[0][0], o[0][1], o[1][0], o[1][1]);
     int n, ty, tx;

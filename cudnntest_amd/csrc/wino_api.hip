@@ -132,6 +132,29 @@ struct Scratch {
 // The arena opens with the arrival counters of the epilogue GEMM's tail workgroups (zero whenever no
 // kernel is running); U, V and the product follow.  The product region doubles as the tail workgroups'
 // partial sums: the epilogue path has no product tensor.
+// Whether a launch orders its workgroup ids by XCD (8 tile patches side by side, one per XCD): only if that keeps
+// the XCDs evenly loaded.  With pTiles tile patches the padded order has ceil(pTiles/8)*8 slots; it is used when
+// at most an eighth of them is empty, otherwise ids walk the patches in plain order and the hardware's round-robin
+// spreads them (a layer with one tile patch would otherwise run on one XCD: 32 of 256 CUs).
+bool xcd_map_ok(int pTiles) {
+    const int padded = (pTiles + 7) / 8 * 8;
+    return pTiles >= 8 && (padded - pTiles) * 8 <= padded;
+}
+
+// How many runs the staged GEMM's channel reduction is cut into.  A layer with fewer 128x128 workgroups than CUs
+// leaves CUs idle while each workgroup walks the whole reduction, so the reduction is cut until there is one
+// workgroup per CU (more than one per CU measured slower again: N=1, C=K=512, H=14 in fp32 takes 37 us uncut,
+// 22 us in 2 runs, 16 us in 4, 23 us in 6, 20 us in 8), each run at least 4 stages long.  The partial products
+// are summed by the output transform in a fixed order.
+int gemm_splits(int dtype, int Cp, int Kp, long Pp) {
+    const long wgs = 16L * (Kp / GEMM_BM) * (Pp / GEMM_BN);
+    const int chunks = Cp / c_pad(dtype);          // stages of the reduction: 4 channel vectors each
+    const long s = std::min<long>(256 / std::max<long>(wgs, 1), chunks / 4);
+    if (s <= 1) return 1;
+    const int per = (int)((chunks + s - 1) / s);
+    return (chunks + per - 1) / per;
+}
+
 Scratch scratch_layout(const Geometry& g, int dtype) {
     const size_t es = dtype_size(dtype);
     const size_t nxi = (size_t)(g.m + 2) * (g.m + 2);
@@ -140,7 +163,8 @@ Scratch scratch_layout(const Geometry& g, int dtype) {
     s.u_off = kCounterBytes;
     s.v_off = s.u_off + al(nxi * (size_t)g.Cp * g.Kp * es);
     s.m_off = s.v_off + al(nxi * (size_t)g.Cp * g.Pp * es);
-    s.total = s.m_off + al(nxi * (size_t)g.Kp * g.Pp * sizeof(float));
+    const size_t copies = g.m == 2 ? (size_t)gemm_splits(dtype, g.Cp, g.Kp, g.Pp) : 1;
+    s.total = s.m_off + al(copies * nxi * (size_t)g.Kp * g.Pp * sizeof(float));
     return s;
 }
 
@@ -216,7 +240,8 @@ inline ActStrides out_strides(int layout, unsigned flags, int N, int K, int Ho, 
 
 template <typename T>
 int launch_output_transform(int layout, int order, int porder, unsigned flags, const void* bias, int N, int K, int Ho,
-                            int Wo, int Kp, long P, long Pp, const float* Mo, void* y, hipStream_t st) {
+                            int Wo, int Kp, long P, long Pp, const float* Mo, void* y, hipStream_t st,
+                            int splits = 1) {
     const int th = (Ho + 1) / 2, tw = (Wo + 1) / 2;
     const Epilogue ep = make_epilogue(flags, bias);
     if (porder == WINO_PRODUCT_PK) {
@@ -224,41 +249,46 @@ int launch_output_transform(int layout, int order, int porder, unsigned flags, c
         while (bx < K && bx < 256) bx *= 2;
         dim3 block(bx, 256 / bx), grid((K + bx - 1) / bx, (unsigned)((P + block.y - 1) / block.y));
         hipLaunchKernelGGL(output_transform_pk_kernel<T>, grid, block, 0, st, Mo, (T*)y,
-                           out_strides(layout, flags, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, ep);
+                           out_strides(layout, flags, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, ep, splits);
     } else {
         dim3 grid((unsigned)((P + 255) / 256), K), block(256);
         hipLaunchKernelGGL(output_transform_generic_kernel<T>, grid, block, 0, st, Mo, (T*)y,
-                           out_strides(layout, flags, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, ep);
+                           out_strides(layout, flags, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, ep, splits);
     }
     LAUNCH_CHECK("output_transform");
     return WINO_OK;
 }
 
 template <typename T, int NV, bool PK>
-int launch_gemm_t(int nxi, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, hipStream_t st) {
+int launch_gemm_t(int nxi, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo, int splits,
+                  hipStream_t st) {
     const int kTiles = Kp / GEMM_BM, pTiles = (int)(Pp / GEMM_BN);
-    dim3 grid((unsigned)((pTiles + 7) / 8 * 8 * kTiles), nxi), block(256);
+    const int chunks = Cp / (NV * ChanVec<T>::n), per = (chunks + splits - 1) / splits;
+    if (splits < 1 || (long)per * (splits - 1) >= chunks)
+        return fail(WINO_ERR_INVALID, "reduction of %d stages cannot be cut into %d runs", chunks, splits);
+    const bool xm = xcd_map_ok(pTiles);
+    dim3 grid((unsigned)((xm ? (pTiles + 7) / 8 * 8 : pTiles) * kTiles), nxi, splits), block(256);
     constexpr int RING = sizeof(T) == 4 ? 4 : 2;     // from measurements, see gemm.hpp
     hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK, RING>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp,
-                       Kp, Pp, kTiles, pTiles);
+                       Kp, Pp, kTiles, pTiles, per, xm ? 1 : 0);
     LAUNCH_CHECK("batched_gemm");
     return WINO_OK;
 }
 
 int launch_gemm(int nxi, int dtype, int porder, int Cp, int Kp, long Pp, const void* U, const void* V, float* Mo,
-                hipStream_t st) {
+                hipStream_t st, int splits = 1) {
     // slab per barrier: 4 channel vectors = 16 channels (fp32) or 32 (16-bit); Cp is a multiple of that
     const bool pk = porder == WINO_PRODUCT_PK;
     switch (dtype) {
     case WINO_F32:
-        return pk ? launch_gemm_t<float, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, st)
-                  : launch_gemm_t<float, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<float, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, splits, st)
+                  : launch_gemm_t<float, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, splits, st);
     case WINO_F16:
-        return pk ? launch_gemm_t<f16_t, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, st)
-                  : launch_gemm_t<f16_t, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<f16_t, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, splits, st)
+                  : launch_gemm_t<f16_t, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, splits, st);
     case WINO_BF16:
-        return pk ? launch_gemm_t<bf16_t, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, st)
-                  : launch_gemm_t<bf16_t, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, st);
+        return pk ? launch_gemm_t<bf16_t, 4, true>(nxi, Cp, Kp, Pp, U, V, Mo, splits, st)
+                  : launch_gemm_t<bf16_t, 4, false>(nxi, Cp, Kp, Pp, U, V, Mo, splits, st);
     }
     return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -293,11 +323,12 @@ int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geomet
             (size_t)tail_ids * 4 * 64 * 256 * sizeof(float) > ts.part_bytes)
             tail_groups = 0;
     }
-    const int main_ids = (pGroups - tail_groups) * group;
+    const bool xm = tail_groups > 0 || xcd_map_ok(pTiles);      // (a cut-up last round implies hundreds of patches)
+    const int main_ids = xm ? (pGroups - tail_groups) * group : pTiles * kTiles;
     hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING>), dim3((unsigned)(main_ids + tail_groups * group * 4)),
                        dim3(256), 0, st, (const T*)U, (const T*)V, (T*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P,
                        g.Cp, g.Kp, g.Pp, order, ep, kTiles, pTiles, main_ids, tail_groups ? ts.part : nullptr,
-                       tail_groups ? ts.cnt : nullptr);
+                       tail_groups ? ts.cnt : nullptr, xm ? 1 : 0);
     LAUNCH_CHECK("gemm_rows");
     return WINO_OK;
 }
@@ -327,11 +358,12 @@ int launch_fused_rows_t(int src, int dst, int order, unsigned flags, const void*
     const int kTiles = (g.K + GO_T - 1) / GO_T;
     const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
     const int pGroups = (pTiles + 7) / 8;
-    dim3 grid((unsigned)(pGroups * 8 * kTiles)), block(256);
+    const bool xm = xcd_map_ok(pTiles);
+    dim3 grid((unsigned)((xm ? pGroups * 8 : pTiles) * kTiles)), block(256);
     hipLaunchKernelGGL((fused_rows_kernel<T, SWAP, XM, NVG>), grid, block, 0, st, (const T*)x, (const T*)U, (T*)y,
                        act_strides(src, g.N, g.C, g.H, g.W), out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo), g.N, g.C, g.K,
                        g.H, g.W, g.pad, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, order, make_epilogue(flags, bias),
-                       kTiles, pTiles);
+                       kTiles, pTiles, xm ? 1 : 0);
     LAUNCH_CHECK("fused_rows");
     return WINO_OK;
 }
@@ -508,7 +540,7 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     if (!fused_ok) return WINO_ALGO_EPILOGUE;
     if (nhwc) {
         if (g.C >= 16 && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
-    } else if (g.C <= 64 && g.K <= 64) {
+    } else if (g.C <= 64 && g.K <= 64 && patches >= 2048) {   // (fewer patches: measured 5-19 % behind EPILOGUE)
         return WINO_ALGO_FUSED;
     }
     return WINO_ALGO_EPILOGUE;
@@ -617,13 +649,14 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         return launch_gemm_out(dst, dtype, order, flags, bias, g, U, V, y, ts, st);
     }
     const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
+    const int splits = gemm_splits(dtype, g.Cp, g.Kp, g.Pp);
     {
         StageScope t(WINO_STAGE_GEMM, st);
-        rc = launch_gemm(16, dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
+        rc = launch_gemm(16, dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st, splits);
         if (rc) return rc;
     }
     StageScope t(WINO_STAGE_OUTPUT, st);
-    DISPATCH_DTYPE(dtype, launch_output_transform<T>(dst, order, porder, flags, bias, N, K, g.Ho, g.Wo, g.Kp, g.P, g.Pp, Mo, y, st));
+    DISPATCH_DTYPE(dtype, launch_output_transform<T>(dst, order, porder, flags, bias, N, K, g.Ho, g.Wo, g.Kp, g.P, g.Pp, Mo, y, st, splits));
 }
 
 __global__ void warmup_kernel() {}

@@ -192,3 +192,22 @@ def test_tensors_that_are_only_element_aligned(C, dtype, layout, algo):
                        relu=True, out=out)
         assert got.data_ptr() % 16 != 0
         assert torch.equal(got, want), (shift, (got.float() - want.float()).abs().max().item())
+
+
+@pytest.mark.parametrize("shape", [(1, 512, 128, 14, 14), (1, 144, 130, 10, 12), (2, 208, 64, 7, 7), (1, 256, 512, 28, 28)])
+def test_staged_gemm_with_its_reduction_cut_into_runs(oracle, shape):
+    """Layers with few workgroups have the channel reduction of the staged GEMM cut into runs (several partial
+    products, summed by the output transform): deep reductions on small images, with run lengths that
+    do and do not divide the channel count, both product orientations.  Integers: bit-exact."""
+    N, C, K, H, W = shape
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=sum(shape), integer=True)
+    want = oracle.direct_conv(x, w, 1)
+    for dst in LAYOUTS:
+        got = host(ops.conv(dev(x), dev(w), 1, ops.NCHW, dst, ops.ALGO_STAGED, relu=True))
+        assert np.array_equal(got, synth.act_to_layout(np.maximum(want, 0), dst)), dst
+    for dtype in (ops.F16, ops.BF16):
+        xf, wf = synth.conv_inputs(N, C, K, H, W, seed=7 + sum(shape))
+        got = host(ops.conv(dev(xf, dtype), dev(wf, dtype), 1, ops.NCHW, ops.NCHW, ops.ALGO_STAGED))
+        from gpu_util import rounded
+        ref = oracle.direct_conv(rounded(xf, dtype, oracle), rounded(wf, dtype, oracle), 1)
+        assert oracle.rel_l2(got, ref) <= TOL[dtype]
