@@ -19,6 +19,18 @@
  * view of a device allocation works).  The Winograd-domain operands U, V and the
  * product tensor move as 16-byte vectors and must be 16-byte aligned, a caller's
  * workspace 256-byte aligned; anything else is refused with WINO_ERR_INVALID.
+ *
+ * Concurrency: the whole-layer calls (wino_conv*, wino_stack_forward*) of one
+ * device share that device's scratch arena -- transformed operands, product
+ * tensor, arrival counters -- as the calls of the reference's driver share the
+ * three scratch buffers it allocates once and hands to every wrapper call
+ * (comparison/layoutCompare.cu:124-126, wrapedConv_NCHW.cuh:335).  Issue them in order on one
+ * stream, or serialise the streams yourself: two layers in flight at once on one
+ * device overwrite each other's scratch.  The stage entry points touch only the
+ * buffers they are given and may overlap freely.  Any entry point may be called
+ * from several host threads (the error text is per thread, the arena's
+ * bookkeeping is locked) under the same rule; growing the arena synchronises the
+ * device.
  */
 #ifndef WINO_AMD_H
 #define WINO_AMD_H
