@@ -817,6 +817,23 @@ int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int 
         else if (src == WINO_CHWN && dst == WINO_NCHW) d = {N, C * HW, 1, N, 0, C * HW, 0};
         else if (src == WINO_NHWC && dst == WINO_CHWN) d = {C, N, HW, HW * C, C, HW * N, N};
         else d = {N, C, HW, HW * N, N, HW * C, C};               // CHWN -> NHWC
+        // 2-byte elements move in pairs when every pair is 4-byte aligned on both sides
+        const bool pairs = dtype != WINO_F32 && d.nA % 2 == 0 && d.nB % 2 == 0 && d.sB % 2 == 0 && d.sR % 2 == 0 &&
+                           d.dA % 2 == 0 && d.dR % 2 == 0 && !misaligned(in, 4) && !misaligned(out, 4);
+        if (pairs) {
+            const int TA = d.nA <= 32 ? 32 : (d.nB <= 32 ? 256 : (d.nA <= 64 ? 64 : 128)), TB = 8192 / TA;
+            const long tilesA = (d.nA + TA - 1) / TA, tilesB = (d.nB + TB - 1) / TB;
+            const long blocks = tilesA * tilesB * d.nR;
+            if (blocks >= (1L << 31)) return fail(WINO_ERR_UNSUPPORTED, "layout transform: tensor too large");
+#define PERMUTE2(A, B)                                                                                          \
+    hipLaunchKernelGGL((permute_tiled_pairs_kernel<A, B>), dim3((unsigned)blocks), dim3(256), 0, st,              \
+                       (const uint16_t*)in, (uint16_t*)out, d, (int)tilesA, (int)tilesB)
+            if (TA == 32) PERMUTE2(32, 256); else if (TA == 256) PERMUTE2(256, 32);
+            else if (TA == 64) PERMUTE2(64, 128); else PERMUTE2(128, 64);
+#undef PERMUTE2
+            LAUNCH_CHECK("layout_transform");
+            return WINO_OK;
+        }
         const int TA = d.nA <= 32 ? 32 : (d.nB <= 32 ? 128 : 64), TB = 4096 / TA;
         const long tilesA = (d.nA + TA - 1) / TA, tilesB = (d.nB + TB - 1) / TB;
         const long blocks = tilesA * tilesB * d.nR;

@@ -135,3 +135,21 @@ def test_layout_transform(oracle, src, dst):
     xh = dev(xs, ops.F16)
     assert torch.equal(ops.layout_transform(xh, src, dst).cpu(),
                        torch.from_numpy(synth.act_to_layout(x, dst)).half())
+
+
+@pytest.mark.parametrize("shape", [(4, 6, 10, 8), (2, 64, 14, 14), (32, 66, 6, 6), (34, 130, 4, 2), (3, 8, 5, 6), (1, 2, 2, 2)])
+@pytest.mark.parametrize("src,dst", list(itertools.permutations(LAYOUTS, 2)))
+def test_layout_transform_two_byte_pairs(src, dst, shape):
+    """2-byte tensors with even extents move as 4-byte pairs (tiles of 8192 elements in four shapes); odd extents
+    and views that are only 2-byte aligned take the one-element kernel.  Bit-exact against torch's permute."""
+    N, C, H, W = shape
+    g = torch.Generator(device="cuda").manual_seed(N * 1000 + C)
+    x = torch.randn((N, C, H, W), device="cuda", generator=g).to(torch.bfloat16)
+    perm = {ops.NCHW: (0, 1, 2, 3), ops.NHWC: (0, 2, 3, 1), ops.CHWN: (1, 2, 3, 0)}
+    xs = x.permute(perm[src]).contiguous()
+    want = x.permute(perm[dst]).contiguous()
+    assert torch.equal(ops.layout_transform(xs, src, dst), want)
+    flat = torch.empty(xs.numel() + 1, dtype=xs.dtype, device="cuda")       # a view that starts on an odd element
+    odd = flat[1:].view(xs.shape)
+    odd.copy_(xs)
+    assert torch.equal(ops.layout_transform(odd, src, dst), want)
