@@ -70,12 +70,9 @@ __device__ __forceinline__ void output_tile_transform(const float m[16], float& 
 // padded (Cp/CV) x Kp rectangle and the padding is written as zeros, which is
 // what lets the GEMM run without masks on the reduction dimension.
 template <typename T>
-__global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restrict__ w, T* __restrict__ U,
-                                                                FltStrides s, int K, int C, int Kp, int Cp) {
+__device__ __forceinline__ void filter_transform_thread(const T* __restrict__ w, T* __restrict__ U, FltStrides s,
+                                                        int K, int C, int Kp, int Cp, int k, int cq) {
     constexpr int CV = ChanVec<T>::n;
-    const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    const int cq = blockIdx.y;
-    if (k >= Kp) return;
     float u[CV][16];
     float g[CV][3][3];
     // all CV channels of this vector exist, and the filter bank allows 16-byte loads
@@ -133,6 +130,23 @@ __global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restri
         store_chan_vec<T>(up + xi * plane, v);
     }
 }
+
+template <typename T>
+__global__ __launch_bounds__(256) void filter_transform_kernel(const T* __restrict__ w, T* __restrict__ U,
+                                                                FltStrides s, int K, int C, int Kp, int Cp) {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k < Kp) filter_transform_thread<T>(w, U, s, K, C, Kp, Cp, k, blockIdx.y);
+}
+
+// A filter bank to transform in the same launch as an input transform (w == nullptr: none).  A layer call
+// needs both before its GEMM, the filter transform is a few microseconds of latency-bound work, and a launch
+// of its own costs about as much again: the input transform's grid gets one more z-slice for it.
+struct FilterJob {
+    const void* w;
+    void* U;
+    FltStrides s;
+    int K, C, Kp, Cp;
+};
 
 // ---- input transform, layout-generic ---------------------------------------------
 // One thread per (tile p, channel vector cq), p fastest: every store is a
@@ -219,11 +233,17 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __restrict__ x, T* __restrict__ V, int N,
                                                                    int C, int H, int W, int pad, int th, int tw,
                                                                    long Pp, int Cp, int TR, int TC, int colBlocks,
-                                                                   int chunkLog2) {
+                                                                   int chunkLog2, FilterJob fj) {
     constexpr int CV = ChanVec<T>::n;
     extern __shared__ __attribute__((aligned(16))) unsigned char in_smem_raw[];
     T* in_smem = reinterpret_cast<T*>(in_smem_raw);   // [CV][rows][ldsW], the storage type
-    const int cq = blockIdx.y, n = blockIdx.z;
+    if (fj.w && blockIdx.z == 0) {
+        // the first z-slice transforms the filter bank: channel vector blockIdx.y (the layer's C), filters strided
+        for (int k = blockIdx.x * 256 + threadIdx.x; k < fj.Kp; k += gridDim.x * 256)
+            filter_transform_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, k, blockIdx.y);
+        return;
+    }
+    const int cq = blockIdx.y, n = fj.w ? blockIdx.z - 1 : blockIdx.z;
     const int rb = blockIdx.x / colBlocks, cb = blockIdx.x % colBlocks;
     const int ty0 = rb * TR, tx0 = cb * TC;
     const int rows = 2 * TR + 2;
