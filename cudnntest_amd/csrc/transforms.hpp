@@ -148,6 +148,18 @@ struct FilterJob {
     int K, C, Kp, Cp;
 };
 
+// The filter job of a launch whose grid.x was extended past in_blocks: those workgroups (all y) share the
+// Kp x Cp/CV threads of the job, filters fastest.
+template <typename T, int NT>
+__device__ __forceinline__ void filter_job_blocks(const FilterJob& fj, int in_blocks) {
+    constexpr int CV = ChanVec<T>::n;
+    const long work = (long)fj.Kp * (fj.Cp / CV);
+    const long nthreads = (long)(gridDim.x - in_blocks) * gridDim.y * NT;
+    for (long i = ((long)(blockIdx.x - in_blocks) * gridDim.y + blockIdx.y) * NT + threadIdx.x; i < work; i += nthreads)
+        filter_transform_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, (int)(i % fj.Kp),
+                                   (int)(i / fj.Kp));
+}
+
 // ---- input transform, layout-generic ---------------------------------------------
 // One thread per (tile p, channel vector cq), p fastest: every store is a
 // 16-byte vector and a wave's stores form a contiguous 1 KB run of V.  Reads go
@@ -158,8 +170,13 @@ template <typename T>
 __global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* __restrict__ x, T* __restrict__ V,
                                                                        ActStrides s, int N, int C, int H, int W,
                                                                        int pad, int th, int tw, long P, long Pp,
-                                                                       int Cp, int order) {
+                                                                       int Cp, int order, FilterJob fj,
+                                                                       int in_blocks) {
     constexpr int CV = ChanVec<T>::n;
+    if (fj.w && (int)blockIdx.x >= in_blocks) {
+        filter_job_blocks<T, 256>(fj, in_blocks);
+        return;
+    }
     const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const int cq = blockIdx.y;
     if (p >= P) return;
@@ -356,8 +373,12 @@ template <typename T, int TC, int NQ, int TR>
 __global__ __launch_bounds__(TC * NQ) void input_transform_nhwc_kernel(const T* __restrict__ x, T* __restrict__ V,
                                                                        int N, int C, int H, int W, int pad, int th,
                                                                        int tw, long Pp, int Cp, int colBlocks,
-                                                                       int rowBlocks) {
+                                                                       int rowBlocks, FilterJob fj, int in_blocks) {
     constexpr int CV = ChanVec<T>::n;
+    if (fj.w && (int)blockIdx.x >= in_blocks) {
+        filter_job_blocks<T, TC * NQ>(fj, in_blocks);
+        return;
+    }
     constexpr int HALF = TC + 1;                       // columns of one parity
     constexpr int ROWS = 2 * TR + 2, COLS = 2 * TC + 2;
     constexpr int NT = TC * NQ;

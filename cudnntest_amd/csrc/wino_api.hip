@@ -190,8 +190,6 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
                            const FilterJob& fj = FilterJob{}) {
     constexpr int CV = ChanVec<T>::n;
     const int CQ = g.Cp / CV;
-    if (fj.w && !input_is_nchw_tiled(layout, order, g))
-        return fail(WINO_ERR_INVALID, "this input transform cannot carry a filter job");
     if (input_is_nchw_tiled(layout, order, g)) {
         // TR x TC tiles per workgroup, TR*TC <= 256, halo of CV channels in LDS (<= 60 KB).
         // TR is kept a multiple of 8 when it can be, so a workgroup's run of V (TR*tw
@@ -224,16 +222,24 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
         (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
         constexpr int TC = 32, NQ = 8, TR = 2;
         const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
-        dim3 grid((unsigned)((long)g.N * rowBlocks * colBlocks), (CQ + NQ - 1) / NQ), block(TC * NQ);
+        const long in_blocks = (long)g.N * rowBlocks * colBlocks;
+        const int gy = (CQ + NQ - 1) / NQ;
+        // a filter job gets workgroups appended along x: enough, over all y, for one thread per (filter, channel vector)
+        const long extra = fj.w ? ((long)fj.Kp * CQ + (long)TC * NQ * gy - 1) / ((long)TC * NQ * gy) : 0;
+        if (in_blocks + extra >= (1L << 31)) return fail(WINO_ERR_UNSUPPORTED, "input transform: too many workgroups");
+        dim3 grid((unsigned)(in_blocks + extra), gy), block(TC * NQ);
         hipLaunchKernelGGL((input_transform_nhwc_kernel<T, TC, NQ, TR>), grid, block, 0, st, (const T*)x, (T*)V, g.N,
-                           g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, rowBlocks);
+                           g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, rowBlocks, fj, (int)in_blocks);
         LAUNCH_CHECK("input_transform_nhwc");
         return WINO_OK;
     }
-    dim3 grid((unsigned)((g.P + 255) / 256), CQ), block(256);
+    const long in_blocks = (g.P + 255) / 256;
+    const long extra = fj.w ? (fj.Kp + 255) / 256 : 0;          // x all CQ rows of the grid
+    if (in_blocks + extra >= (1L << 31)) return fail(WINO_ERR_UNSUPPORTED, "input transform: too many workgroups");
+    dim3 grid((unsigned)(in_blocks + extra), CQ), block(256);
     hipLaunchKernelGGL(input_transform_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
                        act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
-                       g.Cp, order);
+                       g.Cp, order, fj, (int)in_blocks);
     LAUNCH_CHECK("input_transform");
     return WINO_OK;
 }
@@ -640,10 +646,9 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
     float* Mo = (float*)(b + sc.m_off);
     const int order = tile_order_for(src, dst);
 
-    // The filter transform rides in the input transform's launch where that kernel can carry it (a launch of
-    // its own costs as much as its few microseconds of work); with stage timing on it stays a launch of its
-    // own, so that its span can be measured.
-    const bool ride = !Upre && algo != WINO_ALGO_FUSED && !g_timing && input_is_nchw_tiled(src, order, g);
+    // The filter transform rides in the input transform's launch (a launch of its own costs as much as its few
+    // microseconds of work); with stage timing on it stays a launch of its own, so that its span can be measured.
+    const bool ride = !Upre && algo != WINO_ALGO_FUSED && !g_timing;
     if (Upre) {
         U = const_cast<void*>(Upre);
     } else if (!ride) {
