@@ -141,9 +141,21 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     // x_prep fixes the stage to request (offsets, masks, sign); x_load_unit / x_load_all issue the
     // loads; v_unit turns the staged values of one channel into row i of B^T d B; v_write stores
     // the four coordinates into stage S of V.
-    T xa[4][UN], xb[4][UN];                    // [column][channel]; XM_ROW: [element of the quadruple][channel]
-    unsigned ma_c = 0, mb_c = 0, cok_c = 0;    // all ones when patch row ra / rb lies inside the image; bit u: channel u is real
-    float sg_c = 0.f;
+    // DEEP (2-byte operands): a stage's MFMAs are too short to cover the latency of the raw rows requested at its
+    // head, and a stage took as long as a trip to memory.  There the raw rows are requested TWO stages ahead, into
+    // two register sets that alternate with the stage parity, and the filter rows travel through registers (with a
+    // direct-to-LDS load pending the compiler would wait for every load in flight, the newest raw rows included).
+    constexpr bool DEEP = sizeof(T) == 2 && XM != XM_CHANVEC;   // (channel-vector loads: two k-groups per stage measured faster, and both do not fit the registers)
+    constexpr int NSET = DEEP ? 2 : 1;
+    typedef std::integral_constant<int, 0> set0_t;
+    typedef std::integral_constant<int, 1> set1_t;
+    // The raw values stay as loaded (packed quadruples / channel chunks) until v_unit takes them apart: split at
+    // the load, the unpacking of 2-byte elements would sit right behind the load and wait for it.
+    T xa[XM == XM_SCALAR ? NSET : 1][4][UN], xb[XM == XM_SCALAR ? NSET : 1][4][UN];   // XM_SCALAR: [set][column][channel]
+    Quad<T> qa_[XM == XM_ROW ? NSET : 1][UN], qb_[XM == XM_ROW ? NSET : 1][UN];        // XM_ROW: [set][channel], 4 columns each
+    chunk_t ca_[XM == XM_CHANVEC ? NSET : 1][4], cb_[XM == XM_CHANVEC ? NSET : 1][4];  // XM_CHANVEC: [set][column], UN channels each
+    unsigned ma_c[NSET], mb_c[NSET], cok_c[NSET];   // all ones when patch row ra / rb lies inside the image; bit u: channel u is real
+    float sg_c[NSET];
     unsigned ma_n = 0, mb_n = 0, cok_n, ra_off = 0, rb_off = 0;
     float sg_n = 0.f;
     int c_n;
@@ -167,41 +179,57 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
 #pragma unroll
         for (int u = 0; u < UN; ++u) cok_n |= (c_n + u < C) ? 1u << u : 0u;
     };
-    auto x_load_unit = [&](int u) {            // XM_SCALAR, XM_ROW
+    auto x_load_unit = [&](auto set, int u) {  // XM_SCALAR, XM_ROW
+        constexpr int Q = decltype(set)::value;
         const unsigned coff = ((cok_n >> u) & 1u) ? (unsigned)((c_n + u) * xs.c) : 0u;
         if (XM == XM_ROW) {
             // channel plane: a wave-uniform (scalar) base; the lane adds its 32-bit byte offset
             const char* plane = reinterpret_cast<const char*>(x) + (size_t)coff * sizeof(T);
-            const Quad<T> qa = *reinterpret_cast<const Quad<T>*>(plane + ra_off);
-            const Quad<T> qb = *reinterpret_cast<const Quad<T>*>(plane + rb_off);
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) { xa[jj][u] = qa.v[jj]; xb[jj][u] = qb.v[jj]; }
+            qa_[XM == XM_ROW ? Q : 0][u] = *reinterpret_cast<const Quad<T>*>(plane + ra_off);
+            qb_[XM == XM_ROW ? Q : 0][u] = *reinterpret_cast<const Quad<T>*>(plane + rb_off);
         } else {
 #pragma unroll
             for (int jj = 0; jj < 4; ++jj) {
-                xa[jj][u] = x[ra_off + coff + u_col[jj]];
-                xb[jj][u] = x[rb_off + coff + u_col[jj]];
+                xa[XM == XM_SCALAR ? Q : 0][jj][u] = x[ra_off + coff + u_col[jj]];
+                xb[XM == XM_SCALAR ? Q : 0][jj][u] = x[rb_off + coff + u_col[jj]];
             }
         }
     };
-    auto x_load_all = [&]() {                  // XM_CHANVEC: C % UN == 0, all UN channels real or none
+    auto x_load_all = [&](auto set) {          // XM_CHANVEC: C % UN == 0, all UN channels real or none
+        constexpr int Q = decltype(set)::value;
         const unsigned coff = cok_n ? (unsigned)c_n : 0u;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-            const chunk_t va = *reinterpret_cast<const chunk_t*>(x + (ra_off + coff + u_col[jj]));
-            const chunk_t vb = *reinterpret_cast<const chunk_t*>(x + (rb_off + coff + u_col[jj]));
-            __builtin_memcpy(xa[jj], &va, sizeof(chunk_t));
-            __builtin_memcpy(xb[jj], &vb, sizeof(chunk_t));
+            ca_[XM == XM_CHANVEC ? Q : 0][jj] = *reinterpret_cast<const chunk_t*>(x + (ra_off + coff + u_col[jj]));
+            cb_[XM == XM_CHANVEC ? Q : 0][jj] = *reinterpret_cast<const chunk_t*>(x + (rb_off + coff + u_col[jj]));
         }
     };
-    auto take_next = [&]() { ma_c = ma_n; mb_c = mb_n; cok_c = cok_n; sg_c = sg_n; };
+    auto take_next = [&](auto set) {
+        constexpr int Q = decltype(set)::value;
+        ma_c[Q] = ma_n; mb_c[Q] = mb_n; cok_c[Q] = cok_n; sg_c[Q] = sg_n;
+    };
     T out[4][UN];
-    auto v_unit = [&](int u) {
-        const bool ok = (cok_c >> u) & 1u;
-        const unsigned mau = ok ? ma_c : 0u, mbu = ok ? mb_c : 0u;
+    auto v_unit = [&](auto set, int u) {
+        constexpr int Q = decltype(set)::value;
+        const bool ok = (cok_c[Q] >> u) & 1u;
+        const unsigned mau = ok ? ma_c[Q] : 0u, mbu = ok ? mb_c[Q] : 0u;
         float da[4], db[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) { da[q] = to_f32(xa[q][u]); db[q] = to_f32(xb[q][u]); }
+        for (int q = 0; q < 4; ++q) {
+            if constexpr (XM == XM_ROW) {
+                da[q] = to_f32(qa_[Q][u].v[q]);
+                db[q] = to_f32(qb_[Q][u].v[q]);
+            } else if constexpr (XM == XM_CHANVEC) {
+                T ea[UN], eb[UN];
+                __builtin_memcpy(ea, &ca_[Q][q], sizeof(chunk_t));
+                __builtin_memcpy(eb, &cb_[Q][q], sizeof(chunk_t));
+                da[q] = to_f32(ea[u]);
+                db[q] = to_f32(eb[u]);
+            } else {
+                da[q] = to_f32(xa[Q][q][u]);
+                db[q] = to_f32(xb[Q][q][u]);
+            }
+        }
         if (XM == XM_ROW) {
             // patch column j = element j + dcol of the quadruple; elements that fall outside it are
             // columns outside the image, zeroed by cw below
@@ -220,7 +248,7 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
         float r[4];
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj)
-            r[jj] = mask_keep(fmaf(sg_c, mask_keep(db[jj], mbu), mask_keep(da[jj], mau)), cw[jj]);
+            r[jj] = mask_keep(fmaf(sg_c[Q], mask_keep(db[jj], mbu), mask_keep(da[jj], mau)), cw[jj]);
         out[0][u] = from_f32<T>(r[0] - r[2]);
         out[1][u] = from_f32<T>(r[1] + r[2]);
         out[2][u] = from_f32<T>(r[2] - r[1]);
@@ -244,21 +272,21 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
     constexpr int UPP = (UN + NR - 2) / (NR - 1);
     constexpr int WP = (UN + UPP - 1) / UPP;
     static_assert(WP < NR, "pieces must fit the runs");
-    auto v_piece = [&](auto par, int piece) {
+    auto v_piece = [&](auto par, auto set, int piece) {     // set: the raw rows to transform; par: the stage of V they become
         if (piece < WP) {
 #pragma unroll
-            for (int u = piece * UPP; u < (piece + 1) * UPP && u < UN; ++u) v_unit(u);
+            for (int u = piece * UPP; u < (piece + 1) * UPP && u < UN; ++u) v_unit(set, u);
         } else if (piece == WP) {
             v_write(par);
         }
     };
-    auto x_load_stage = [&](int row_i, int st) {
+    auto x_load_stage = [&](auto set, int row_i, int st) {
         x_prep(row_i, st);
-        take_next();
-        if (XM == XM_CHANVEC) x_load_all();
+        take_next(set);
+        if (XM == XM_CHANVEC) x_load_all(set);
         else {
 #pragma unroll
-            for (int u = 0; u < UN; ++u) x_load_unit(u);
+            for (int u = 0; u < UN; ++u) x_load_unit(set, u);
         }
     };
     // ---- the filter rows of a stage: 4*NV rows of 64 vectors, wave w issues rows w, w+4, ... --
@@ -285,10 +313,36 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
             uptr[q] += inc;
         }
     };
-    int ni = 0, nstg = 0;                      // (row, stage) after the one being multiplied
+    // DEEP: the filter rows as register loads (requested at the head of a stage, written to LDS at its tail)
+    vec ureg[DEEP ? NV : 1];
+    auto u_req = [&](int row_i, int st) {
+        typedef __attribute__((address_space(1))) const vec* gvec_p;
+        const bool last = row_i == 3 && st == nst - 1;
+        const uint64_t inc = last ? 0 : (st == nst - 1 ? wrapU : stepU);
+#pragma unroll
+        for (int q = 0; q < NV; ++q) {
+            ureg[DEEP ? q : 0] = *reinterpret_cast<gvec_p>(uptr[q] + lane_off);
+            uptr[q] += inc;
+        }
+    };
+    auto u_commit = [&](auto par) {
+        constexpr int S = decltype(par)::value;
+#pragma unroll
+        for (int q = 0; q < NV; ++q) {
+            const int r = wave + 4 * q;
+            const int j = r / NV, v = r % NV;
+            (S ? Us1 : Us0)[j][v][lane] = ureg[DEEP ? q : 0];
+        }
+    };
+    int ni = 0, nstg = 0;                      // (row, stage) of the filter rows to request: the one after the stage being multiplied
+    int xi_ = 0, xst_ = 0;                     // (row, stage) of the raw rows to request: the same, or one further (DEEP)
     auto advance = [&]() {
         if (++nstg == nst) { nstg = 0; ++ni; }
         if (ni > 3) { ni = 3; nstg = nst - 1; }      // past the end: repeat the last stage (never read)
+    };
+    auto advance_x = [&]() {
+        if (++xst_ == nst) { xst_ = 0; ++xi_; }
+        if (xi_ > 3) { xi_ = 3; xst_ = nst - 1; }
     };
     vec fu[2], fv[2];
     // first: the stage opens a Winograd row, its MFMAs start from a zero accumulator
@@ -302,16 +356,21 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
             fv[r & 1] = S ? Vs1[j][v][(SWAP ? wm : wn) * 32 + l32] : Vs0[j][v][(SWAP ? wm : wn) * 32 + l32];
         };
         // the next stage: filter rows and raw patch rows requested first, multiplied stage in between,
-        // the raw rows transformed and written during the last MFMA runs
-        u_load(other_t{}, ni, nstg);
-        x_load_stage(ni, nstg);
+        // the raw rows transformed and written during the last MFMA runs.  DEEP: the raw rows requested here
+        // are those of the stage after the next (set S); the ones transformed below arrived a stage ago (set 1-S)
+        typedef std::integral_constant<int, DEEP ? S : 0> lset_t;
+        typedef std::integral_constant<int, DEEP ? 1 - S : 0> vset_t;
+        if constexpr (DEEP) u_req(ni, nstg);
+        else u_load(other_t{}, ni, nstg);
+        x_load_stage(lset_t{}, xi_, xst_);
         advance();
+        advance_x();
         frag_load(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             if (r + 1 < NR) frag_load(r + 1);
-            if (r >= NR - 1 - WP) v_piece(other_t{}, r - (NR - 1 - WP));
+            if (r >= NR - 1 - WP) v_piece(other_t{}, vset_t{}, r - (NR - 1 - WP));
             if (FIRST && r < 4) {
 #pragma unroll
                 for (int q = 0; q < 16; ++q) acc[r][q] = 0.f;
@@ -320,20 +379,33 @@ __global__ __launch_bounds__(256, 2) void fused_rows_kernel(const T* __restrict_
             else Mma<T>::run(fu[r & 1], fv[r & 1], acc[r & 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0) lgkmcnt(0)
+        if constexpr (DEEP) {
+            u_commit(other_t{});                     // (the compiler waits for exactly these loads)
+            __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only: the newest raw rows stay in flight
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0070);      // vmcnt(0) lgkmcnt(0)
+        }
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");               // no LDS access moves across the barrier
     };
 
-    // prologue: stage (0, 0) of both operands in LDS
-    x_load_stage(0, 0);
-    u_load(par0_t{}, 0, 0);
+    // prologue: stage (0, 0) of both operands in LDS (DEEP: and the raw rows of the stage after it requested)
+    x_load_stage(set0_t{}, 0, 0);
+    advance_x();
+    if constexpr (DEEP) {
+        u_req(0, 0);
+        x_load_stage(set1_t{}, xi_, xst_);
+        advance_x();
+    } else {
+        u_load(par0_t{}, 0, 0);
+    }
     advance();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int piece = 0; piece <= WP; ++piece) v_piece(par0_t{}, piece);
+    for (int piece = 0; piece <= WP; ++piece) v_piece(par0_t{}, set0_t{}, piece);
+    if constexpr (DEEP) u_commit(par0_t{});
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_waitcnt(DEEP ? 0xC07F : 0x0070);
     __syncthreads();
 
     for (int i = 0; i < 4; ++i) {
