@@ -21,6 +21,7 @@ Prints ONE JSON line:
                algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4)
   cpu_baseline the oracle's fp32 OpenMP direct convolution on this host's cores (reported, not a target)
   stages       per-stage ms and achieved GB/s (algorithmic bytes) or TFLOP/s
+  ms_per_step_filters_prepared   the same K steps with the filter bank transformed beforehand (single-layer runs)
   layout_transforms   the stand-alone permutations of the layer's input between its layout and the other two
                (wino_layout_transform; bytes = read + write), timed apart from the convolution
 """
@@ -235,6 +236,20 @@ def main():
         "roofline": roofline,
         "stages": stages,
     }
+
+    # ---- the same K steps with the filter bank transformed beforehand (filter transform excluded) ----
+    if not multi and stack is None and resolved[0] in ("staged", "epilogue", "fused"):
+        x0, w0, y0 = tensors[0]
+        U0 = ops.filter_transform(w0, layout)
+        a0 = {"staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE, "fused": ops.ALGO_FUSED}[resolved[0]]
+        for _ in range(args.warmup):
+            ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0)
+        torch.cuda.synchronize()
+        tp = time.perf_counter()
+        for _ in range(args.steps):
+            ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0)
+        torch.cuda.synchronize()
+        out["ms_per_step_filters_prepared"] = round((time.perf_counter() - tp) * 1e3 / args.steps, 4)
 
     # ---- the stand-alone layout permutations of the layer's input, timed separately ------------
     if not multi and stack is None:
