@@ -18,7 +18,8 @@ Prints ONE JSON line:
   ms_per_step  ms per layer (per 13-layer pass for vgg16_all13)
   roofline     the dominant kernel -- the batched GEMM, or the kernel that contains it -- timed with
                HIP events recorded by the library on the launch stream, against the dense MFMA peak;
-               algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4)
+               algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4); single-layer runs add
+               the kernel's algorithmic bytes, flop/byte, min(MFMA peak, flop/byte x 8 TB/s) and its fraction of 8 TB/s
   cpu_baseline the oracle's fp32 OpenMP direct convolution on this host's cores (reported, not a target)
   stages       per-stage ms and achieved GB/s (algorithmic bytes) or TFLOP/s
   ms_per_step_filters_prepared   the same K steps with the filter bank transformed beforehand (single-layer runs)
@@ -223,6 +224,25 @@ def main():
                 "flops_per_launch": gemm_flops if not multi else None}
 
     N0, C0, K0, H0 = layers[0]
+    if not multi:
+        # the dominant kernel's algorithmic bytes, its arithmetic intensity, and what the two roofs allow together
+        Pn = ops.geometry(dt, N0, C0, K0, H0, H0, 1)["P"]
+        xb, yb = N0 * C0 * H0 * H0 * es, N0 * K0 * H0 * H0 * es
+        kb = {"staged": 16 * Pn * C0 * es + 16 * K0 * C0 * es + 16 * Pn * K0 * 4,
+              "epilogue": 16 * Pn * C0 * es + 16 * K0 * C0 * es + yb,
+              "fused": xb + 16 * K0 * C0 * es + yb,
+              "direct": xb + 9 * K0 * C0 * es + yb}.get(algo_label)
+        if kb:
+            ai = gemm_flops / kb
+            gbs = kb / (gemm_ms * 1e-3) / 1e9
+            roofline.update(algorithmic_bytes=kb, flop_per_byte=round(ai, 1),
+                            attainable=round(min(peak, ai * HBM_PEAK_GBS / 1e3), 1),
+                            frac_hbm=round(gbs / HBM_PEAK_GBS, 3))
+            if ai * HBM_PEAK_GBS / 1e3 < peak:
+                # the memory roof is the lower one for this kernel and type: it is the bound that is reported
+                roofline.update(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                                frac=round(gbs / HBM_PEAK_GBS, 4), mfma_achieved=round(achieved, 2),
+                                mfma_frac=round(achieved / peak, 4))
     out = {
         "metric": "effective TFLOP/s (direct-conv FLOPs), VGG-16 3x3 layer, N=32",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
