@@ -1,0 +1,49 @@
+"""Index arithmetic past 2^31: a layer whose transformed operands hold more than 2^31 elements (N=768, C=K=256,
+H=W=56 in fp32: x and y 617 M elements = 2.5 GB each, the transformed input V 2.47 G elements = 9.9 GB, the product
+tensor of the staged pipeline as much again, byte offsets past 2^33).  The oracle convolves the LAST image (the far
+end of every index space) with three filters; the two pipelines must agree with each other over the whole tensor."""
+import pytest
+import torch
+
+from cudnntest_amd import ops
+from gpu_util import TOL, host
+
+pytestmark = pytest.mark.gpu
+N, C, K, H = 768, 256, 256, 56
+
+
+def _rel(a, b):
+    # norms in chunks: a float64 copy of a 2.5 GB tensor is not needed
+    num = sum(((a[i:i + 64].double() - b[i:i + 64].double()) ** 2).sum().item() for i in range(0, a.shape[0], 64))
+    den = sum((b[i:i + 64].double() ** 2).sum().item() for i in range(0, b.shape[0], 64))
+    return (num / den) ** 0.5
+
+
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC])
+def test_more_than_2_31_elements_per_operand(oracle, layout):
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * 2 ** 30:
+        pytest.skip("needs 40 GB of free device memory")
+    g = torch.Generator(device="cuda").manual_seed(31)
+    x = torch.rand((N, C, H, H), device="cuda", generator=g) * 2 - 1
+    w = torch.randn((K, C, 3, 3), device="cuda", generator=g) * (2.0 / (9 * C)) ** 0.5
+    assert 16 * (N * 28 * 28) * C > 2 ** 31
+    ks = [0, K // 2, K - 1]
+    want = oracle.direct_conv_f32(host(x[N - 1:]), host(w[ks]), 1)
+    if layout == ops.NHWC:
+        xl, wl = x.permute(0, 2, 3, 1).contiguous(), w.permute(0, 2, 3, 1).contiguous()
+        del x
+    else:
+        xl, wl = x, w
+    ys = {}
+    for algo in (ops.ALGO_EPILOGUE, ops.ALGO_STAGED):
+        y = ops.conv(xl, wl, 1, layout, algo=algo)
+        y_nchw = y.permute(0, 3, 1, 2) if layout == ops.NHWC else y
+        assert tuple(y_nchw.shape) == (N, K, H, H)
+        err = oracle.rel_l2(host(y_nchw[N - 1:][:, ks]), want)
+        assert err <= TOL[ops.F32], (algo, err)
+        ys[algo] = y
+    assert _rel(ys[ops.ALGO_STAGED], ys[ops.ALGO_EPILOGUE]) <= 1e-5
+    # leave the scratch arena at its usual size for the tests that follow
+    del ys, y, xl
+    torch.cuda.empty_cache()
