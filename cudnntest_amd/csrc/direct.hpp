@@ -170,4 +170,170 @@ __global__ __launch_bounds__(256) void direct_small_c_kernel(const T* __restrict
     }
 }
 
+// The same for 2-byte tensors on the 16-bit matrix instruction: the 9*C <= 36 taps of an output are NE =
+// ceil(9*C/16) v_mfma_f32_32x32x16 (2 for C = 3) instead of 14 fp32 ones -- a fourteenth of the matrix time.
+// The products are the same (two 2-byte values multiply exactly in fp32 either way), only the order in which
+// an instruction sums its 16 of them is the hardware's.  A lane holds 8 consecutive taps per instruction:
+// kk = 16e + 8*lh + i.
+__host__ inline size_t direct16_lds_bytes(int C, int K) {
+    if (C < 1 || C > 4) return 0;
+    const size_t ne = (9 * C + 15) / 16, kt = (K + 31) / 32;
+    return kt * ne * 64 * 16 + kt * 32 * sizeof(float);
+}
+
+template <typename T, int NE, bool SWAP>
+__global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                               T* __restrict__ y, ActStrides xs, FltStrides ws,
+                                                               ActStrides ys, int N, int C, int K, int H, int W,
+                                                               int pad, int Ho, int Wo, int batch_minor, long Q,
+                                                               int groups, Epilogue ep) {
+    static_assert(sizeof(T) == 2, "2-byte tensors");
+    typedef typename Mma<T>::vec vec;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem16[];
+    const int KT = (K + 31) / 32;
+    vec* sW = reinterpret_cast<vec*>(smem16);                              // [KT][NE][64]
+    float* sB = reinterpret_cast<float*>(smem16 + (size_t)KT * NE * 64 * 16);   // [KT*32] bias
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int nk = 9 * C;
+
+    for (int i = tid; i < KT * NE * 64; i += 256) {
+        const int ln = i & 63, e = (i >> 6) % NE, kt = (i >> 6) / NE;
+        const int k = kt * 32 + (ln & 31);
+        T v8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int kk = 16 * e + 8 * (ln >> 5) + j;
+            const bool ok = k < K && kk < nk;
+            const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
+            const T v = w[ok ? k * ws.k + c * ws.c + r * ws.r + q * ws.s : 0];
+            v8[j] = ok ? v : from_f32<T>(0.f);
+        }
+        vec pk;
+        __builtin_memcpy(&pk, v8, 16);
+        sW[i] = pk;
+    }
+    for (int i = tid; i < KT * 32; i += 256) sB[i] = i < K ? bias_of<T>(ep, i) : 0.f;
+
+    int off[NE][8];
+    unsigned rs[NE];                          // per tap j: bits 4j..4j+3 = r | s << 2; taps past 9*C: r = s = 3 (never inside)
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        rs[e] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int kk = 16 * e + 8 * lh + j;
+            const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
+            const bool real = kk < nk;
+            off[e][j] = real ? (int)(c * xs.c + r * xs.h + q * xs.w) : 0;
+            rs[e] |= (real ? ((unsigned)r | (unsigned)q << 2) : 15u) << (4 * j);
+        }
+    }
+    __syncthreads();
+
+#pragma unroll 1
+    for (int gi = 0; gi < groups; ++gi) {
+        const long q0 = ((long)blockIdx.x * 4 + wave) * (groups * 32) + gi * 32;
+        if (q0 >= Q) break;                   // wave-uniform
+        const long q = q0 + l32;
+        const bool qok = q < Q;
+        const unsigned qu = (unsigned)(qok ? q : Q - 1);
+        int n, oh, ow;
+        if (batch_minor) {
+            const unsigned t = qu / (unsigned)N;
+            n = (int)(qu - t * (unsigned)N);
+            oh = (int)(t / (unsigned)Wo);
+            ow = (int)(t - (unsigned)oh * (unsigned)Wo);
+        } else {
+            const unsigned t = qu / (unsigned)Wo;
+            ow = (int)(qu - t * (unsigned)Wo);
+            n = (int)(t / (unsigned)Ho);
+            oh = (int)(t - (unsigned)n * (unsigned)Ho);
+        }
+        unsigned rmask = 0, cmask = 0;        // bit t: tap row / column t of this pixel lies inside the image (bit 3 never)
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            rmask |= (oh + t - pad >= 0 && oh + t - pad < H) ? 1u << t : 0u;
+            cmask |= (ow + t - pad >= 0 && ow + t - pad < W) ? 1u << t : 0u;
+        }
+        const int base = (int)(n * xs.n + (long)(oh - pad) * xs.h + (long)(ow - pad) * xs.w);
+        const int safe = (int)(n * xs.n + (long)oh * xs.h + (long)ow * xs.w);
+        vec b[NE];
+        if (__ballot(rmask != 7u || cmask != 7u) == 0) {
+            // every tap of every pixel of the group inside its image (taps past 9*C read channel 0 and meet a zero weight)
+            T raw[NE][8];
+#pragma unroll
+            for (int e = 0; e < NE; ++e)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) raw[e][j] = x[(unsigned)(base + off[e][j])];
+#pragma unroll
+            for (int e = 0; e < NE; ++e) __builtin_memcpy(&b[e], raw[e], 16);
+        } else {
+            T raw[NE][8];
+#pragma unroll
+            for (int e = 0; e < NE; ++e)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const unsigned t = rs[e] >> (4 * j);
+                    const bool in = ((rmask >> (t & 3u)) & (cmask >> ((t >> 2) & 3u)) & 1u) != 0;
+                    const T v = x[(unsigned)(in ? base + off[e][j] : safe)];
+                    raw[e][j] = in ? v : from_f32<T>(0.f);
+                }
+#pragma unroll
+            for (int e = 0; e < NE; ++e) __builtin_memcpy(&b[e], raw[e], 16);
+        }
+
+        const unsigned yq = (unsigned)(n * ys.n + oh * ys.h + ow * ys.w + 4 * lh * ys.c);
+#pragma unroll 1
+        for (int kt = 0; kt < KT; ++kt) {
+            floatx16 acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            const vec* wk = sW + (size_t)kt * NE * 64 + lane;
+            vec a[NE];
+#pragma unroll
+            for (int e = 0; e < NE; ++e) a[e] = wk[e * 64];
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                if (SWAP) Mma<T>::run(b[e], a[e], acc);
+                else Mma<T>::run(a[e], b[e], acc);
+            }
+            if (SWAP) {
+                const int k = kt * 32 + l32;
+                const float bk = sB[k];
+                if (k < K) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const long pq = q0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                        float v = acc[r] + bk;
+                        if (ep.relu) v = fmaxf(v, 0.f);
+                        if (pq < Q) y[pq * K + k] = from_f32<T>(v);
+                    }
+                }
+                continue;
+            }
+            float bv[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bv[r] = sB[kt * 32 + 8 * (r >> 2) + (r & 3) + 4 * lh];
+            const T* yk = y + (size_t)kt * 32 * ys.c;
+            auto put = [&](int r) {
+                float v = acc[r] + bv[r];
+                if (ep.relu) v = fmaxf(v, 0.f);
+                const_cast<T*>(yk + (size_t)(8 * (r >> 2) + (r & 3)) * ys.c)[yq] = from_f32<T>(v);
+            };
+            if (!qok) continue;
+            if (kt * 32 + 32 <= K) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) put(r);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (kt * 32 + 8 * (r >> 2) + (r & 3) + 4 * lh < K) put(r);
+            }
+        }
+    }
+}
+
 }  // namespace wino

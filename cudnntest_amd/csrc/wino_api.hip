@@ -521,11 +521,29 @@ int launch_direct_t(int src, int dst, unsigned flags, const void* bias, const Ge
     else                                                                                                            \
         hipLaunchKernelGGL((direct_small_c_kernel<T, NE, false>), grid, block, lds, st, (const T*)x, (const T*)w, (T*)y, \
                            xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, minor, Q, groups, ep)
-    switch (g.C) {
-    case 1: DIRECT_LAUNCH(5); break;
-    case 2: DIRECT_LAUNCH(9); break;
-    case 3: DIRECT_LAUNCH(14); break;
-    default: DIRECT_LAUNCH(18); break;
+    if constexpr (sizeof(T) == 2) {
+        // 2-byte tensors: the 16-bit matrix instruction, 16 taps each
+        const size_t lds16 = direct16_lds_bytes(g.C, g.K);
+#define DIRECT16_LAUNCH(NE)                                                                                          \
+    if (dst == WINO_NHWC)                                                                                           \
+        hipLaunchKernelGGL((direct_small_c16_kernel<T, NE, true>), grid, block, lds16, st, (const T*)x, (const T*)w, \
+                           (T*)y, xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, minor, Q, groups, ep);     \
+    else                                                                                                            \
+        hipLaunchKernelGGL((direct_small_c16_kernel<T, NE, false>), grid, block, lds16, st, (const T*)x, (const T*)w, \
+                           (T*)y, xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, minor, Q, groups, ep)
+        switch (g.C) {
+        case 1: DIRECT16_LAUNCH(1); break;
+        case 4: DIRECT16_LAUNCH(3); break;
+        default: DIRECT16_LAUNCH(2); break;
+        }
+#undef DIRECT16_LAUNCH
+    } else {
+        switch (g.C) {
+        case 1: DIRECT_LAUNCH(5); break;
+        case 2: DIRECT_LAUNCH(9); break;
+        case 3: DIRECT_LAUNCH(14); break;
+        default: DIRECT_LAUNCH(18); break;
+        }
     }
 #undef DIRECT_LAUNCH
     LAUNCH_CHECK("direct_small_c");
