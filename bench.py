@@ -215,7 +215,8 @@ def main():
     if not multi:
         stages["gemm"].update(min_ms=round(st["gemm"][1], 4), max_ms=round(st["gemm"][2], 4))
     kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
-              "staged_f4": "gemm_128x128_kernel", "direct": "direct_small_c_kernel"}
+              "staged_f4": "gemm_128x128_kernel",
+              "direct": "direct_small_c_kernel" if args.dtype == "f32" else "direct_small_c16_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"
     traffic = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label))
     roofline = {"bound": "mfma", "kernel": kernel.get(algo_label, "per-layer choice"),
