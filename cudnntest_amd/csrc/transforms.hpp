@@ -337,24 +337,44 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     const int tr = tid / TC, tc = tid % TC;
     const int ty = ty0 + tr, tx = tx0 + tc;
     if (tr >= TR || ty >= th || tx >= tw) return;
-    float v[CV][16];
-#pragma unroll
-    for (int ch = 0; ch < CV; ++ch) {
+    const long p = ((long)n * th + ty) * tw + tx;
+    const size_t plane = (size_t)Cp * Pp;
+    T* vp = V + ((size_t)cq * Pp + p) * CV;
+    auto tile_of = [&](int ch, float (&out)[16]) {
         float d[4][4];
         const T* base = in_smem + ch * per_ch + (2 * tr) * ldsW + 2 * tc;
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds_row4<T>(base + i * ldsW, d[i]);
-        input_tile_transform(d, v[ch]);
-    }
-    const long p = ((long)n * th + ty) * tw + tx;
-    const size_t plane = (size_t)Cp * Pp;
-    T* vp = V + ((size_t)cq * Pp + p) * CV;
+        input_tile_transform(d, out);
+    };
+    if constexpr (sizeof(T) == 2) {
+        // 8 channels x 16 coordinates: rounded and packed two channels to a register as they are produced (64
+        // registers instead of 128 fp32 values held until the stores)
+        uint32_t wd[16][CV / 2];
 #pragma unroll
-    for (int xi = 0; xi < 16; ++xi) {
-        float o[CV];
+        for (int ch = 0; ch < CV; ++ch) {
+            float vc[16];
+            tile_of(ch, vc);
 #pragma unroll
-        for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
-        store_chan_vec<T>(vp + xi * plane, o);
+            for (int xi = 0; xi < 16; ++xi) {
+                const uint32_t bits = __builtin_bit_cast(uint16_t, from_f32<T>(vc[xi]));
+                wd[xi][ch / 2] = (ch & 1) ? (wd[xi][ch / 2] | bits << 16) : bits;
+            }
+        }
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi)
+            *reinterpret_cast<uint4*>(vp + xi * plane) = make_uint4(wd[xi][0], wd[xi][1], wd[xi][2], wd[xi][3]);
+    } else {
+        float v[CV][16];
+#pragma unroll
+        for (int ch = 0; ch < CV; ++ch) tile_of(ch, v[ch]);
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi) {
+            float o[CV];
+#pragma unroll
+            for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
+            store_chan_vec<T>(vp + xi * plane, o);
+        }
     }
 }
 
