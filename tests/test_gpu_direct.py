@@ -66,3 +66,20 @@ def test_what_the_path_is_not_built_for():
         ops.conv_prepared(x, U, 4, algo=ops.ALGO_DIRECT)
     assert e.value.code == -1
     ops.conv_prepared(x, U, 4)
+
+
+@pytest.mark.parametrize("dtype", [ops.F32, ops.BF16])
+def test_direct_with_the_largest_filter_bank_that_fits_lds(oracle, dtype):
+    """K = 544 at C = 3: 17 filter tiles, 63 KB of LDS in fp32 (the path is offered up to 64 KB); K = 576 no
+    longer fits and AUTO goes back to the Winograd kernels.  Integers: bit-exact either way."""
+    from gpu_util import dev, host
+    N, C, H, W = 1, 3, 9, 10
+    for K, want_algo in ((544, ops.ALGO_DIRECT), (576, None)):
+        x, w = synth.conv_inputs(N, C, K, H, W, seed=K, integer=True)
+        got_algo = ops.pick_algo(ops.NCHW, dtype, N, C, K, H, W)
+        if want_algo is None:
+            assert got_algo != ops.ALGO_DIRECT
+        else:
+            assert got_algo == want_algo
+        y = host(ops.conv(dev(x, dtype), dev(w, dtype), 1, ops.NCHW))
+        assert np.array_equal(y, oracle.direct_conv(x, w, 1))
