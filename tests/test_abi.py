@@ -117,3 +117,17 @@ def test_product_never_imports_the_oracle():
     for f in glob.glob(os.path.join(ROOT, "cudnntest_amd", "*.py")):
         text = open(f).read()
         assert "import oracle" not in text and "from oracle" not in text, f
+
+
+def test_bench_refuses_more_than_one_gpu_and_runs_nothing_without_one():
+    """bench.py measures one GPU: --gpus N > 1 exits with a message before touching a device; without a GPU the
+    default run exits with a message as well (no CPU path stands in for the kernels)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr
+    import torch
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True, text=True)
+        assert r.returncode != 0 and "no GPU" in r.stderr
