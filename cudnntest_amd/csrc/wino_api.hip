@@ -561,9 +561,16 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     // the single-kernel path addresses the input with 32-bit byte offsets
     const bool fused_ok = (long)g.N * g.C * g.H * g.W * (long)dtype_size(dtype) < (1L << 32);
     if (dtype == WINO_F32) {
+        // (a short reduction into one filter tile runs best as the single kernel from 64 patches on:
+        // N = 8, C = K = 64, H = 56, 98 patches: 0.038 against 0.044 ms)
+        if (patches >= 64 && g.C <= 64 && g.K <= 64 && fused_ok) return WINO_ALGO_FUSED;
         if (patches < 128) return WINO_ALGO_STAGED;      // a 64x64 patch for every other CU at most
-        // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel
-        if (g.C <= 128 && g.K <= 128 && fused_ok) return WINO_ALGO_FUSED;
+        // few channels: V would be 4x the input and is consumed by few filter tiles -- build it in the kernel.
+        // With one filter tile (K <= 64) no tile is transformed twice, whatever C (C = 256, K = 64, H = 56:
+        // 0.185 against 0.233 ms); with two, the single kernel needs many patches to win (C = K = 128: 196
+        // patches 0.067 against 0.062 ms for EPILOGUE, 392 a tie, 12544 0.57 against 0.63)
+        if (fused_ok && g.K <= 64 && g.C <= 256) return WINO_ALGO_FUSED;
+        if (g.C <= 128 && g.K <= 128) return (fused_ok && patches >= 512) ? WINO_ALGO_FUSED : WINO_ALGO_EPILOGUE;
         if (patches < 256) return WINO_ALGO_STAGED;      // not even one 64x64 patch per CU
         if (g.C <= 256) return WINO_ALGO_EPILOGUE;
         // many channels: the 128x128 GEMM's lower L2 traffic per flop wins, unless there are few tiles or the
@@ -579,8 +586,10 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     if (patches < 64 || (g.C >= 256 && patches < 128) || (g.C >= 512 && patches < 256)) return WINO_ALGO_STAGED;
     if (!fused_ok) return WINO_ALGO_EPILOGUE;
     if (nhwc) {
-        if (g.C >= 16 && g.C <= 128 && g.K <= 128) return WINO_ALGO_FUSED;
-    } else if (g.C <= 64 && g.K <= 64 && patches >= 2048) {   // (fewer patches: measured 5-19 % behind EPILOGUE)
+        // (one filter tile: any C up to 256; two: only with many patches -- C = K = 128 at 196 patches is 6 % behind EPILOGUE)
+        if (g.C >= 16 && g.K <= 64 && g.C <= 256) return WINO_ALGO_FUSED;
+        if (g.C >= 16 && g.C <= 128 && g.K <= 128 && patches >= 1024) return WINO_ALGO_FUSED;
+    } else if (g.C <= 64 && g.K <= 64 && patches >= 1536) {   // (fewer patches: measured behind EPILOGUE)
         return WINO_ALGO_FUSED;
     }
     return WINO_ALGO_EPILOGUE;
