@@ -246,6 +246,49 @@ template <> __device__ __forceinline__ void lds_row4<bf16_t>(const bf16_t* p, fl
     d[2] = __uint_as_float(v << 16); d[3] = __uint_as_float(v & 0xffff0000u);
 }
 
+// The 16 coordinates of one tile for the CV channels of a vector, built from LDS planes [ch][rows][ldsW] that hold
+// the zero padding (`base`: the tile's first element in the first plane, at an even column), and stored as 16
+// vectors of V, `plane` elements apart.
+template <typename T>
+__device__ __forceinline__ void tile_from_lds_store(const T* base, int per_ch, int ldsW, T* vp, size_t plane) {
+    constexpr int CV = ChanVec<T>::n;
+    auto tile_of = [&](int ch, float (&out)[16]) {
+        float d[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds_row4<T>(base + ch * per_ch + i * ldsW, d[i]);
+        input_tile_transform(d, out);
+    };
+    if constexpr (sizeof(T) == 2) {
+        // 8 channels x 16 coordinates: rounded and packed two channels to a register as they are produced (64
+        // registers instead of 128 fp32 values held until the stores)
+        uint32_t wd[16][CV / 2];
+#pragma unroll
+        for (int ch = 0; ch < CV; ++ch) {
+            float vc[16];
+            tile_of(ch, vc);
+#pragma unroll
+            for (int xi = 0; xi < 16; ++xi) {
+                const uint32_t bits = __builtin_bit_cast(uint16_t, from_f32<T>(vc[xi]));
+                wd[xi][ch / 2] = (ch & 1) ? (wd[xi][ch / 2] | bits << 16) : bits;
+            }
+        }
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi)
+            *reinterpret_cast<uint4*>(vp + xi * plane) = make_uint4(wd[xi][0], wd[xi][1], wd[xi][2], wd[xi][3]);
+    } else {
+        float v[CV][16];
+#pragma unroll
+        for (int ch = 0; ch < CV; ++ch) tile_of(ch, v[ch]);
+#pragma unroll
+        for (int xi = 0; xi < 16; ++xi) {
+            float o[CV];
+#pragma unroll
+            for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
+            store_chan_vec<T>(vp + xi * plane, o);
+        }
+    }
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __restrict__ x, T* __restrict__ V, int N,
                                                                    int C, int H, int W, int pad, int th, int tw,
@@ -340,42 +383,89 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     const long p = ((long)n * th + ty) * tw + tx;
     const size_t plane = (size_t)Cp * Pp;
     T* vp = V + ((size_t)cq * Pp + p) * CV;
-    auto tile_of = [&](int ch, float (&out)[16]) {
-        float d[4][4];
-        const T* base = in_smem + ch * per_ch + (2 * tr) * ldsW + 2 * tc;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lds_row4<T>(base + i * ldsW, d[i]);
-        input_tile_transform(d, out);
-    };
-    if constexpr (sizeof(T) == 2) {
-        // 8 channels x 16 coordinates: rounded and packed two channels to a register as they are produced (64
-        // registers instead of 128 fp32 values held until the stores)
-        uint32_t wd[16][CV / 2];
-#pragma unroll
-        for (int ch = 0; ch < CV; ++ch) {
-            float vc[16];
-            tile_of(ch, vc);
-#pragma unroll
-            for (int xi = 0; xi < 16; ++xi) {
-                const uint32_t bits = __builtin_bit_cast(uint16_t, from_f32<T>(vc[xi]));
-                wd[xi][ch / 2] = (ch & 1) ? (wd[xi][ch / 2] | bits << 16) : bits;
-            }
-        }
-#pragma unroll
-        for (int xi = 0; xi < 16; ++xi)
-            *reinterpret_cast<uint4*>(vp + xi * plane) = make_uint4(wd[xi][0], wd[xi][1], wd[xi][2], wd[xi][3]);
-    } else {
-        float v[CV][16];
-#pragma unroll
-        for (int ch = 0; ch < CV; ++ch) tile_of(ch, v[ch]);
-#pragma unroll
-        for (int xi = 0; xi < 16; ++xi) {
-            float o[CV];
-#pragma unroll
-            for (int e = 0; e < CV; ++e) o[e] = v[e][xi];
-            store_chan_vec<T>(vp + xi * plane, o);
-        }
+    tile_from_lds_store<T>(in_smem + (2 * tr) * ldsW + 2 * tc, per_ch, ldsW, vp, plane);
+}
+
+// ---- input transform, NCHW source, small images -------------------------------------
+// Images whose tiles do not fill a workgroup (th*tw <= 128): a workgroup takes one image and NQ = 256 / (th*tw)
+// consecutive channel vectors.  Their channel planes are one contiguous run of the source, read word by word
+// (VEC elements per 4-byte or 2-byte word, a row being W / VEC words) with consecutive lanes on consecutive words,
+// and scattered into LDS planes [ch][2*th+2][2*tw+2] whose zero padding was written beforehand; thread
+// (channel vector, tile) then builds its tile as in the tiled kernel.  A thread walks the run 256 words at a
+// time; (stepC, stepH, stepW) is that stride split into planes, rows and words by the host, so the position of a
+// word costs two compares instead of two divisions.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void input_transform_nchw_small_kernel(const T* __restrict__ x, T* __restrict__ V,
+                                                                         int C, int H, int W, int pad, int th, int tw,
+                                                                         long Pp, int Cp, int NQ, int groups,
+                                                                         int in_blocks, int stepC, int stepH,
+                                                                         int stepW, FilterJob fj) {
+    constexpr int CV = ChanVec<T>::n;
+    constexpr int NB = 8;                              // loads in flight per thread
+    extern __shared__ __attribute__((aligned(16))) unsigned char in_smem_raw[];
+    if (fj.w && (int)blockIdx.x >= in_blocks) {
+        filter_job_blocks<T, 256>(fj, in_blocks);
+        return;
     }
+    typedef typename std::conditional<sizeof(T) * VEC == 4, uint32_t, uint16_t>::type raw_t;
+    typedef typename std::conditional<sizeof(T) == 4, uint32_t, uint16_t>::type elem_t;
+    T* in_smem = reinterpret_cast<T*>(in_smem_raw);
+    elem_t* smem_bits = reinterpret_cast<elem_t*>(in_smem_raw);
+    const int tid = threadIdx.x;
+    const int n = blockIdx.x / groups, cq0 = (blockIdx.x - n * groups) * NQ;
+    const int nq = min(NQ, Cp / CV - cq0);             // channel vectors of this workgroup
+    const int c0 = cq0 * CV;
+    const int nch = max(min(nq * CV, C - c0), 0);      // channels that exist; the others stay zero
+    const int rows = 2 * th + 2, ldsW = 2 * tw + 2, per_ch = rows * ldsW;
+    const int Ww = W / VEC;
+    const int words = nch * H * Ww;
+    const raw_t* xw = reinterpret_cast<const raw_t*>(x + ((size_t)n * C + c0) * H * W);
+
+    int idx = tid;
+    int ch = tid / (H * Ww);
+    int h = (tid - ch * H * Ww) / Ww;
+    int w = tid - ch * H * Ww - h * Ww;
+    raw_t buf[NB];
+    int dst[NB];                                       // LDS element index of the word's first element, -1: past the run
+    auto load_batch = [&]() {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            buf[i] = xw[min(idx, words - 1)];          // always a valid address; a word past the run is not stored
+            dst[i] = idx < words ? ch * per_ch + (h + pad) * ldsW + w * VEC + pad : -1;
+            idx += 256;
+            w += stepW;
+            if (w >= Ww) { w -= Ww; ++h; }
+            h += stepH;
+            if (h >= H) { h -= H; ++ch; }
+            ch += stepC;
+        }
+    };
+    if (words > 0) load_batch();
+    {
+        const int nvec = nq * CV * per_ch * (int)sizeof(T) / 16;   // per_ch is a multiple of 4 elements
+        uint4* z = reinterpret_cast<uint4*>(in_smem_raw);
+        for (int i = tid; i < nvec; i += 256) z[i] = make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();
+    for (int done = 0; done < words;) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            if (dst[i] >= 0) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) smem_bits[dst[i] + e] = (elem_t)(buf[i] >> (8 * sizeof(T) * e));
+            }
+        done += NB * 256;
+        if (done < words) load_batch();
+    }
+    __syncthreads();
+
+    const int tiles = th * tw;
+    const int q = tid / tiles, t = tid - q * tiles;
+    if (q >= nq) return;
+    const int ty = t / tw, tx = t - ty * tw;
+    const long p = (long)n * tiles + t;
+    T* vp = V + ((size_t)(cq0 + q) * Pp + p) * CV;
+    tile_from_lds_store<T>(in_smem + q * CV * per_ch + (2 * ty) * ldsW + 2 * tx, per_ch, ldsW, vp, (size_t)Cp * Pp);
 }
 
 // ---- input transform, NHWC source, LDS-transposed ---------------------------------------

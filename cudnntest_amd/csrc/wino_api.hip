@@ -190,6 +190,32 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
                            const FilterJob& fj = FilterJob{}) {
     constexpr int CV = ChanVec<T>::n;
     const int CQ = g.Cp / CV;
+    if (layout == WINO_NCHW && order == WINO_TILES_BATCH_MAJOR && g.th * g.tw <= 256) {
+        // small images: one image and NQ channel vectors per workgroup, thread per (channel vector, tile)
+        const int tiles = g.th * g.tw;
+        const int NQ = std::min(std::min(256 / tiles, 32), CQ);
+        const int groups = (CQ + NQ - 1) / NQ;
+        const long in_blocks = (long)g.N * groups;
+        const long extra = fj.w ? ((long)fj.Kp * CQ + 255) / 256 : 0;
+        if (in_blocks + extra >= (1L << 31)) return fail(WINO_ERR_UNSUPPORTED, "input transform: too many workgroups");
+        // 2-byte types move pairs (4 bytes per lane) when every channel plane starts 4-byte aligned
+        const bool vec2 = sizeof(T) == 2 && g.W % 2 == 0 && !misaligned(x, 4);
+        const int Ww = vec2 ? g.W / 2 : g.W;
+        const int stepC = 256 / (g.H * Ww), stepH = (256 - stepC * g.H * Ww) / Ww,
+                  stepW = 256 - stepC * g.H * Ww - stepH * Ww;
+        const size_t lds = (size_t)NQ * CV * (2 * g.th + 2) * (2 * g.tw + 2) * sizeof(T);
+        dim3 grid((unsigned)(in_blocks + extra)), block(256);
+        if (vec2)
+            hipLaunchKernelGGL((input_transform_nchw_small_kernel<T, (sizeof(T) == 2 ? 2 : 1)>), grid, block, lds, st,
+                               (const T*)x, (T*)V, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, NQ, groups,
+                               (int)in_blocks, stepC, stepH, stepW, fj);
+        else
+            hipLaunchKernelGGL((input_transform_nchw_small_kernel<T, 1>), grid, block, lds, st, (const T*)x, (T*)V,
+                               g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, NQ, groups, (int)in_blocks, stepC, stepH,
+                               stepW, fj);
+        LAUNCH_CHECK("input_transform_nchw_small");
+        return WINO_OK;
+    }
     if (input_is_nchw_tiled(layout, order, g)) {
         // TR x TC tiles per workgroup, TR*TC <= 256, halo of CV channels in LDS (<= 60 KB).
         // TR is kept a multiple of 8 when it can be, so a workgroup's run of V (TR*tw
@@ -220,18 +246,28 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
     }
     if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && g.C % CV == 0 &&
         (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-        constexpr int TC = 32, NQ = 8, TR = 2;
-        const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
-        const long in_blocks = (long)g.N * rowBlocks * colBlocks;
-        const int gy = (CQ + NQ - 1) / NQ;
-        // a filter job gets workgroups appended along x: enough, over all y, for one thread per (filter, channel vector)
-        const long extra = fj.w ? ((long)fj.Kp * CQ + (long)TC * NQ * gy - 1) / ((long)TC * NQ * gy) : 0;
-        if (in_blocks + extra >= (1L << 31)) return fail(WINO_ERR_UNSUPPORTED, "input transform: too many workgroups");
-        dim3 grid((unsigned)(in_blocks + extra), gy), block(TC * NQ);
-        hipLaunchKernelGGL((input_transform_nhwc_kernel<T, TC, NQ, TR>), grid, block, 0, st, (const T*)x, (T*)V, g.N,
-                           g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, rowBlocks, fj, (int)in_blocks);
-        LAUNCH_CHECK("input_transform_nhwc");
-        return WINO_OK;
+        // 256 threads = TC tile columns x NQ channel vectors.  Narrow images take narrow blocks (a 7-tile row in a
+        // 32-wide block leaves three threads in four without a tile) as long as the layer has the channel vectors
+        // to fill the other axis.
+        auto launch = [&](auto tc_c) -> int {
+            constexpr int TC = decltype(tc_c)::value, NQ = 256 / TC, TR = 2;
+            const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
+            const long in_blocks = (long)g.N * rowBlocks * colBlocks;
+            const int gy = (CQ + NQ - 1) / NQ;
+            // a filter job gets workgroups appended along x: enough, over all y, for one thread per (filter, channel vector)
+            const long extra = fj.w ? ((long)fj.Kp * CQ + (long)TC * NQ * gy - 1) / ((long)TC * NQ * gy) : 0;
+            if (in_blocks + extra >= (1L << 31))
+                return fail(WINO_ERR_UNSUPPORTED, "input transform: too many workgroups");
+            dim3 grid((unsigned)(in_blocks + extra), gy), block(TC * NQ);
+            hipLaunchKernelGGL((input_transform_nhwc_kernel<T, TC, NQ, TR>), grid, block, 0, st, (const T*)x, (T*)V,
+                               g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, rowBlocks, fj,
+                               (int)in_blocks);
+            LAUNCH_CHECK("input_transform_nhwc");
+            return WINO_OK;
+        };
+        if (g.tw <= 8 && CQ >= 32) return launch(std::integral_constant<int, 8>{});
+        if (g.tw <= 16 && CQ >= 16 && sizeof(T) == 2) return launch(std::integral_constant<int, 16>{});
+        return launch(std::integral_constant<int, 32>{});
     }
     const long in_blocks = (g.P + 255) / 256;
     const long extra = fj.w ? (fj.Kp + 255) / 256 : 0;          // x all CQ rows of the grid

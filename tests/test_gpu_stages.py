@@ -53,6 +53,46 @@ def test_input_transform(oracle, layout, order, shape, pad):
     assert not V[:, C:, :P].any(), "channel padding must be zero"
 
 
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape,pad", [((2, 170, 14, 14), 1),     # several channel vectors per workgroup, ragged last group
+                                       ((3, 136, 7, 7), 1),       # 16 tiles per image
+                                       ((2, 20, 22, 20), 1),      # two channel vectors per workgroup
+                                       ((1, 9, 28, 30), 1),       # one image per workgroup, channel padding
+                                       ((2, 12, 15, 13), 0),      # odd width: 2-byte elements move one by one
+                                       ((2, 12, 16, 12), 0),      # no padding, even width
+                                       ((2, 512, 14, 14), 1),     # NHWC: 8-tile-wide blocks
+                                       ((1, 256, 28, 28), 1),     # NHWC: 16-tile-wide blocks (2-byte)
+                                       ((300, 4, 2, 2), 1)])      # one tile per image, many images
+def test_input_transform_small_images(oracle, layout, dtype, shape, pad):
+    """Images that fit one workgroup take their own NCHW kernel (a contiguous run of channel planes per workgroup)
+    and narrow NHWC blocks: bit-exact on small integers for every element type."""
+    N, C, H, W = shape
+    x = synth.small_ints(N * C * H * W, 91 + sum(shape), -8, 8).reshape(N, C, H, W)
+    xl = synth.act_to_layout(x, layout)
+    V = unpack_operand(ops.input_transform(dev(xl, dtype), pad, layout, ops.TILES_BATCH_MAJOR), dtype)
+    want = oracle.wino_input_transform(xl, pad, layout)
+    th, tw = oracle.wino_tiles(2, H, W, pad)
+    P = N * th * tw
+    assert np.array_equal(V[:, :C, :P], want)
+    assert not V[:, C:, :P].any(), "channel padding must be zero"
+
+
+def test_input_transform_small_images_unaligned_view(oracle):
+    """A 2-byte NCHW tensor that starts on an odd element: same bits as the aligned one."""
+    N, C, H, W = 2, 24, 14, 14
+    x = synth.small_ints(N * C * H * W, 5, -8, 8).reshape(N, C, H, W)
+    flat = torch.zeros(N * C * H * W + 1, dtype=torch.bfloat16, device="cuda")
+    flat[1:] = dev(x, ops.BF16).reshape(-1)
+    view = flat[1:].view(N, C, H, W)
+    assert view.data_ptr() % 4 == 2
+    got = ops.input_transform(view, 1, ops.NCHW, ops.TILES_BATCH_MAJOR)
+    want = ops.input_transform(dev(x, ops.BF16), 1, ops.NCHW, ops.TILES_BATCH_MAJOR)
+    assert torch.equal(got, want)
+    ref = oracle.wino_input_transform(x, 1, ops.NCHW)
+    assert np.array_equal(unpack_operand(got, ops.BF16)[:, :C, :N * 49], ref)
+
+
 @pytest.mark.parametrize("porder", [ops.PRODUCT_KP, ops.PRODUCT_PK])
 @pytest.mark.parametrize("C,K,P", [(16, 128, 128), (3, 5, 30), (64, 64, 784), (40, 130, 300), (256, 256, 512)])
 def test_batched_gemm(oracle, C, K, P, porder):
