@@ -78,6 +78,24 @@ def test_input_transform_small_images(oracle, layout, dtype, shape, pad):
     assert not V[:, C:, :P].any(), "channel padding must be zero"
 
 
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape,pad", [((2, 17, 9, 6), 1), ((4, 16, 28, 28), 1), ((6, 40, 8, 7), 0), ((32, 8, 12, 12), 1),
+                                       ((3, 9, 6, 6), 1)])
+def test_input_transform_chwn_two_byte(oracle, dtype, shape, pad):
+    """2-byte CHWN sources, batch-minor tiles (eight channels per thread, lanes along n): bit-exact on small
+    integers, channel padding zero."""
+    N, C, H, W = shape
+    x = synth.small_ints(N * C * H * W, 123 + sum(shape), -8, 8).reshape(N, C, H, W)
+    xl = synth.act_to_layout(x, ops.CHWN)
+    V = unpack_operand(ops.input_transform(dev(xl, dtype), pad, ops.CHWN, ops.TILES_BATCH_MINOR), dtype)
+    want = oracle.wino_input_transform(xl, pad, ops.CHWN)
+    th, tw = oracle.wino_tiles(2, H, W, pad)
+    P = N * th * tw
+    got = V[:, :C, :P][:, :, np.argsort(batch_minor_perm(N, th, tw))]
+    assert np.array_equal(got, want)
+    assert not V[:, C:, :P].any(), "channel padding must be zero"
+
+
 def test_input_transform_small_images_unaligned_view(oracle):
     """A 2-byte NCHW tensor that starts on an odd element: same bits as the aligned one."""
     N, C, H, W = 2, 24, 14, 14
