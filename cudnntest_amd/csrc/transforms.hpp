@@ -171,14 +171,23 @@ __global__ __launch_bounds__(256) void input_transform_generic_kernel(const T* _
                                                                        ActStrides s, int N, int C, int H, int W,
                                                                        int pad, int th, int tw, long P, long Pp,
                                                                        int Cp, int order, FilterJob fj,
-                                                                       int in_blocks) {
+                                                                       int in_blocks, int cq_fast) {
     constexpr int CV = ChanVec<T>::n;
     if (fj.w && (int)blockIdx.x >= in_blocks) {
         filter_job_blocks<T, 256>(fj, in_blocks);
         return;
     }
-    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const int cq = blockIdx.y;
+    // Workgroups are dispatched along x first.  cq_fast re-deals the ids so that the channel vectors of one run of
+    // tiles follow each other instead of the tile runs of one channel vector (faster while x and V together fit the
+    // last-level cache, slower beyond: measured on CHWN sources).
+    long pb = blockIdx.x;
+    int cq = blockIdx.y;
+    if (cq_fast) {
+        const long lin = (long)blockIdx.y * in_blocks + blockIdx.x;
+        pb = lin / gridDim.y;
+        cq = (int)(lin - pb * gridDim.y);
+    }
+    const long p = pb * blockDim.x + threadIdx.x;
     if (p >= P) return;
     int n, ty, tx;
     decode_tile(p, order, N, th, tw, n, ty, tx);
