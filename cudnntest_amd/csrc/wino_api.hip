@@ -672,7 +672,7 @@ int conv_f4_impl(int src, int dst, int dtype, unsigned flags, int N, int C, int 
     return wino_f4_output_transform(dst, dtype, order, porder, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
 }
 
-int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
+int conv_pass(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
               const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
@@ -754,10 +754,57 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
 
 __global__ void warmup_kernel() {}
 
+// How many passes over the batch a layer call makes.  The epilogue pipeline of a 2-byte layer is bound by memory
+// on both sides of V (written by the input transform, read by the GEMM); when V is much larger than the 256 MB
+// last-level cache, running the two kernels on one part of the batch after the other lets the GEMM find V still
+// cached and the next pass overwrite the same addresses.  Batch-major tensors only (a part of the batch is then a
+// contiguous slice of x, V and y).  Measured (bf16, N=32, NCHW): C=K=128, H=112 (V 411 MB) 280 us in one pass,
+// 236 in two, 253 in three; C=64, K=128, H=112 (205 MB) 158 -> 143 in two; C=K=256, H=56 (205 MB, but only 1568
+// workgroups) 166 -> 172 in two: a pass aims at 105 MB of V and keeps at least ~1500 GEMM workgroups (two rounds
+// of the chip).
+int batch_passes(int src, int dst, int dtype, int algo, const Geometry& g) {
+    if (algo != WINO_ALGO_EPILOGUE || dtype == WINO_F32 || src == WINO_CHWN || dst == WINO_CHWN) return 1;
+    const double v_bytes = 16.0 * (double)g.P * g.Cp * dtype_size(dtype);
+    const long wgs = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
+    const long by_cache = (long)(v_bytes / 105e6 + 0.5), by_work = wgs / 1500;
+    return (int)std::max(1L, std::min<long>(g.N, std::min(by_cache, by_work)));
+}
+
+int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
+              const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
+    Geometry g;
+    int passes = 1;
+    if (valid_layout(src) && valid_layout(dst) && valid_dtype(dtype) && x && y && (w || Upre) &&
+        make_geometry(dtype, N, C, K, H, W, pad, &g) && algo >= WINO_ALGO_AUTO && algo <= WINO_ALGO_DIRECT) {
+        if (algo == WINO_ALGO_AUTO) algo = (w && direct_ok(dst, flags, g)) ? WINO_ALGO_DIRECT : pick_algo(src, dtype, g);
+        passes = batch_passes(src, dst, dtype, algo, g);
+    }
+    if (passes <= 1) return conv_pass(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, Upre, bias, y, stream);
+    const size_t es = dtype_size(dtype);
+    const size_t x_img = (size_t)C * H * W * es;
+    const size_t y_img = (size_t)K * ((flags & WINO_FLAG_POOL2) ? (size_t)(g.Ho / 2) * (g.Wo / 2) : (size_t)g.Ho * g.Wo) * es;
+    const int per = (N + passes - 1) / passes;
+    for (int n0 = 0; n0 < N; n0 += per) {
+        const int nn = std::min(per, N - n0);
+        const int rc = conv_pass(src, dst, dtype, algo, flags, nn, C, K, H, W, pad, (const char*)x + n0 * x_img,
+                                 Upre ? nullptr : w, Upre, bias, (char*)y + n0 * y_img, stream);
+        if (rc) return rc;
+        if (!Upre) {
+            // the first pass left the transformed filters at the head of the arena; the later ones reuse them
+            Geometry gp;
+            make_geometry(dtype, nn, C, K, H, W, pad, &gp);
+            void* base = nullptr;
+            const int rc2 = arena_get(scratch_layout(gp, dtype).total, &base);
+            if (rc2) return rc2;
+            Upre = (char*)base + scratch_layout(gp, dtype).u_off;
+        }
+    }
+    return WINO_OK;
+}
+
 }  // namespace
 
 extern "C" {
-
 int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
               const void* x, const void* w, void* y, void* stream) {
     if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
