@@ -322,7 +322,7 @@ int launch_gemm_t(int nxi, int Cp, int Kp, long Pp, const void* U, const void* V
         return fail(WINO_ERR_INVALID, "reduction of %d stages cannot be cut into %d runs", chunks, splits);
     const bool xm = xcd_map_ok(pTiles);
     dim3 grid((unsigned)((xm ? (pTiles + 7) / 8 * 8 : pTiles) * kTiles), nxi, splits), block(256);
-    constexpr int RING = sizeof(T) == 4 ? 4 : 2;     // from measurements, see gemm.hpp
+    constexpr int RING = sizeof(T) == 4 ? 4 : 3;     // from measurements, see gemm.hpp
     hipLaunchKernelGGL((gemm_128x128_kernel<T, NV, PK, RING>), grid, block, 0, st, (const T*)U, (const T*)V, Mo, Cp,
                        Kp, Pp, kTiles, pTiles, per, xm ? 1 : 0);
     LAUNCH_CHECK("batched_gemm");
