@@ -195,7 +195,8 @@ __global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* _
             for (int b = 0; b < 4; ++b) o[a][b] = fmaxf(o[a][b], 0.f);
     }
     T* yp = y + n * s.n + k * s.c;
-    if (s.w == 1 && (Wo & 3) == 0 && (s.h & 3) == 0 && (s.c & 3) == 0 && (s.n & 3) == 0) {
+    if (s.w == 1 && (Wo & 3) == 0 && (s.h & 3) == 0 && (s.c & 3) == 0 && (s.n & 3) == 0 &&
+        (reinterpret_cast<uintptr_t>(y) & (4 * sizeof(T) - 1)) == 0) {
         // W-contiguous destination, rows a multiple of 4 wide: one 4-element store per output row
         struct alignas(4 * sizeof(T)) Quad { T e[4]; };
 #pragma unroll

@@ -51,8 +51,26 @@ bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p
 size_t elem_bytes(int dtype) { return dtype == WINO_F32 ? 4 : 2; }
 bool valid_order(int o) { return o == WINO_TILES_BATCH_MAJOR || o == WINO_TILES_BATCH_MINOR; }
 
-// ---- scratch arena: one grow-only allocation per device ------------------------
 constexpr int kMaxDevices = 16;
+
+// Compute units of the current device, asked once per device.  The launch heuristics below (how many workgroups
+// are resident at once, when a reduction is cut so that every CU has work) are derived from it; an MI355X has 256
+// in 8 XCDs of 32, which is also what is assumed if the runtime cannot tell.
+int device_cus() {
+    static int cus[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+// workgroups of the row-at-a-time GEMM resident at once: 2 per CU (64 KB of LDS, fp32) or 3 (48 KB, 2-byte operands)
+long rows_slots(int dtype) { return (long)device_cus() * (dtype == WINO_F32 ? 2 : 3); }
+
+// ---- scratch arena: one grow-only allocation per device ------------------------
 struct Arena {
     void* own = nullptr;
     size_t own_bytes = 0;
@@ -92,6 +110,21 @@ int arena_get(size_t bytes, void** out) {
     return WINO_OK;
 }
 
+// Where a whole-layer call takes its scratch from: the device's arena (grown on demand), or a fixed buffer that
+// is never grown.
+struct ScratchSource {
+    void* fixed = nullptr;
+    size_t fixed_bytes = 0;
+    int get(size_t bytes, void** out) const {
+        if (!fixed) return arena_get(bytes, out);
+        if (bytes > fixed_bytes)
+            return fail(WINO_ERR_WORKSPACE, "this problem needs %zu bytes of scratch, the built-in buffer holds %zu",
+                        bytes, fixed_bytes);
+        *out = fixed;
+        return WINO_OK;
+    }
+};
+
 unsigned long arena_generation(int dev) {
     std::lock_guard<std::mutex> lk(g_arena_mu);
     return g_arena[dev].generation;
@@ -103,6 +136,7 @@ struct StageSpan {
     hipEvent_t a, b;
 };
 bool g_timing = false;
+thread_local bool t_no_timing = false;       // set while a call that must not create events is running
 std::vector<StageSpan> g_spans;
 std::mutex g_spans_mu;
 
@@ -111,7 +145,7 @@ struct StageScope {
     int stage;
     hipStream_t st;
     hipEvent_t a = nullptr, b = nullptr;
-    StageScope(int stage_, hipStream_t st_) : on(g_timing), stage(stage_), st(st_) {
+    StageScope(int stage_, hipStream_t st_) : on(g_timing && !t_no_timing), stage(stage_), st(st_) {
         if (on) {
             on = hipEventCreate(&a) == hipSuccess && hipEventCreate(&b) == hipSuccess &&
                  hipEventRecord(a, st) == hipSuccess;
@@ -149,22 +183,50 @@ bool xcd_map_ok(int pTiles) {
 int gemm_splits(int dtype, int Cp, int Kp, long Pp) {
     const long wgs = 16L * (Kp / GEMM_BM) * (Pp / GEMM_BN);
     const int chunks = Cp / c_pad(dtype);          // stages of the reduction: 4 channel vectors each
-    const long s = std::min<long>(256 / std::max<long>(wgs, 1), chunks / 4);
+    const long s = std::min<long>(device_cus() / std::max<long>(wgs, 1), chunks / 4);
     if (s <= 1) return 1;
     const int per = (int)((chunks + s - 1) / s);
     return (chunks + per - 1) / per;
 }
 
-Scratch scratch_layout(const Geometry& g, int dtype) {
+// The epilogue GEMM's cut-up last round.  Workgroups resident at once: 2 per CU (64 KB of LDS, fp32) or 3 (48 KB,
+// 2-byte operands).  If the last round of 64x64 patches would occupy at most 60 % of them, its patches are cut
+// into TAIL workgroups, one Winograd row each (measured: a last round of 272 of 512 gains 8 %, one of 424 loses
+// 4 %).  fp32 only: with 2-byte operands a patch is short and the cut costs more than the idle CUs (measured).
+// Returns the number of groups of 8 tile patches (x all filter tiles) that are cut, 0 for none; each cut patch
+// needs an arrival counter and four rows of 64 x 256 partial sums.
+int rows_tail_groups(int dtype, const Geometry& g) {
+    if (dtype != WINO_F32) return 0;
+    const int kTiles = (g.K + GO_T - 1) / GO_T;
+    const int pTiles = (int)((g.P + GO_T - 1) / GO_T);
+    const int pGroups = (pTiles + 7) / 8, group = 8 * kTiles;
+    const long slots = rows_slots(dtype), real = (long)pTiles * kTiles;
+    if (!(real > slots && real % slots != 0 && 5 * (real % slots) <= 3 * slots)) return 0;
+    const int tail_groups = (int)((real % slots + group - 1) / group);
+    if (tail_groups >= pGroups || (long)tail_groups * group > (long)(kCounterBytes / sizeof(int))) return 0;
+    return tail_groups;
+}
+inline size_t tail_part_bytes(int dtype, const Geometry& g) {
+    return (size_t)rows_tail_groups(dtype, g) * 8 * ((g.K + GO_T - 1) / GO_T) * 4 * 64 * 256 * sizeof(float);
+}
+
+// What a pipeline keeps in scratch: STAGED (and the F(4x4) mode) U, V and the product; EPILOGUE U, V and the
+// partial sums of its cut-up workgroups; FUSED U only.  The default is the largest of them.
+Scratch scratch_layout(const Geometry& g, int dtype, int algo = WINO_ALGO_STAGED) {
     const size_t es = dtype_size(dtype);
     const size_t nxi = (size_t)(g.m + 2) * (g.m + 2);
     auto al = [](size_t v) { return (v + 255) / 256 * 256; };
     Scratch s;
     s.u_off = kCounterBytes;
     s.v_off = s.u_off + al(nxi * (size_t)g.Cp * g.Kp * es);
+    if (algo == WINO_ALGO_FUSED) {
+        s.m_off = s.total = s.v_off;
+        return s;
+    }
     s.m_off = s.v_off + al(nxi * (size_t)g.Cp * g.Pp * es);
     const size_t copies = g.m == 2 ? (size_t)gemm_splits(dtype, g.Cp, g.Kp, g.Pp) : 1;
-    s.total = s.m_off + al(copies * nxi * (size_t)g.Kp * g.Pp * sizeof(float));
+    const size_t product = copies * nxi * (size_t)g.Kp * g.Pp * sizeof(float);
+    s.total = s.m_off + al(algo == WINO_ALGO_EPILOGUE ? tail_part_bytes(dtype, g) : product);
     return s;
 }
 
@@ -227,7 +289,7 @@ int launch_input_transform(int layout, int order, const Geometry& g, const void*
         const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
         const int ldsW = 2 * TC + 2;
         // 2-byte types move image-aligned column pairs (4 bytes per lane) when every row starts 4-byte aligned
-        const bool vec2 = sizeof(T) == 2 && (g.W % 2 == 0);
+        const bool vec2 = sizeof(T) == 2 && g.W % 2 == 0 && !misaligned(x, 4);
         const int span = vec2 ? ldsW + 2 : ldsW;          // loaded columns per row (one extra pair on the left)
         const int perUnit = vec2 ? 128 : 64;
         int chunkLog2 = 0;
@@ -363,20 +425,9 @@ int launch_gemm_rows_t(int order, unsigned flags, const void* bias, const Geomet
     const int group = 8 * kTiles;                         // workgroup ids per group of 8 tile patches
     const ActStrides ys = out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo);
     const Epilogue ep = make_epilogue(flags, bias);
-    // Workgroups resident at once: 256 CUs x 2 (64 KB of LDS, fp32) or x 3 (48 KB, 2-byte operands).  If the
-    // last round would occupy at most 60 % of them, its patches are cut into TAIL workgroups (measured: a last
-    // round of 272 of 512 gains 8 %, one of 424 loses 4 %).
-    const long slots = 256L * (sizeof(T) == 2 ? 3 : 2);
-    const long real = (long)pTiles * kTiles;
-    int tail_groups = 0;
-    // (fp32 only: with 2-byte operands a patch is short and the cut costs more than the idle CUs, measured)
-    if (sizeof(T) == 4 && ts.part && real > slots && real % slots != 0 && 5 * (real % slots) <= 3 * slots) {
-        tail_groups = (int)((real % slots + group - 1) / group);
-        const long tail_ids = (long)tail_groups * group;
-        if (tail_groups >= pGroups || tail_ids > (long)(kCounterBytes / sizeof(int)) ||
-            (size_t)tail_ids * 4 * 64 * 256 * sizeof(float) > ts.part_bytes)
-            tail_groups = 0;
-    }
+    // a small last round is cut into TAIL workgroups (rows_tail_groups) when the caller brought scratch for it
+    int tail_groups = ts.part ? rows_tail_groups(sizeof(T) == 4 ? WINO_F32 : WINO_F16, g) : 0;
+    if (tail_part_bytes(sizeof(T) == 4 ? WINO_F32 : WINO_F16, g) > ts.part_bytes) tail_groups = 0;
     const bool xm = tail_groups > 0 || xcd_map_ok(pTiles);      // (a cut-up last round implies hundreds of patches)
     const int main_ids = xm ? (pGroups - tail_groups) * group : pTiles * kTiles;
     hipLaunchKernelGGL((gemm_rows_kernel<T, SWAP, NVG, RING>), dim3((unsigned)(main_ids + tail_groups * group * 4)),
@@ -616,8 +667,8 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
         // many channels: the 128x128 GEMM's lower L2 traffic per flop wins, unless there are few tiles or the
         // 64x64 patches fill their rounds of 512 resident workgroups (a small last round is cut up, see
         // launch_gemm_rows_t)
-        const long rem = patches % 512;
-        const bool full_rounds = patches > 512 && (rem == 0 || 5 * rem <= 3 * 512);
+        const long slots = rows_slots(WINO_F32), rem = patches % slots;
+        const bool full_rounds = patches > slots && (rem == 0 || 5 * rem <= 3 * slots);
         return (g.P <= 4096 || full_rounds) ? WINO_ALGO_EPILOGUE : WINO_ALGO_STAGED;
     }
     // 16-bit operands: the fp32 product tensor is the largest HBM stream, so STAGED only for tiny problems;
@@ -635,15 +686,15 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     return WINO_ALGO_EPILOGUE;
 }
 
-int conv_f4_impl(int src, int dst, int dtype, unsigned flags, int N, int C, int K, int H, int W, int pad,
-                 const void* x, const void* w, const void* Upre, void* y, void* stream) {
+int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned flags, int N, int C, int K, int H, int W,
+                 int pad, const void* x, const void* w, const void* Upre, void* y, void* stream) {
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g, 4))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype);
     void* base = nullptr;
-    int rc = arena_get(sc.total, &base);
+    int rc = ss.get(sc.total, &base);
     if (rc) return rc;
     char* b = (char*)base;
     void* U = b + sc.u_off;
@@ -672,8 +723,8 @@ int conv_f4_impl(int src, int dst, int dtype, unsigned flags, int N, int C, int 
     return wino_f4_output_transform(dst, dtype, order, porder, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
 }
 
-int conv_pass(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
-              const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
+int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
+              int W, int pad, const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
     if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_DIRECT) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
@@ -700,12 +751,12 @@ int conv_pass(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         if (bias || (flags & WINO_FLAG_POOL2))
             return fail(WINO_ERR_UNSUPPORTED, "bias and pooling are not built for the F(4x4,3x3) mode");
     }
-    if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(src, dst, dtype, flags, N, C, K, H, W, pad, x, w, Upre, y, stream);
+    if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(ss, src, dst, dtype, flags, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
     hipStream_t st = (hipStream_t)stream;
-    const Scratch sc = scratch_layout(g, dtype);
+    const Scratch sc = scratch_layout(g, dtype, algo);
     void* base = nullptr;
-    int rc = arena_get(sc.total, &base);
+    int rc = ss.get(sc.total, &base);
     if (rc) return rc;
     char* b = (char*)base;
     void* U = b + sc.u_off;
@@ -770,8 +821,8 @@ int batch_passes(int src, int dst, int dtype, int algo, const Geometry& g) {
     return (int)std::max(1L, std::min<long>(g.N, std::min(by_cache, by_work)));
 }
 
-int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
-              const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
+int conv_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
+              int W, int pad, const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     Geometry g;
     int passes = 1;
     if (valid_layout(src) && valid_layout(dst) && valid_dtype(dtype) && x && y && (w || Upre) &&
@@ -779,14 +830,14 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
         if (algo == WINO_ALGO_AUTO) algo = (w && direct_ok(dst, flags, g)) ? WINO_ALGO_DIRECT : pick_algo(src, dtype, g);
         passes = batch_passes(src, dst, dtype, algo, g);
     }
-    if (passes <= 1) return conv_pass(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, Upre, bias, y, stream);
+    if (passes <= 1) return conv_pass(ss, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, Upre, bias, y, stream);
     const size_t es = dtype_size(dtype);
     const size_t x_img = (size_t)C * H * W * es;
     const size_t y_img = (size_t)K * ((flags & WINO_FLAG_POOL2) ? (size_t)(g.Ho / 2) * (g.Wo / 2) : (size_t)g.Ho * g.Wo) * es;
     const int per = (N + passes - 1) / passes;
     for (int n0 = 0; n0 < N; n0 += per) {
         const int nn = std::min(per, N - n0);
-        const int rc = conv_pass(src, dst, dtype, algo, flags, nn, C, K, H, W, pad, (const char*)x + n0 * x_img,
+        const int rc = conv_pass(ss, src, dst, dtype, algo, flags, nn, C, K, H, W, pad, (const char*)x + n0 * x_img,
                                  Upre ? nullptr : w, Upre, bias, (char*)y + n0 * y_img, stream);
         if (rc) return rc;
         if (!Upre) {
@@ -794,9 +845,10 @@ int conv_impl(int src, int dst, int dtype, int algo, unsigned flags, int N, int 
             Geometry gp;
             make_geometry(dtype, nn, C, K, H, W, pad, &gp);
             void* base = nullptr;
-            const int rc2 = arena_get(scratch_layout(gp, dtype).total, &base);
+            const Scratch scp = scratch_layout(gp, dtype, algo);
+            const int rc2 = ss.get(scp.total, &base);
             if (rc2) return rc2;
-            Upre = (char*)base + scratch_layout(gp, dtype).u_off;
+            Upre = (char*)base + scp.u_off;
         }
     }
     return WINO_OK;
@@ -808,23 +860,23 @@ extern "C" {
 int wino_conv(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
               const void* x, const void* w, void* y, void* stream) {
     if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
-    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, nullptr, y, stream);
+    return conv_impl(ScratchSource{}, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, nullptr, y, stream);
 }
 int wino_conv_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
                  const void* x, const void* w, const void* bias, void* y, void* stream) {
     if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
-    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, bias, y, stream);
+    return conv_impl(ScratchSource{}, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, bias, y, stream);
 }
 
 int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W,
                        int pad, const void* x, const void* U, void* y, void* stream) {
     if (!U) return fail(WINO_ERR_INVALID, "null transformed-filter pointer");
-    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, nullptr, y, stream);
+    return conv_impl(ScratchSource{}, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, nullptr, y, stream);
 }
 int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W,
                           int pad, const void* x, const void* U, const void* bias, void* y, void* stream) {
     if (!U) return fail(WINO_ERR_INVALID, "null transformed-filter pointer");
-    return conv_impl(src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, bias, y, stream);
+    return conv_impl(ScratchSource{}, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, bias, y, stream);
 }
 
 int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int pad) {
@@ -1141,7 +1193,7 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
     for (int l = 0; l < n; ++l) {
         const auto& L = s->layers[l];
         void* out = l + 1 == n ? y : s->act[l & 1];
-        int rc = conv_impl(L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
+        int rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
                            L.wraw, L.U, L.has_bias ? L.bias : nullptr, out, stream);
         if (rc) return rc;
         in = out;
@@ -1217,6 +1269,8 @@ int wino_stack_set_layer(wino_stack_t* s, int layer, const void* w, const void* 
     if (!s || !w) return fail(WINO_ERR_INVALID, "null pointer");
     if (layer < 0 || layer >= (int)s->layers.size()) return fail(WINO_ERR_INVALID, "no layer %d", layer);
     auto& L = s->layers[layer];
+    // a recorded pass holds the layer's bias pointer (or its absence) in its kernel arguments
+    stack_drop_graph(s);
     int rc = wino_filter_transform(L.layout_in, s->dtype, L.K, L.C, w, L.U, stream);
     if (rc) return rc;
     if (L.wraw)

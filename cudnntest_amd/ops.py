@@ -192,8 +192,12 @@ class ConvStack:
         import ctypes
         descs = (_lib.StackLayer * len(layers))()
         prev = None
+        self._ck = []                      # (C, K) of every layer: what set_layer's tensors must hold
+        c = C
         for d, L in zip(descs, layers):
             d.K = int(L["K"])
+            self._ck.append((c, d.K))
+            c = d.K
             d.layout_in = int(L.get("layout_in", prev if prev is not None else NCHW))
             d.layout_out = int(L.get("layout_out", d.layout_in))
             d.flags = (FLAG_RELU if L.get("relu", False) else 0) | (FLAG_POOL2 if L.get("pool", False) else 0)
@@ -213,6 +217,12 @@ class ConvStack:
     def set_layer(self, layer, w, bias=None):
         if w.dtype != self.dtype or (bias is not None and bias.dtype != self.dtype):
             raise TypeError("filters and bias must have the stack's dtype")
+        if 0 <= layer < len(self._ck):     # (a layer that does not exist is the library's to refuse)
+            C, K = self._ck[layer]
+            if w.numel() != 9 * K * C:
+                raise ValueError(f"layer {layer} takes a bank of {K} x {C} 3x3 filters, got {w.numel()} elements")
+            if bias is not None and bias.numel() != K:
+                raise ValueError(f"layer {layer} takes {K} bias values, got {bias.numel()}")
         _lib.check(_lib.load().wino_stack_set_layer(self._h, layer, _ptr(w), _ptr(bias) if bias is not None else None,
                                                     _stream()), "wino_stack_set_layer")
 

@@ -211,3 +211,22 @@ def test_staged_gemm_with_its_reduction_cut_into_runs(oracle, shape):
         from gpu_util import rounded
         ref = oracle.direct_conv(rounded(xf, dtype, oracle), rounded(wf, dtype, oracle), 1)
         assert oracle.rel_l2(got, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("algo", [ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_STAGED_F4])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16, ops.BF16])
+def test_element_aligned_views_of_images_larger_than_a_workgroup(dtype, algo):
+    """H=W=40 (400 tiles per image: the LDS-tiled NCHW input transform, whose 2-byte form loads 4-byte pairs
+    only from 4-byte aligned tensors) and, for F(4x4,3x3), an output tensor whose 4-element row stores need a
+    16- or 8-byte aligned base: odd element offsets give the bits of the aligned call."""
+    from gpu_util import TORCH_DT
+    N, C, K, H = 2, 16, 64, 40
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = (torch.rand((N, C, H, H), device="cuda", generator=g) - 0.5).to(TORCH_DT[dtype])
+    w = (torch.randn((K, C, 3, 3), device="cuda", generator=g) * 0.1).to(TORCH_DT[dtype])
+    want = ops.conv(x, w, 1, ops.NCHW, algo=algo, relu=True)
+    for shift in (1, 3):
+        out = _view_at(torch.zeros_like(want), shift)
+        got = ops.conv(_view_at(x, shift), _view_at(w, shift), 1, ops.NCHW, algo=algo, relu=True, out=out)
+        assert got.data_ptr() % 8 != 0
+        assert torch.equal(got, want), (shift, (got.float() - want.float()).abs().max().item())

@@ -127,3 +127,32 @@ def test_stack_replayed_from_a_graph_matches_eager_launches(oracle):
         out2.zero_()
         assert torch.equal(st.forward(x2, out=out2, graph=True), want2), rep
     st.close()
+
+
+def test_stack_graph_follows_a_change_of_bias(oracle):
+    """set_layer after a recorded pass -- a bias added, then removed again -- is seen by the next replay: the
+    recorded launches hold the bias pointer (or its absence), so setting a layer drops the recording."""
+    N, C, H = 2, 3, 12
+    layers = [dict(K=8, relu=True), dict(K=8, relu=True)]
+    params = make_params(oracle, C, layers, ops.F32)
+    st = ops.ConvStack(torch.float32, N, C, H, H, layers)
+    x = dev(synth.uniform_pm1(N * C * H * H, 0xB5).reshape(N, C, H, H))
+    out = torch.empty(st.out_shape, device="cuda")
+    for i, (w, b) in enumerate(params):
+        st.set_layer(i, dev(w), None)
+    no_bias = st.forward(x).clone()
+    assert torch.equal(st.forward(x, out=out, graph=True), no_bias)
+    for i, (w, b) in enumerate(params):
+        st.set_layer(i, dev(w), dev(b + 0.5))
+    with_bias = st.forward(x).clone()
+    assert not torch.equal(with_bias, no_bias)
+    assert torch.equal(st.forward(x, out=out, graph=True), with_bias)
+    assert torch.equal(st.forward(x, out=out, graph=True), with_bias)
+    st.set_layer(1, dev(params[1][0]), None)
+    want = st.forward(x).clone()
+    assert torch.equal(st.forward(x, out=out, graph=True), want)
+    with pytest.raises(ValueError):          # a bank of the wrong size is refused before it reaches the device
+        st.set_layer(0, torch.zeros((8, 4, 3, 3), device="cuda"))
+    with pytest.raises(ValueError):
+        st.set_layer(0, dev(params[0][0]), torch.zeros(7, device="cuda"))
+    st.close()
