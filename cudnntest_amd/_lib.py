@@ -38,6 +38,7 @@ SYMBOLS = {
     "wino_conv_prepared": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp]),
     "wino_conv_ex": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp, _vp]),
     "wino_conv_prepared_ex": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp, _vp]),
+    "wino_conv_noalloc": (_i, [_i, _i, _i, _i, _u] + [_i] * 6 + [_vp, _vp, _vp, _vp, _vp]),
     "wino_pick_algo": (_i, [_i] * 8),
     "wino_geometry": (_i, [_i] * 7 + [ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l),
                                      ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_l)]),

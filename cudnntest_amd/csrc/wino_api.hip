@@ -18,6 +18,10 @@
 
 using namespace wino;
 
+// Scratch of wino_conv_noalloc: a fixed buffer in the library's own device image, one copy per GPU, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress (see noalloc_scratch below).
+static __device__ __align__(256) unsigned char scratch[WINO_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -111,7 +115,7 @@ int arena_get(size_t bytes, void** out) {
 }
 
 // Where a whole-layer call takes its scratch from: the device's arena (grown on demand), or a fixed buffer that
-// is never grown.
+// is never grown (the entry point that allocates nothing).
 struct ScratchSource {
     void* fixed = nullptr;
     size_t fixed_bytes = 0;
@@ -805,6 +809,40 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
 
 __global__ void warmup_kernel() {}
 
+// ---- scratch of the entry point that allocates nothing --------------------------------------------
+// The file-scope array `scratch` is laid out like the arena: arrival counters first, then U, V and the product or
+// partial sums.  Host code never uses the array's name as an address: each device's copy is looked up once
+// (noalloc_scratch) and that pointer is what kernels and the fill below receive.
+constexpr size_t kNoAllocBytes = WINO_NOALLOC_SCRATCH_BYTES;
+void* g_noalloc_ptr[kMaxDevices] = {};
+std::mutex g_noalloc_mu;
+
+__global__ void fill_zero_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// The current device's copy of `scratch`; on the first call for a device its arrival counters are cleared by a
+// kernel on `st` (a fill kernel, not a memset: the caller may be recording a graph).  Later launches leave the
+// counters at zero themselves.
+int noalloc_scratch(hipStream_t st, void** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(WINO_ERR_UNSUPPORTED, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_noalloc_mu);
+    if (!g_noalloc_ptr[dev]) {
+        void* ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr || misaligned(ptr, 256)) return fail(WINO_ERR_HIP, "built-in scratch buffer not found on device %d", dev);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(kCounterBytes / 4 / 256)), dim3(256), 0, st, (unsigned*)ptr,
+                           (int)(kCounterBytes / 4));
+        LAUNCH_CHECK("fill_zero");
+        g_noalloc_ptr[dev] = ptr;
+    }
+    *out = g_noalloc_ptr[dev];
+    return WINO_OK;
+}
+
 // How many passes over the batch a layer call makes.  The epilogue pipeline of a 2-byte layer is bound by memory
 // on both sides of V (written by the input transform, read by the GEMM); when V is much larger than the 256 MB
 // last-level cache, running the two kernels on one part of the batch after the other lets the GEMM find V still
@@ -877,6 +915,20 @@ int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags,
                           int pad, const void* x, const void* U, const void* bias, void* y, void* stream) {
     if (!U) return fail(WINO_ERR_INVALID, "null transformed-filter pointer");
     return conv_impl(ScratchSource{}, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, nullptr, U, bias, y, stream);
+}
+
+int wino_conv_noalloc(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H, int W, int pad,
+                      const void* x, const void* w, const void* bias, void* y, void* stream) {
+    if (!w) return fail(WINO_ERR_INVALID, "null filter pointer");
+    struct NoTiming {                          // stage timing creates events: not in this call
+        NoTiming() { t_no_timing = true; }
+        ~NoTiming() { t_no_timing = false; }
+    } guard;
+    ScratchSource ss;
+    const int rc = noalloc_scratch((hipStream_t)stream, &ss.fixed);
+    if (rc) return rc;
+    ss.fixed_bytes = kNoAllocBytes;
+    return conv_impl(ss, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, bias, y, stream);
 }
 
 int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int pad) {
@@ -1356,7 +1408,8 @@ int wino_stack_destroy(wino_stack_t* s) {
 int wino_warmup(void) {
     hipLaunchKernelGGL(warmup_kernel, dim3(1), dim3(1), 0, 0);
     LAUNCH_CHECK("warmup");
-    return WINO_OK;
+    void* unused = nullptr;                    // also the set-up of wino_conv_noalloc's buffer on this device
+    return noalloc_scratch(nullptr, &unused);
 }
 
 int wino_sync(void* stream) {

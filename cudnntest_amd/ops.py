@@ -167,6 +167,25 @@ def conv(x, w, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None, 
     return out
 
 
+def conv_noalloc(x, w, out, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, bias=None, pool=False):
+    """conv() into the caller's `out` through wino_conv_noalloc: the library's scratch is its built-in fixed buffer,
+    nothing is allocated (not here either: `out` is required).  Problems that need more scratch are refused."""
+    dst = src if dst is None else dst
+    N, C, H, W = act_dims(src, x)
+    K, C2 = flt_dims(src, w)
+    if C2 != C:
+        raise ValueError(f"filter bank has {C2} channels, input has {C}")
+    if w.dtype != x.dtype:
+        raise TypeError("x and w must share a dtype")
+    bias = _check_bias(bias, x, K)
+    out = _out_for(dst, x, N, K, H + 2 * pad - 2, W + 2 * pad - 2, pool, out)
+    flags = (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0)
+    rc = _lib.load().wino_conv_noalloc(int(src), int(dst), _dt(x), algo, flags, N, C, K, H, W, pad, _ptr(x), _ptr(w),
+                                       _ptr(bias) if bias is not None else None, _ptr(out), _stream())
+    _lib.check(rc, "wino_conv_noalloc")
+    return out
+
+
 def conv_prepared(x, U, K, pad=1, src=NCHW, dst=None, algo=ALGO_AUTO, relu=False, out=None, bias=None, pool=False):
     """Same with the filter bank already transformed by filter_transform()."""
     dst = src if dst is None else dst

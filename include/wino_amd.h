@@ -124,6 +124,24 @@ int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags,
                           int H, int W, int pad, const void *x, const void *U, const void *bias, void *y,
                           void *stream);
 
+/*
+ * wino_conv_ex for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose callers allocate their three
+ * scratch buffers themselves (comparison/layoutCompare.cu:124-126).  Same arguments, same kernels and the same
+ * bits as wino_conv_ex; the scratch (transformed operands, product or partial sums, arrival counters) is a
+ * fixed buffer of WINO_NOALLOC_SCRATCH_BYTES inside the library's device image, one per GPU, held until the
+ * process ends, instead of the arena.  The call makes no hipMalloc / hipFree and creates no events (stage timing
+ * does not see it).  A problem whose pipeline needs more scratch than the buffer holds is refused with
+ * WINO_ERR_WORKSPACE and a message giving both sizes: ask for WINO_ALGO_FUSED (keeps only the transformed
+ * filters, 16*Cp*Kp elements) or WINO_ALGO_DIRECT, or use a smaller batch.  The first call on a device looks the
+ * buffer up and clears its counters with a small kernel on `stream`; wino_warmup() does the same ahead of time
+ * (do one of the two before recording a graph).  Every call on a GPU shares that GPU's buffer: calls that overlap
+ * on one GPU (two streams, two threads) race, exactly as whole-layer calls sharing the arena do.
+ */
+#define WINO_NOALLOC_SCRATCH_BYTES (64u << 20)
+int wino_conv_noalloc(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
+                      int W, int pad, const void *x, const void *w, const void *bias, void *y, void *stream);
+
 /* the algorithm WINO_ALGO_AUTO resolves to for this problem (a wino_algo_t), or a negative status;
  * layout is that of the input tensor */
 int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int pad);

@@ -1,0 +1,66 @@
+"""wino_conv_noalloc -- the whole-layer call whose scratch is a fixed buffer inside the library's device image --
+against wino_conv_ex, the entry point it is a variant of: the same kernels, so the same bits.  Two calls in a
+row, the second on a smaller input (the buffer keeps the first call's contents; what must start at zero is the
+arrival counters, which the kernels leave at zero), for every pipeline that uses scratch; a problem beyond the
+buffer is refused with the workspace status and nothing is launched."""
+import numpy as np
+import pytest
+import torch
+
+from cudnntest_amd import _lib, ops, synth
+from gpu_util import TORCH_DT, dev, host
+
+pytestmark = pytest.mark.gpu
+LIMIT = 64 << 20          # WINO_NOALLOC_SCRATCH_BYTES
+
+
+def both(x, w, b, layout, algo, **kw):
+    want = ops.conv(x, w, 1, layout, algo=algo, bias=b, **kw)
+    got = torch.full_like(want, float("nan"))
+    ops.conv_noalloc(x, w, got, 1, layout, algo=algo, bias=b, **kw)
+    return got, want
+
+
+@pytest.mark.parametrize("algo", [ops.ALGO_AUTO, ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_STAGED_F4])
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.BF16])
+def test_two_calls_in_a_row_match_the_allocating_entry_point(oracle, dtype, layout, algo):
+    f4 = algo == ops.ALGO_STAGED_F4
+    # first a layer that fills a good part of the buffer, then a smaller one with other channel and filter counts
+    for (N, C, K, H) in [(4, 64, 96, 56), (1, 24, 40, 13)]:
+        x, w = synth.conv_inputs(N, C, K, H, H, seed=900 + C, layout=layout, integer=True)
+        bias = None if f4 else dev(synth.small_ints(K, seed=4, lo=-2, hi=2).astype(np.float32), dtype)
+        got, want = both(dev(x, dtype), dev(w, dtype), bias, layout, algo, relu=True)
+        assert torch.equal(got, want), (N, C, K, H)
+        if not f4 and dtype == ops.F32:     # and the oracle itself: small integers are exact in every fp32 pipeline
+            ref = oracle.direct_conv(x, w, 1, layout)
+            ref = synth.act_from_layout(ref, layout) + host(bias)[None, :, None, None]
+            ref = synth.act_to_layout(np.ascontiguousarray(np.maximum(ref, 0).astype(np.float32)), layout)
+            assert np.array_equal(host(got), ref)
+
+
+def test_cut_up_rounds_share_the_counters_from_call_to_call():
+    """fp32 epilogue GEMM with a small last round (N=65: 520 patches on 512 places): the cut-up patches use the
+    arrival counters and the partial-sum region of the buffer; three calls in a row, then a smaller problem."""
+    C, K, H, W = 8, 64, 32, 64
+    for N in (65, 65, 65, 3):
+        x, w = synth.conv_inputs(N, C, K, H, W, seed=70 + N)
+        got, want = both(dev(x), dev(w), None, ops.NCHW, ops.ALGO_EPILOGUE)
+        assert torch.equal(got, want), N
+
+
+def test_a_problem_beyond_the_buffer_is_refused():
+    N, C, K, H = 8, 64, 64, 112          # V alone: 16 * 25088 * 64 * 4 bytes = 103 MB
+    x = torch.zeros((N, C, H, H), device="cuda")
+    w = torch.zeros((K, C, 3, 3), device="cuda")
+    out = torch.full((N, K, H, H), 7.0, device="cuda")
+    with pytest.raises(_lib.WinoError) as e:
+        ops.conv_noalloc(x, w, out, algo=ops.ALGO_EPILOGUE)
+    assert e.value.code == -4 and str(LIMIT) in str(e.value)
+    torch.cuda.synchronize()
+    assert bool((out == 7.0).all())      # nothing ran
+    # the single-kernel pipeline keeps only the transformed filters and fits
+    x.uniform_(-1, 1)
+    w.normal_(0, 0.05)
+    ops.conv_noalloc(x, w, out, algo=ops.ALGO_FUSED)
+    assert torch.equal(out, ops.conv(x, w, algo=ops.ALGO_FUSED))
