@@ -14,21 +14,29 @@ Before the W warm-up steps the step runs untimed for --ramp-ms (200 ms): the GPU
 tens of milliseconds of load to reach its working frequency, and W steps of a 0.5 ms layer do not give it that.
 
 Prints ONE JSON line:
-  value        effective TFLOP/s = direct-convolution FLOPs (2*N*K*C*H*W*9) / time
-  ms_per_step  ms per layer (per 13-layer pass for vgg16_all13)
+  ms_per_step  the MEDIAN of the K steps' own durations (an event on the launch stream after every step), ms per layer
+               (per 13-layer pass for vgg16_all13); ms_per_step_wall_mean is host wall time over the same K steps / K
+  value        effective TFLOP/s = direct-convolution FLOPs (2*N*K*C*H*W*9) / ms_per_step
   roofline     the dominant kernel -- the batched GEMM, or the kernel that contains it -- timed with
                HIP events recorded by the library on the launch stream, against the dense MFMA peak;
-               algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4); single-layer runs add
-               the kernel's algorithmic bytes, flop/byte, min(MFMA peak, flop/byte x 8 TB/s) and its fraction of 8 TB/s
+               algorithmic flops per launch = 2*16*P*K*C (2*36*P*K*C with --algo staged_f4, the direct-convolution count
+               for the direct kernels); single-layer runs add the kernel's algorithmic bytes, flop/byte,
+               min(MFMA peak, flop/byte x 8 TB/s) and its fraction of 8 TB/s; traffic = HBM bytes per launch
+               measured with rocprofv3 --pmc (traffic_source names the summary under profiles/), null where
+               no such run is committed
   cpu_baseline the oracle's fp32 OpenMP direct convolution on this host's cores (reported, not a target)
   stages       per-stage ms and achieved GB/s (algorithmic bytes) or TFLOP/s
   ms_per_step_filters_prepared   the same K steps with the filter bank transformed beforehand (single-layer runs)
   layout_transforms   the stand-alone permutations of the layer's input between its layout and the other two
                (wino_layout_transform; bytes = read + write), timed apart from the convolution
+  configs      (default workload only, after its timed region) the other benchmark configurations, a few steps
+               each: ms (median), effective TFLOP/s, the dominant kernel with its fraction of the MFMA peak and of
+               min(MFMA peak, flop/byte x 8 TB/s); for the 13-layer f16 / bf16 passes also per layer
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -56,16 +64,30 @@ WORKLOADS = {
     "ref_H22_C128_K128_N128": [(128, 128, 128, 22)],
 }
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (summaries and the copy-kernel scale factor under profiles/), keyed by
-# (workload, layout, dtype, resolved algo).
+# script (the summary file holds the counters and the copy-kernel scale factor), keyed by
+# (workload, layout, dtype, resolved algo): (bytes, summary under profiles/).
 MEASURED_TRAFFIC = {
-    # profiles/epilogue_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 596.1 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
-    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"): 707.3e6,
-    # profiles/staged_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt: 449.1 MB fetched + 411.0 MB written
-    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"): 860.1e6,
-    # profiles/fused_fp32_nchw_vgg16_conv1_2_N32_hbm_traffic.txt: 596.4 MB fetched + 411.0 MB written
-    ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"): 1007.4e6,
+    # 596.1 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"):
+        (707.3e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt"),
+    # 449.1 MB fetched + 411.0 MB written
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"):
+        (860.1e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt"),
+    # 596.4 MB fetched + 411.0 MB written
+    ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"):
+        (1007.4e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_hbm_traffic.txt"),
 }
+# what the default run also times, after the headline's timed region: (name, workload, dtype)
+OTHER_CONFIGS = [
+    ("cfg1_N1_C64_K64_H56_f32", "cfg1_N1_C64_K64_H56", "f32"),
+    ("cfg3a_N64_C512_K512_H28_f32", "vgg16_conv4_N64_C512_K512_H28", "f32"),
+    ("cfg3b_N64_C512_K512_H14_f32", "vgg16_conv5_N64_C512_K512_H14", "f32"),
+    ("cfg4_N32_C64_K64_H224_f32", "vgg16_conv1_2_N32_C64_K64_H224", "f32"),
+    ("cfg5_vgg16_all13_N32_f16", "vgg16_all13", "f16"),
+    ("cfg5_vgg16_all13_N32_bf16", "vgg16_all13", "bf16"),
+]
+KERNEL_OF = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
+             "staged_f4": "gemm_128x128_kernel", "direct": "direct conv kernel"}
 
 
 def main():
@@ -84,6 +106,8 @@ def main():
                     help="untimed steps before the warm-up, for this long: the shader clock needs tens of ms of "
                          "sustained load to leave its idle level (2.1 -> 2.4 GHz measured), more than W short steps give")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default workload: skip the `configs` object (the other benchmark configurations)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain copy kernel of the first layer's input (known size) three times, so a "
                          "rocprofv3 --pmc run of this script can scale FETCH_SIZE / WRITE_SIZE")
@@ -106,13 +130,126 @@ def main():
     if args.graph and args.workload != "vgg16_stack":
         print("bench.py: --graph applies to --workload vgg16_stack", file=sys.stderr)
         sys.exit(2)
-    layers = WORKLOADS[args.workload] or [(args.batch, C, K, H) for (C, K, H) in synth.VGG16_CONV]   # (N, C, K, H)
+    LAYOUT = {"NCHW": ops.NCHW, "NHWC": ops.NHWC, "CHWN": ops.CHWN}
+    TDT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+    DT = {"f32": ops.F32, "f16": ops.F16, "bf16": ops.BF16}
+    ALGO = {"auto": ops.ALGO_AUTO, "staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE,
+            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4, "direct": ops.ALGO_DIRECT}
+
+    def layers_of(workload):
+        return WORKLOADS[workload] or [(args.batch, C, K, H) for (C, K, H) in synth.VGG16_CONV]   # (N, C, K, H)
+
+    def timed(step, steps, warmup, group=1):
+        """(median ms per step, wall-clock mean ms per step) of exactly `steps` steps after `warmup`.  An event is
+        recorded on the launch stream after every `group` steps and the median is taken over those spans (group > 1
+        for steps of a few tens of microseconds, where an event between two launches would be part of what is timed)."""
+        for _ in range(warmup):
+            step()
+        spans = steps // group
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(spans + 1)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev[0].record()
+        for i in range(spans):
+            for _ in range(group):
+                step()
+            ev[i + 1].record()
+        for _ in range(steps - spans * group):
+            step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        per = [ev[i].elapsed_time(ev[i + 1]) / group for i in range(spans)]
+        return statistics.median(per), (t1 - t0) * 1e3 / steps
+
+    def staged_pass(step, steps):
+        """per-stage (sum, min, max, spans) of `steps` more steps, the library bracketing every stage with events"""
+        ops.stage_timing(True)
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        st = ops.stage_stats()
+        ops.stage_timing(False)
+        return st
+
+    def kernel_roofline(layout, dtype, a, N, C, K, H, gemm_ms):
+        """the dominant kernel of one layer against both roofs"""
+        dt, es, peak = DT[dtype], (4 if dtype == "f32" else 2), MFMA_PEAK_TFLOPS[dtype]
+        name = ops.ALGO_NAMES[a]
+        f4 = a == ops.ALGO_STAGED_F4
+        g = ops.f4_geometry(dt, N, C, K, H, H, 1) if f4 else ops.geometry(dt, N, C, K, H, H, 1)
+        P, nxi = g["P"], (36 if f4 else 16)
+        xb, yb = N * C * H * H * es, N * K * H * H * es
+        flops = 2.0 * N * K * C * H * H * 9 if a == ops.ALGO_DIRECT else 2.0 * nxi * P * K * C
+        kb = {"staged": nxi * P * C * es + nxi * K * C * es + nxi * P * K * 4,
+              "staged_f4": nxi * P * C * es + nxi * K * C * es + nxi * P * K * 4,
+              "epilogue": 16 * P * C * es + 16 * K * C * es + yb,
+              "fused": xb + 16 * K * C * es + yb,
+              "direct": xb + 9 * K * C * es + yb}[name]
+        ai = flops / kb
+        attainable = min(peak, ai * HBM_PEAK_GBS / 1e3)
+        achieved = flops / (gemm_ms * 1e-3) / 1e12
+        return {"algo": name, "kernel": KERNEL_OF[name], "kernel_ms": round(gemm_ms, 4), "flops": flops,
+                "algorithmic_bytes": kb, "flop_per_byte": round(ai, 1), "achieved_tflops": round(achieved, 2),
+                "frac_mfma": round(achieved / peak, 4), "attainable_tflops": round(attainable, 1),
+                "frac_of_attainable": round(achieved / attainable, 4),
+                "bound": "mfma" if attainable >= peak else "hbm",
+                "GBps": round(kb / (gemm_ms * 1e-3) / 1e9, 1)}
+
+    def device_tensors(layers, layout, dtype, seed):
+        """x, w, y of every layer, generated on the device (seeded): uniform[-1, 1) activations, N(0, sqrt(2/(9C))) filters"""
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        out = []
+        for (N, C, K, H) in layers:
+            x = (torch.rand(ops.act_shape(layout, N, C, H, H), device="cuda", generator=g) * 2 - 1).to(TDT[dtype])
+            wshape = {ops.NCHW: (K, C, 3, 3), ops.NHWC: (K, 3, 3, C), ops.CHWN: (C, 3, 3, K)}[layout]
+            w = (torch.randn(wshape, device="cuda", generator=g) * (2.0 / (9 * C)) ** 0.5).to(TDT[dtype])
+            y = torch.empty(ops.act_shape(layout, N, K, H, H), dtype=TDT[dtype], device="cuda")
+            out.append((x, w, y))
+        return out
+
+    def other_config(workload, dtype):
+        """one of the other benchmark configurations, NCHW, the automatic choice of pipeline: a few steps"""
+        layout, layers = ops.NCHW, layers_of(workload)
+        many = len(layers) > 1
+        tens = device_tensors(layers, layout, dtype, 0xBE7C)
+
+        def run(sel):
+            for (x, w, y) in sel:
+                ops.conv(x, w, 1, layout, relu=many, out=y)
+        tiny = layers[0][0] == 1                      # N = 1: a step is a few tens of microseconds
+        steps = 20 if many else (200 if tiny else 30)
+        ms, wall = timed(lambda: run(tens), steps, 5, group=10 if tiny else 1)
+        flops = sum(2.0 * N * K * C * H * H * 9 for (N, C, K, H) in layers)
+        res = {"ms": round(ms, 4), "ms_wall_mean": round(wall, 4), "steps": steps,
+               "effective_tflops": round(flops / (ms * 1e-3) / 1e12, 2), "dtype": dtype, "layout": "NCHW"}
+        per_layer, k_flops, k_ms = [], 0.0, 0.0
+        for (N, C, K, H), t in zip(layers, tens):
+            a = ops.pick_algo(layout, DT[dtype], N, C, K, H, H)
+            st = staged_pass(lambda: run([t]), 10)
+            r = kernel_roofline("NCHW", dtype, a, N, C, K, H, st["gemm"][0] / 10)
+            k_flops += r["flops"]
+            k_ms += r["kernel_ms"]
+            if many:
+                lms, _ = timed(lambda: run([t]), 10, 2)
+                per_layer.append({"C": C, "K": K, "H": H, "ms": round(lms, 4),
+                                  "input_ms": round(st["input"][0] / 10, 4), **{k: r[k] for k in (
+                                      "algo", "kernel_ms", "flop_per_byte", "achieved_tflops", "attainable_tflops",
+                                      "frac_of_attainable", "bound")}})
+            else:
+                res.update(algo=r["algo"], kernel=r["kernel"], kernel_ms=r["kernel_ms"], frac=r["frac_mfma"],
+                           attainable_tflops=r["attainable_tflops"], frac_of_attainable=r["frac_of_attainable"],
+                           bound=r["bound"])
+        if many:
+            ach = k_flops / (k_ms * 1e-3) / 1e12
+            res.update(kernel="per-layer choice", kernel_ms=round(k_ms, 4), frac=round(ach / MFMA_PEAK_TFLOPS[dtype], 4),
+                       bound="per layer", layers=per_layer)
+        del tens
+        torch.cuda.empty_cache()
+        return res
+
+    layers = layers_of(args.workload)
     multi = len(layers) > 1
-    layout = {"NCHW": ops.NCHW, "NHWC": ops.NHWC, "CHWN": ops.CHWN}[args.layout]
-    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
-    dt = {"f32": ops.F32, "f16": ops.F16, "bf16": ops.BF16}[args.dtype]
-    algo = {"auto": ops.ALGO_AUTO, "staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE,
-            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4, "direct": ops.ALGO_DIRECT}[args.algo]
+    layout, tdt, dt, algo = LAYOUT[args.layout], TDT[args.dtype], DT[args.dtype], ALGO[args.algo]
     es = 4 if args.dtype == "f32" else 2
 
     stack = None
@@ -158,27 +295,14 @@ def main():
         for _ in range(10):
             step()
         torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
 
-    # ---- timed region: exactly K steps -------------------------------------------------
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    # ---- timed region: exactly K steps after W warm-up steps ----------------------------
+    ms_per_step, ms_wall = timed(step, args.steps, args.warmup)
     direct_flops = sum(2.0 * N * K * C * H * H * 9 for (N, C, K, H) in layers)
     value = direct_flops / (ms_per_step * 1e-3) / 1e12
 
     # ---- the same K steps again, the library bracketing every stage with HIP events --------
-    ops.stage_timing(True)
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    st = ops.stage_stats()
-    ops.stage_timing(False)
+    st = staged_pass(step, args.steps)
 
     per_step = {k: (v[0] / args.steps) for k, v in st.items()}        # ms per step, summed over layers
     gemm_flops = alg_in = alg_out = alg_flt = 0.0
@@ -214,40 +338,31 @@ def main():
     stages["gemm"] = {"ms": round(gemm_ms, 4), "TFLOPs": round(achieved, 2)}
     if not multi:
         stages["gemm"].update(min_ms=round(st["gemm"][1], 4), max_ms=round(st["gemm"][2], 4))
-    kernel = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
-              "staged_f4": "gemm_128x128_kernel",
-              "direct": "direct_small_c_kernel" if args.dtype == "f32" else "direct_small_c16_kernel"}
     algo_label = resolved[0] if len(set(resolved)) == 1 else "mixed"
-    traffic = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label))
-    roofline = {"bound": "mfma", "kernel": kernel.get(algo_label, "per-layer choice"),
+    traffic, traffic_source = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label), (None, None))
+    roofline = {"bound": "mfma", "kernel": KERNEL_OF.get(algo_label, "per-layer choice"),
                 "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": traffic,
+                "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
                 "flops_per_launch": gemm_flops if not multi else None}
 
     N0, C0, K0, H0 = layers[0]
     if not multi:
         # the dominant kernel's algorithmic bytes, its arithmetic intensity, and what the two roofs allow together
-        Pn = ops.geometry(dt, N0, C0, K0, H0, H0, 1)["P"]
-        xb, yb = N0 * C0 * H0 * H0 * es, N0 * K0 * H0 * H0 * es
-        kb = {"staged": 16 * Pn * C0 * es + 16 * K0 * C0 * es + 16 * Pn * K0 * 4,
-              "epilogue": 16 * Pn * C0 * es + 16 * K0 * C0 * es + yb,
-              "fused": xb + 16 * K0 * C0 * es + yb,
-              "direct": xb + 9 * K0 * C0 * es + yb}.get(algo_label)
-        if kb:
-            ai = gemm_flops / kb
-            gbs = kb / (gemm_ms * 1e-3) / 1e9
-            roofline.update(algorithmic_bytes=kb, flop_per_byte=round(ai, 1),
-                            attainable=round(min(peak, ai * HBM_PEAK_GBS / 1e3), 1),
-                            frac_hbm=round(gbs / HBM_PEAK_GBS, 3))
-            if ai * HBM_PEAK_GBS / 1e3 < peak:
-                # the memory roof is the lower one for this kernel and type: it is the bound that is reported
-                roofline.update(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                                frac=round(gbs / HBM_PEAK_GBS, 4), mfma_achieved=round(achieved, 2),
-                                mfma_frac=round(achieved / peak, 4))
+        r = kernel_roofline(args.layout, args.dtype, ops.pick_algo(layout, dt, N0, C0, K0, H0, H0)
+                            if algo == ops.ALGO_AUTO else algo, N0, C0, K0, H0, gemm_ms)
+        roofline.update(algorithmic_bytes=r["algorithmic_bytes"], flop_per_byte=r["flop_per_byte"],
+                        attainable=r["attainable_tflops"], frac_of_attainable=r["frac_of_attainable"],
+                        frac_hbm=round(r["GBps"] / HBM_PEAK_GBS, 3))
+        if r["bound"] == "hbm":
+            # the memory roof is the lower one for this kernel and type: it is the bound that is reported
+            roofline.update(bound="hbm", achieved=r["GBps"], peak=HBM_PEAK_GBS, unit="GB/s",
+                            frac=round(r["GBps"] / HBM_PEAK_GBS, 4), mfma_achieved=round(achieved, 2),
+                            mfma_frac=round(achieved / peak, 4))
     out = {
         "metric": "effective TFLOP/s (direct-conv FLOPs), VGG-16 3x3 layer, N=32",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_wall_mean": round(ms_wall, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": args.workload, "layers": len(layers), "N": N0, "C": C0, "K": K0, "H": H0, "W": H0,
                    "pad": 1, "layout": args.layout, "algo": args.algo, "resolved_algo": resolved,
@@ -263,14 +378,8 @@ def main():
         x0, w0, y0 = tensors[0]
         U0 = ops.filter_transform(w0, layout)
         a0 = {"staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE, "fused": ops.ALGO_FUSED}[resolved[0]]
-        for _ in range(args.warmup):
-            ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0)
-        torch.cuda.synchronize()
-        tp = time.perf_counter()
-        for _ in range(args.steps):
-            ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0)
-        torch.cuda.synchronize()
-        out["ms_per_step_filters_prepared"] = round((time.perf_counter() - tp) * 1e3 / args.steps, 4)
+        out["ms_per_step_filters_prepared"] = round(
+            timed(lambda: ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0), args.steps, args.warmup)[0], 4)
 
     # ---- the stand-alone layout permutations of the layer's input, timed separately ------------
     if not multi and stack is None:
@@ -282,20 +391,20 @@ def main():
                 continue
             x1 = ops.layout_transform(x0, layout, dst_l)
             for (a, la, lb) in ((x0, layout, dst_l), (x1, dst_l, layout)):
-                for _ in range(3):
-                    ops.layout_transform(a, la, lb)
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(20):
-                    ops.layout_transform(a, la, lb)
-                e1.record()
-                torch.cuda.synchronize()
-                ms = e0.elapsed_time(e1) / 20
+                ms, _ = timed(lambda: ops.layout_transform(a, la, lb), 100, 3, group=20)
                 gbs = 2.0 * x0.numel() * es / (ms * 1e-3) / 1e9
                 perms[f"{names[la]}->{names[lb]}"] = {"ms": round(ms, 4), "GBps": round(gbs, 1),
                                                       "frac_hbm": round(gbs / HBM_PEAK_GBS, 3)}
             del x1
         out["layout_transforms"] = perms
+
+    # ---- the other benchmark configurations (default run only) ----------------------------------
+    default_run = (args.workload == "vgg16_conv3_N32_C256_K256_H56" and args.layout == "NCHW" and args.dtype == "f32"
+                   and args.algo == "auto")
+    if default_run and not args.no_other_configs:
+        del tensors
+        torch.cuda.empty_cache()
+        out["configs"] = {name: other_config(wl, dty) for (name, wl, dty) in OTHER_CONFIGS}
 
     if not args.no_cpu_baseline:
         import oracle
