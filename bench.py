@@ -99,6 +99,8 @@ def main():
     ap.add_argument("--layout", default="NCHW", choices=["NCHW", "NHWC", "CHWN"])
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
     ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4", "direct"])
+    ap.add_argument("--shape", default=None, metavar="N,C,K,H",
+                    help="a single layer of this shape instead of a named workload (kernel experiments)")
     ap.add_argument("--batch", type=int, default=32, help="N of the vgg16_all13 / vgg16_stack workloads")
     ap.add_argument("--graph", action="store_true",
                     help="vgg16_stack: replay the pass from a HIP graph (one submission instead of ~30 launches)")
@@ -135,6 +137,10 @@ def main():
     DT = {"f32": ops.F32, "f16": ops.F16, "bf16": ops.BF16}
     ALGO = {"auto": ops.ALGO_AUTO, "staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE,
             "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4, "direct": ops.ALGO_DIRECT}
+
+    if args.shape:
+        WORKLOADS["custom"] = [tuple(int(v) for v in args.shape.split(","))]
+        args.workload = "custom"
 
     def layers_of(workload):
         return WORKLOADS[workload] or [(args.batch, C, K, H) for (C, K, H) in synth.VGG16_CONV]   # (N, C, K, H)

@@ -12,6 +12,7 @@
 #include "common.hpp"
 #include "fused.hpp"
 #include "direct.hpp"
+#include "direct16.hpp"
 #include "gemm.hpp"
 #include "transforms.hpp"
 #include "transforms_f4.hpp"
@@ -650,6 +651,100 @@ int launch_direct(int src, int dst, int dtype, unsigned flags, const void* bias,
     DISPATCH_DTYPE(dtype, launch_direct_t<T>(src, dst, flags, bias, g, x, w, y, st));
 }
 
+// ---- direct convolution of 2-byte NCHW tensors on the 16-bit matrix instruction (direct16.hpp) ----------------
+// Block shape for a layer: BC columns (even, at most 32: the one that wastes the fewest lanes on the image's width,
+// the widest among equals), BR = pixels per workgroup / BC rows, shrunk until the block's input rows fit a buffer
+// (LR * PW <= D16_PLANE pixel slots) and its load tasks fit three rounds of the 256 threads.
+// rows: blocks of 16 rows x 32 columns whose waves own 4 consecutive rows of one image (Ho a multiple of 4).
+bool direct16_plan(const Geometry& g, int npg, bool rows, D16Geom* d) {
+    const int PB = 128 * npg;
+    int BC = 0;
+    long best = 0;
+    for (int bc = 32; bc >= 8; bc -= 2) {
+        const long padded = (long)((g.Wo + bc - 1) / bc) * bc;
+        if (BC == 0 || padded < best) { BC = bc; best = padded; }
+    }
+    const long G = (long)g.N * g.Ho;
+    if (rows) {
+        if (npg != 4 || g.Ho % 4 != 0 || G < 16) return false;
+        BC = 32;
+    }
+    int BR = (int)std::min<long>(PB / BC, G);
+    auto lr_of = [&](int br) { return br + 2 + 2 * ((g.Ho + br - 2) / g.Ho); };
+    const int PW = BC + 2, PP = BC / 2 + 1 + g.pad;
+    if (!rows)
+        while (BR > 1 && (lr_of(BR) * PW > D16_PLANE || 2 * lr_of(BR) * PP > 768)) --BR;
+    if (lr_of(BR) * PW > D16_PLANE || 2 * lr_of(BR) * PP > 768) return false;
+    d->N = g.N; d->C = g.C; d->K = g.K; d->H = g.H; d->W = g.W; d->pad = g.pad; d->Ho = g.Ho; d->Wo = g.Wo;
+    d->BR = BR; d->BC = BC; d->PW = PW; d->LR = lr_of(BR); d->PP = PP;
+    d->colBlocks = (g.Wo + BC - 1) / BC;
+    d->rowBlocks = (int)((G + BR - 1) / BR);
+    d->maxcross = (g.Ho + BR - 2) / g.Ho;
+    d->kTiles = (g.K + D16_KT - 1) / D16_KT;
+    d->CQ = (int)round_up(g.C, 32) / 8;
+    d->Kp = (int)round_up(g.K, D16_KT);
+    d->G = G;
+    return true;
+}
+
+size_t direct16_bank_bytes(const Geometry& g) { return (size_t)9 * round_up(g.C, 32) * round_up(g.K, D16_KT) * 2; }
+
+bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
+    D16Geom d;
+    return dtype != WINO_F32 && src == WINO_NCHW && dst == WINO_NCHW && g.C % 8 == 0 && g.W % 2 == 0 &&
+           !(flags & WINO_FLAG_POOL2) && (long)g.N * g.K * g.Ho * g.Wo < (1L << 31) &&
+           (long)g.C * g.H * g.W * 2 * 8 < (1L << 32) && direct16_plan(g, 4, false, &d);
+}
+
+template <typename T, int NPG, bool ROWS>
+int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
+    static bool attr_set = false;                // (per instantiation; the attribute is a property of the kernel)
+    if (!attr_set) {
+        HIP_TRY(hipFuncSetAttribute((const void*)direct16_kernel<T, NPG, ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    2 * D16_BUF));
+        attr_set = true;
+    }
+    // persistent grid: two workgroups per CU (or as many as there are tiles), a multiple of the 8 XCDs
+    const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
+    if ((long)d.rowBlocks * d.colBlocks >= (1L << 28)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: too many pixel blocks");
+    const long blocks = std::min<long>(2L * device_cus(), (tiles + 7) / 8 * 8) / 8 * 8;
+    hipLaunchKernelGGL((direct16_kernel<T, NPG, ROWS>), dim3((unsigned)std::max<long>(blocks, 8)), dim3(256), 2 * D16_BUF, st,
+                       (const T*)x, (const T*)W9, (T*)y, d, ep);
+    LAUNCH_CHECK("direct16");
+    return WINO_OK;
+}
+
+// W9: room for direct16_bank_bytes(g), 16-byte aligned
+int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
+                    void* W9, void* y, hipStream_t st) {
+    if (misaligned(x, 4)) return fail(WINO_ERR_UNSUPPORTED, "the 16-bit direct path loads column pairs: x must be 4-byte aligned");
+    D16Geom d;
+    // pixels per tile: 512, fewer when that leaves the chip short of tiles; blocks of whole rows when the layer allows
+    int npg = 4;
+    const bool rows = direct16_plan(g, 4, true, &d) &&
+                      (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
+    if (!rows) {
+        for (; npg > 1; npg >>= 1) {
+            if (!direct16_plan(g, npg, false, &d)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: no block shape for this layer");
+            if ((long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus()) break;
+        }
+        if (!direct16_plan(g, npg, false, &d)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: no block shape for this layer");
+    }
+    const Epilogue ep = make_epilogue(flags, bias);
+    const FltStrides fs = flt_strides(WINO_NCHW, g.K, g.C);
+    dim3 pgrid((d.Kp + 255) / 256, d.CQ);
+#define D16_GO(T)                                                                                                  \
+    hipLaunchKernelGGL(direct16_pack_kernel<T>, pgrid, dim3(256), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
+    LAUNCH_CHECK("direct16_pack");                                                                                 \
+    if (rows) return launch_direct16_t<T, 4, true>(d, ep, x, W9, y, st);                                           \
+    if (npg == 4) return launch_direct16_t<T, 4, false>(d, ep, x, W9, y, st);                                      \
+    if (npg == 2) return launch_direct16_t<T, 2, false>(d, ep, x, W9, y, st);                                      \
+    return launch_direct16_t<T, 1, false>(d, ep, x, W9, y, st)
+    if (dtype == WINO_F16) { D16_GO(f16_t); }
+    D16_GO(bf16_t);
+#undef D16_GO
+}
+
 int pick_algo(int layout, int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
     const bool nhwc = layout == WINO_NHWC;
@@ -688,6 +783,22 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
         return WINO_ALGO_FUSED;
     }
     return WINO_ALGO_EPILOGUE;
+}
+
+// Where AUTO leaves the Winograd kernels: layers with C <= 4 (direct.hpp), and 2-byte NCHW layers with large images
+// and enough tiles for the whole chip (direct16.hpp; measured on the VGG-16 shapes at N = 32 in bf16: 222 against
+// 373 us at C = K = 64, H = 224; 150 against 245 us at C = K = 128, H = 112; 148 against 164 us at C = K = 256, H = 56;
+// from 28 x 28 down the Winograd pipelines are faster).  x: the input tensor if known (its alignment decides).
+bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x) {
+    if (!direct16_ok(src, dst, dtype, flags, g) || misaligned(x, 4)) return false;
+    if (g.Ho < 48 || g.Wo < 48) return false;
+    const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
+    return tiles >= 2L * device_cus();
+}
+int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, bool have_w) {
+    if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
+    if (have_w && auto_direct16(src, dst, dtype, flags, g, x)) return WINO_ALGO_DIRECT;
+    return pick_algo(src, dtype, g);
 }
 
 int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned flags, int N, int C, int K, int H, int W,
@@ -743,13 +854,21 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     if (flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)) return fail(WINO_ERR_INVALID, "unknown flags 0x%x", flags);
     if ((flags & WINO_FLAG_POOL2) && (g.Ho < 2 || g.Wo < 2))
         return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", g.Ho, g.Wo);
-    if (algo == WINO_ALGO_AUTO) algo = (w && direct_ok(dst, flags, g)) ? WINO_ALGO_DIRECT : pick_algo(src, dtype, g);
+    if (algo == WINO_ALGO_AUTO) algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
     if (algo == WINO_ALGO_DIRECT) {
         if (!w) return fail(WINO_ERR_INVALID, "the direct path needs the filter bank, not its Winograd transform");
-        if (!direct_ok(dst, flags, g))
-            return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for C <= 4 without pooling");
+        if (direct_ok(dst, flags, g)) {
+            StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
+            return launch_direct(src, dst, dtype, flags, bias, g, x, w, y, (hipStream_t)stream);
+        }
+        if (!direct16_ok(src, dst, dtype, flags, g))
+            return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for C <= 4, and for 2-byte NCHW tensors with "
+                                              "C a multiple of 8 and an even width; no pooling");
+        void* base = nullptr;
+        const int rcb = ss.get(kCounterBytes + direct16_bank_bytes(g), &base);
+        if (rcb) return rcb;
         StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-        return launch_direct(src, dst, dtype, flags, bias, g, x, w, y, (hipStream_t)stream);
+        return launch_direct16(dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
     }
     if (algo == WINO_ALGO_STAGED_F4) {
         if (bias || (flags & WINO_FLAG_POOL2))
@@ -865,7 +984,7 @@ int conv_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     int passes = 1;
     if (valid_layout(src) && valid_layout(dst) && valid_dtype(dtype) && x && y && (w || Upre) &&
         make_geometry(dtype, N, C, K, H, W, pad, &g) && algo >= WINO_ALGO_AUTO && algo <= WINO_ALGO_DIRECT) {
-        if (algo == WINO_ALGO_AUTO) algo = (w && direct_ok(dst, flags, g)) ? WINO_ALGO_DIRECT : pick_algo(src, dtype, g);
+        if (algo == WINO_ALGO_AUTO) algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
         passes = batch_passes(src, dst, dtype, algo, g);
     }
     if (passes <= 1) return conv_pass(ss, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, Upre, bias, y, stream);
@@ -937,7 +1056,7 @@ int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
-    return direct_ok(layout, 0, g) ? WINO_ALGO_DIRECT : pick_algo(layout, dtype, g);
+    return resolve_auto(layout, layout, dtype, 0, g, nullptr, true);
 }
 
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp, int* Kp,
@@ -1306,7 +1425,10 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         make_geometry(dtype, N, L.C, L.K, L.H, L.W, 1, &g);
         hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
-        if (e == hipSuccess && L.C <= 4) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
+        // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte NCHW layers)
+        const bool direct16_layer = dtype != WINO_F32 && L.layout_in == WINO_NCHW && L.layout_out == WINO_NCHW &&
+                                    L.C % 8 == 0 && !(L.flags & WINO_FLAG_POOL2);
+        if (e == hipSuccess && (L.C <= 4 || direct16_layer)) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         if (e != hipSuccess) return bail(e);
     }
     for (int i = 0; i < 2 && raw->act_bytes; ++i) {

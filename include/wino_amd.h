@@ -57,11 +57,18 @@ typedef enum {
     WINO_ALGO_STAGED_F4 = 4, /* the staged pipeline in F(4x4,3x3) -- 6x6 tiles, 36 coordinates, the reference's
                                own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101).
                                Never chosen by WINO_ALGO_AUTO. */
-    WINO_ALGO_DIRECT = 5     /* no Winograd at all: the 9*C <= 36 products of an output as one short MFMA
-                               reduction, for layers with C <= 4 (the network's first layer, which the
-                               reference runs through the same wrappers: comparison/layoutCompare.cu:38-46).
-                               Bias and ReLU, no pooling; needs the filter bank itself (not
-                               wino_conv_prepared).  What WINO_ALGO_AUTO picks for such layers. */
+    WINO_ALGO_DIRECT = 5     /* no Winograd at all, the convolution itself on the matrix cores.  Two kernels:
+                               layers with C <= 4 (the network's first layer, which the reference runs through
+                               the same wrappers: comparison/layoutCompare.cu:38-46): the 9*C <= 36 products of an
+                               output as one short MFMA reduction, any layout, fp32 or 2-byte;
+                               2-byte NCHW -> NCHW layers with C a multiple of 8, an even width and a 4-byte aligned
+                               x: an implicit GEMM on the 16-bit instruction with fp32 accumulation -- with 2-byte
+                               operands the Winograd pipelines are bound by the transformed input in memory, the
+                               direct product by nothing but the multiplies (the stage it replaces is
+                               comparison/GEMM.cuh:124-253; the reference's own direct kernel in tile geometry is
+                               Conv_fuse, fusedTest/winotrans.cuh:1868).
+                               Bias and ReLU, no pooling; needs the filter bank itself (not wino_conv_prepared).
+                               What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW layers. */
 } wino_algo_t;
 
 /* order of the tile index p inside the transformed operands */

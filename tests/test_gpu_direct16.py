@@ -1,0 +1,79 @@
+"""The direct (implicit-GEMM) path for 2-byte NCHW tensors (WINO_ALGO_DIRECT with more than four channels): the
+convolution itself on the 16-bit matrix instruction with fp32 accumulation, no Winograd transform.  Oracle: the CPU
+direct convolution (layoutTest/NCHW/data/WinoTran_NCHW.py:200-228 restated).  On small integers every product and
+sum is exact in fp32, so the result must be the oracle's value rounded once to the tensor's type, bit for bit; on
+floats the layer tolerance applies (relative L2 2e-2)."""
+import numpy as np
+import pytest
+import torch
+
+from cudnntest_amd import _lib, ops, synth
+from gpu_util import TOL, TORCH_DT, dev, host, rounded
+
+pytestmark = pytest.mark.gpu
+# (N, C, K, H, W): blocks that span several images (14x14, 6x8), widths that do and do not fill a block's columns,
+# channel counts with half a stage left over (8, 24, 40), filter counts off the 64-filter tile, a single row
+SHAPES = [(2, 16, 64, 14, 14), (5, 8, 40, 6, 8), (1, 24, 130, 37, 20), (3, 40, 70, 9, 66), (2, 64, 64, 40, 34),
+          (1, 16, 8, 1, 2), (4, 32, 96, 28, 28), (2, 16, 64, 224, 224)]
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_integers_round_once(oracle, shape, dtype):
+    N, C, K, H, W = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    for pad in (1, 0):
+        if H + 2 * pad - 2 <= 0 or W + 2 * pad - 2 <= 0:
+            continue
+        want = np.maximum(oracle.direct_conv(x, w, pad) + bias[None, :, None, None], 0).astype(np.float32)
+        got = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
+        assert np.array_equal(host(got), rounded(want, dtype, oracle)), pad
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", [(2, 64, 64, 56, 56), (1, 128, 256, 28, 28), (3, 256, 64, 14, 14)])
+def test_floats_within_tolerance(oracle, shape, dtype):
+    N, C, K, H, W = shape
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=61 + sum(shape))
+    xr, wr = rounded(x, dtype, oracle), rounded(w, dtype, oracle)
+    want = oracle.direct_conv(xr, wr, 1)
+    got = ops.conv(dev(xr, dtype), dev(wr, dtype), 1, algo=ops.ALGO_DIRECT)
+    err = oracle.rel_l2(host(got), want)
+    assert err <= TOL[dtype], err
+    # only the final rounding separates it from the oracle: far inside the layer tolerance
+    assert err <= (1e-3 if dtype == ops.F16 else 5e-3), err
+    # and the Winograd pipelines agree with it within their own rounding
+    other = ops.conv(dev(xr, dtype), dev(wr, dtype), 1, algo=ops.ALGO_EPILOGUE)
+    assert oracle.rel_l2(host(other), host(got)) <= TOL[dtype]
+
+
+def test_element_aligned_views_and_what_is_refused():
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = (torch.rand((2, 16, 12, 12), device="cuda", generator=g) - 0.5).to(torch.bfloat16)
+    w = (torch.randn((64, 16, 3, 3), device="cuda", generator=g) * 0.1).to(torch.bfloat16)
+    want = ops.conv(x, w, algo=ops.ALGO_DIRECT)
+    # w, bias and y may sit at any element offset; x must be 4-byte aligned (column pairs) and is refused otherwise
+    flat = torch.empty(w.numel() + 1, dtype=w.dtype, device="cuda")
+    w1 = flat[1:].view(w.shape)
+    w1.copy_(w)
+    out = torch.empty(want.numel() + 1, dtype=want.dtype, device="cuda")[1:].view(want.shape)
+    assert torch.equal(ops.conv(x, w1, algo=ops.ALGO_DIRECT, out=out), want)
+    xf = torch.empty(x.numel() + 1, dtype=x.dtype, device="cuda")
+    x1 = xf[1:].view(x.shape)
+    x1.copy_(x)
+    with pytest.raises(_lib.WinoError) as e:
+        ops.conv(x1, w, algo=ops.ALGO_DIRECT)
+    assert e.value.code == -2
+    assert torch.equal(ops.conv(x1, w, algo=ops.ALGO_EPILOGUE), ops.conv(x, w, algo=ops.ALGO_EPILOGUE))
+    with pytest.raises(_lib.WinoError) as e:                   # pooling stays with the Winograd pipelines
+        ops.conv(x, w, algo=ops.ALGO_DIRECT, pool=True)
+    assert e.value.code == -2
+    with pytest.raises(_lib.WinoError) as e:                   # and so do the other layouts
+        ops.conv(x.permute(0, 2, 3, 1).contiguous(), w.permute(0, 2, 3, 1).contiguous(), src=ops.NHWC, algo=ops.ALGO_DIRECT)
+    assert e.value.code == -2
+    with pytest.raises(_lib.WinoError):                        # an odd width
+        ops.conv(x[:, :, :, :11].contiguous(), w, algo=ops.ALGO_DIRECT)
+    with pytest.raises(_lib.WinoError):                        # fp32 with more than four channels
+        ops.conv(x.float(), w.float(), algo=ops.ALGO_DIRECT)
