@@ -1,0 +1,398 @@
+// Direct 3x3 convolution of 2-byte NCHW tensors, the kernel for large images (see direct16.hpp for the method):
+// one workgroup of 8 waves per CU, tiles of 64*WF filters x 8/WF waves of 4 rows x 32 columns of output pixels, the
+// waves side by side until they span the image's width (then stacked).
+//
+// What binds the 4-wave kernel of direct16.hpp on large layers is the rate at which a CU draws operands from L2
+// (a wave that issues a stage's requests waits in the CU's request path for as long as the multiplies of half a
+// stage take, and the waves of a workgroup all issue at once), so this one moves fewer bytes per multiply, asks for
+// them earlier, and lets its waves take turns:
+//   * WF = 2: 128 filters share a block's input (the two filter halves are two groups of 4 waves), 59 KB per stage
+//     and CU instead of 82 KB;
+//   * the 160 KB of LDS hold a ring of THREE filter stages and two input stages: the filter rows of stage s+2 are
+//     requested during stage s and have a whole stage to arrive, and so has the input of stage s+2, which waits in
+//     registers until it is written to LDS during stage s+1;
+//   * every wave owns 4 consecutive output rows of one image (the host offers the kernel when Ho is a multiple of
+//     4), so pixel group j, filter row r reads input row j + r of the wave's six: a pixel fragment is fetched once
+//     and multiplied into up to three groups (18 pixel fragments per stage instead of 36);
+//   * a wave does everything that is not a multiply (LDS writes of the input it holds, its requests) in one go,
+//     once per stage, at one of four points of the stage that differs between the two waves of a SIMD: the other
+//     wave multiplies meanwhile, and only two waves of the CU issue requests at a time;
+//   * a block spans the image's width where 8/WF waves of 32 columns can (W <= 256 / WF): the rows a block needs are
+//     then one contiguous run of each channel plane, and a wave's request covers whole cache lines (a request that
+//     touches four 72-byte pieces of four rows costs 190 clocks of the CU's request path, a contiguous one 58).
+// Ring positions are runtime offsets (two additions per stage), so there is one stage body for all tiles.
+#pragma once
+#include "direct16.hpp"
+
+namespace wino {
+
+template <int WF> struct D16R {
+    static constexpr int KT = 64 * WF;                       // filters per tile
+    static constexpr int WP = 8 / WF;                        // waves along the rows of a block
+    static constexpr int FB = 9 * 2 * KT * 16;               // bytes of a filter stage: [tap][channel vector][KT] vectors
+    static constexpr int XPLANE = WF == 2 ? 704 : 1360;      // pixel slots per channel-vector plane (LR * PW must fit)
+    static constexpr int XB = 2 * XPLANE * 16;               // bytes of an input stage
+    static constexpr int LDS = 3 * FB + 2 * XB;
+    static constexpr int FROWS = 18 * WF;                    // 1 KB rows of a filter stage
+    static constexpr int NF = (FROWS + 7) / 8;               // filter requests per wave and stage (some rows twice)
+    static constexpr int NTASK = WF == 2 ? 2 : 3;            // input tasks per thread and stage
+};
+
+template <typename T, int WF>
+__global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restrict__ x, const T* __restrict__ W9,
+                                                               T* __restrict__ y, D16Geom g, Epilogue ep) {
+    typedef typename Mma<T>::vec vec;
+    typedef D16R<WF> P;
+    constexpr int NTASK = P::NTASK;
+    extern __shared__ __attribute__((aligned(16))) unsigned char d16r_smem[];     // [3][FB] filters, [2][XB] input
+    unsigned char* const xsm = d16r_smem + 3 * P::FB;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wf = wave / P::WP, wp = wave % P::WP;          // filter half; position in the block: g.WC waves side by side
+    const int wr = wp / g.WC, wc = wp - wr * g.WC;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int HW = g.H * g.W, Hp = g.Ho + 2;
+    const int nst = g.CQ / 2;                                // stages of 16 channels per tile
+
+    // ---- this workgroup's tiles: sequence items s = s0, s0 + sstep, ... < send of its XCD ------------------
+    const int xcd = blockIdx.x & 7;
+    const int sstep = gridDim.x >> 3;
+    const int npb = g.colBlocks * g.rowBlocks;               // pixel blocks; block pbx*8 + xcd belongs to this XCD
+    const int send = ((npb - xcd + 7) >> 3) * g.kTiles;
+    const int s0 = (int)(blockIdx.x >> 3);
+    if (s0 >= send) return;
+    struct Tile {
+        int k0, c0, n0, oh0;
+    };
+    auto decode = [&](int s) {
+        const int pbx = s / g.kTiles, kt = s - pbx * g.kTiles;
+        const int pb = pbx * 8 + xcd;
+        const int rb = pb / g.colBlocks, cb = pb - rb * g.colBlocks;
+        const long g0 = (long)rb * g.BR;
+        const int n0 = (int)(g0 / g.Ho);
+        return Tile{kt * P::KT, cb * g.BC, n0, (int)(g0 - (long)n0 * g.Ho)};
+    };
+
+    // ---- input tasks of this thread: (channel vector v, LDS row, column pair); what does not depend on the tile ----
+    const int ntask = 2 * g.LR * g.PP;
+    int tpk[NTASK];                                          // LDS row | (first column of the pair relative to c0, + 8) << 8 | v << 20
+    int ldsw[NTASK];                                         // byte offset of the pair's first slot inside an input stage (a multiple of
+                                                             // 16, -16 for the pair left of a row) | bit 0 / 1: slot 0 / 1 exists;
+                                                             // neither: no task
+#pragma unroll
+    for (int q = 0; q < NTASK; ++q) {
+        const int t = tid + 512 * q;
+        const int m = t % g.PP, rr = t / g.PP;
+        const int lr = rr % g.LR, v = min(rr / g.LR, 1);
+        const int slot0 = 2 * m - g.pad;                     // the pair (c0 + 2m - 2 pad, + 1) sits in slots (2m - pad, + 1)
+        tpk[q] = lr | (2 * m - 2 * g.pad + 8) << 8 | v << 20;
+        const int wbits = (slot0 >= 0 && slot0 < g.PW ? 1 : 0) | (slot0 + 1 >= 0 && slot0 + 1 < g.PW ? 2 : 0);
+        ldsw[q] = t < ntask ? (((v * P::XPLANE + lr * g.PW + slot0) * 16) | wbits) : 0;
+    }
+
+    // ---- request cursors: the stage whose input is requested next, and the stage whose filters are ----------------
+    struct Cursor {
+        int s, cs;
+        bool valid;
+    };
+    auto advance = [&](Cursor& c) {
+        if (++c.cs == nst) {
+            c.cs = 0;
+            c.s += sstep;
+            c.valid = c.s < send;
+        }
+    };
+    Cursor cx{s0, 0, true}, cf{s0, 0, true};
+    unsigned xoff[NTASK];                                    // byte offset from (image n0, the stage's first channel), a multiple
+                                                             // of 4 | bit 0: the pair lies inside the image
+    const char* xs = nullptr;                                // image n0, first channel of the stage to request
+    const unsigned hw2 = (unsigned)(HW * 2);
+    auto prep_x = [&](const Tile& t) {
+#pragma unroll
+        for (int q = 0; q < NTASK; ++q) {
+            const int lr = tpk[q] & 0xFF, v = tpk[q] >> 20;
+            const int qq = t.oh0 + lr;                       // padded row index counted from image n0
+            int dn = 0;
+            for (int k = 1; k <= g.maxcross; ++k) dn += qq >= k * Hp ? 1 : 0;
+            const int ih = qq - dn * Hp - g.pad;
+            const int iw = t.c0 + ((tpk[q] >> 8) & 0xFFF) - 8;
+            const bool in = (ldsw[q] & 3) != 0 && t.n0 + dn < g.N && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+            const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 2);
+            const int dnc = min(dn, g.N - 1 - t.n0);
+            xoff[q] = ((unsigned)((dnc * g.C * g.H + ihc) * g.W + iwc) * 2u + (unsigned)v * 8u * hw2) | (in ? 1u : 0u);
+        }
+        xs = reinterpret_cast<const char*>(x) + (size_t)t.n0 * g.C * HW * 2;
+    };
+    // filter rows: request q of this wave moves row (wave + 8q) % FROWS = (tap*2 + v)*WF + half of the stage
+    const unsigned lane_off = lane * 16;
+    unsigned frow_src[P::NF];                                // byte offset of the row inside W9, relative to (k0, stage 0)
+    int frow_dst[P::NF];                                     // and inside a filter stage of LDS
+#pragma unroll
+    for (int q = 0; q < P::NF; ++q) {
+        const int r = (wave + 8 * q) % P::FROWS;
+        const int tap = r / (2 * WF), v = (r / WF) & 1, half = r % WF;
+        frow_src[q] = (unsigned)(((tap * g.CQ + v) * g.Kp + half * 64) * 16);
+        frow_dst[q] = r * 1024;
+    }
+    const char* const w9b = reinterpret_cast<const char*>(W9);
+    const unsigned fstep = (unsigned)(2 * g.Kp * 16);
+    auto f_request = [&](const Cursor& c, int slot) {        // the filter rows of stage c into ring slot `slot`
+        const int pbx = c.s / g.kTiles, kt = c.s - pbx * g.kTiles;
+        const uint64_t base = reinterpret_cast<uint64_t>(w9b) + (uint64_t)kt * P::KT * 16 + (uint64_t)c.cs * fstep;
+#pragma unroll
+        for (int q = 0; q < P::NF; ++q) dma_row(base + frow_src[q], lane_off, d16r_smem + slot * P::FB + frow_dst[q]);
+    };
+    uint32_t raw[NTASK][8];
+    unsigned poff[NTASK];
+    int req_cs = 0;                                          // the stage (inside its tile) whose input was requested last
+    // piece 8q + e of a stage's input requests: channel e of task q.  A stage's second channel vector may lie past
+    // C: the first one is loaded instead, and masked when it is written
+    auto x_piece = [&](int idx) {
+        const int q = idx >> 3, e = idx & 7;
+        if (idx == 0) req_cs = cx.cs;
+        if (e == 0) {
+            const int v = tpk[q] >> 20;
+            const bool vok = cx.cs * 16 + v * 8 < g.C;
+            poff[q] = (xoff[q] & ~3u) - (vok ? 0u : (unsigned)v * 8u * hw2);
+        }
+        raw[q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
+        poff[q] += hw2;
+    };
+    auto x_commit = [&](int xslot) {                         // the stage requested through x_piece into input slot xslot
+#pragma unroll
+        for (int q = 0; q < NTASK; ++q) {
+            if ((ldsw[q] & 3) == 0) continue;
+            const bool keep = (xoff[q] & 1u) && req_cs * 16 + (tpk[q] >> 20) * 8 < g.C;
+            const uint32_t km = keep ? 0xFFFFFFFFu : 0u;
+            uint32_t lo[4], hi[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t a = raw[q][2 * e] & km, b = raw[q][2 * e + 1] & km;
+                lo[e] = __builtin_amdgcn_perm(b, a, 0x05040100u);     // (a.lo16, b.lo16): the pair's first pixel
+                hi[e] = __builtin_amdgcn_perm(b, a, 0x07060302u);     // (a.hi16, b.hi16): its second pixel
+            }
+            unsigned char* dst = xsm + xslot * P::XB + (ldsw[q] & ~15);
+            if (ldsw[q] & 1) *reinterpret_cast<uint4*>(dst) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            if (ldsw[q] & 2) *reinterpret_cast<uint4*>(dst + 16) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        }
+    };
+
+    // ---- the tile being multiplied ------------------------------------------------------------------------------
+    int xw_off = 0;                                          // the wave's first input row, this lane's column: byte offset in an input stage
+    int yoff[4];                                             // element offset of (n, k0, oh, ow) in y per row of the wave, < 0: no pixel
+    int k0c = 0;                                             // first filter of this wave
+    auto prep_pix = [&](const Tile& t) {
+        k0c = t.k0 + wf * 64;
+        const long g0 = (long)t.n0 * g.Ho + t.oh0;
+        const int col = 32 * wc + l32;
+        const bool colok = t.c0 + col < g.Wo;
+        const int ohp = t.oh0 + 4 * wr;                      // the wave's four rows lie in one image: Ho is a multiple of 4
+        int dn = 0;
+        for (int k = 1; k <= g.maxcross; ++k) dn += ohp >= k * g.Ho ? 1 : 0;
+        const int oh = ohp - dn * g.Ho;
+        const bool rowok = g0 + 4 * wr < g.G;
+        const int L = rowok ? dn * Hp + oh - t.oh0 : 0;
+        xw_off = ((lh * P::XPLANE) + L * g.PW + (colok ? col : 0)) * 16;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            yoff[j] = (rowok && colok) ? (int)((((long)(t.n0 + dn) * g.K + k0c) * g.Ho + oh + j) * g.Wo + t.c0 + col) : -1;
+    };
+
+    floatx16 acc[2][4];
+    // ---- one stage of multiplies: 18 steps (filter column s, input row rho), each one pixel fragment and 2 to 6
+    // multiplies.  The order is pinned: the pixel fragment of step t+2 and the filter fragments that the following
+    // steps need are requested before the multiplies of step t, filter row r of the next column as soon as its last
+    // use has issued.  service() -- everything else this wave does in a stage -- runs before step 0, 5, 9 or 14.
+    auto compute = [&](int fslot, int xslot, int site, auto&& service) {
+        const unsigned char* fs = d16r_smem + fslot * P::FB + (lh * P::KT + wf * 64 + l32) * 16;
+        const unsigned char* xrow[6];                        // the wave's six input rows, this lane's column
+#pragma unroll
+        for (int r = 0; r < 6; ++r) xrow[r] = xsm + xslot * P::XB + xw_off + r * g.PW * 16;
+        vec a[3][2], b[3];
+        auto lda = [&](int r, int s) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[r][i] = *reinterpret_cast<const vec*>(fs + (3 * r + s) * (2 * P::KT * 16) + i * 512);
+        };
+        auto ldb = [&](int t) { b[t % 3] = *reinterpret_cast<const vec*>(xrow[t % 6] + (t / 6) * 16); };
+        lda(0, 0);
+        ldb(0);
+        lda(1, 0);
+        ldb(1);
+        lda(2, 0);
+        auto step = [&](int t) {
+            const int s = t / 6, rho = t % 6;
+            if (t + 2 < 18) ldb(t + 2);
+            if (rho == 4 && s < 2) lda(0, s + 1);
+            if (rho == 5 && s < 2) lda(1, s + 1);
+            if (rho == 0 && s > 0) lda(2, s);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = rho - j;
+                if (r < 0 || r > 2) continue;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) Mma<T>::run(a[r][i], b[t % 3], acc[i][j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // (four short loops: one loop of 18 steps around the service code is more than the compiler unrolls)
+        constexpr int SITE_STEP[5] = {0, 5, 9, 14, 18};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (site == k) service();
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = SITE_STEP[k]; t < SITE_STEP[k + 1]; ++t) step(t);
+        }
+    };
+
+    // ---- stores: register r of acc[i][j] is filter k0c + 32*i + 8*(r/4) + 4*lh + r%4, the lane's pixel of row j ----
+    // Offsets into y are 32-bit element offsets (the host checks the tensor size) that run along with the filter
+    // index: from one register pair to the next the filter advances by 2 or by 6.  Rows of y have an even length and
+    // y is 4-byte aligned (the host checks): two neighbouring lanes hold neighbouring columns and exchange values, so
+    // that each stores one 4-byte pair -- the even lane for filter r, the odd lane for filter r+1.
+    // K is a multiple of 64 (the host checks), so a wave's 64 filters exist or the wave has none.  The four rows of
+    // a wave exist together, so a lane stores all its values or none.
+    const unsigned kstride2 = (unsigned)(g.Ho * g.Wo) * 2u;  // bytes between the planes of two filters
+    const bool odd = lane & 1;
+    auto stores = [&]() {
+        if (k0c >= g.K || yoff[0] < 0) return;
+        // (opaque to the optimiser: called from inside the stage loop, the 64 store addresses of a tile would be
+        // loop invariants, computed ahead of the loop and kept in registers)
+        unsigned ks = kstride2;
+        asm volatile("" : "+s"(ks));
+        char* const yb = reinterpret_cast<char*>(y);
+        unsigned o[4];                                       // byte offsets: a scalar base and a 32-bit offset per store
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = ((unsigned)yoff[j] - (odd ? 1u : 0u)) * 2u + (unsigned)(4 * lh + (odd ? 1 : 0)) * ks;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r2 = 0; r2 < 16; r2 += 2) {
+                const int kk = 32 * i + 8 * (r2 >> 2) + 4 * lh + (r2 & 3);     // filter of register r2; r2 + 1: the next one
+                float b0 = 0.f, b1 = 0.f;
+                if (ep.bias) {
+                    b0 = bias_of<T>(ep, k0c + kk);
+                    b1 = bias_of<T>(ep, k0c + kk + 1);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float v0 = acc[i][j][r2] + b0, v1 = acc[i][j][r2 + 1] + b1;
+                    if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
+                    const float got = swap_lane_pairs(odd ? v0 : v1);
+                    const float lo = odd ? got : v0, hi = odd ? v1 : got;
+                    struct alignas(4) Pair { T a, b; };
+                    *reinterpret_cast<Pair*>(yb + o[j]) = Pair{from_f32<T>(lo), from_f32<T>(hi)};
+                    o[j] += ((r2 & 2) ? 6u : 2u) * ks;
+                }
+                __builtin_amdgcn_sched_barrier(0);           // one register pair at a time
+            }
+    };
+
+    // the filters of the stage after the next, into the ring slot that was read last in the previous stage
+    auto f_next = [&](int fslot) {
+        if (!cf.valid) return false;
+        f_request(cf, fslot == 0 ? 2 : fslot - 1);
+        advance(cf);
+        return true;
+    };
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+    };
+    // wait until at most `newest` of this wave's memory requests are outstanding (loads return in order, so those
+    // are the ones issued last), and for its LDS writes; then the workgroup's barrier
+    auto wait_only = [&](int newest) {
+        constexpr int NX = 8 * NTASK;
+        if (newest == 0) __builtin_amdgcn_s_waitcnt(0x0070);
+        else if (newest == P::NF) __builtin_amdgcn_s_waitcnt(0x0070 | P::NF);
+        else if (newest == NX) __builtin_amdgcn_s_waitcnt(0x0070 | (NX & 0xF) | ((NX >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0070 | ((NX + P::NF) & 0xF) | (((NX + P::NF) >> 4) << 14));
+        asm volatile("" ::: "memory");
+    };
+    auto wait_barrier = [&](int newest) {
+        wait_only(newest);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    // ---- prologue: filters of the first two stages, input of the first, requests for the second ----------------------
+    // A stage is one pass of all 8 waves over its 18 steps and one barrier.  Each wave interrupts its multiplies once
+    // per stage, at a step that differs between the two waves of a SIMD and between the SIMDs, to do everything
+    // else: write the input it requested one stage earlier to LDS (stage s+1), request its share of the input of
+    // stage s+2 and of the filters of stage s+2.  While it does, the other wave of its SIMD multiplies, and only two
+    // waves of the CU issue requests at a time (8 waves that issue together wait for each other in the CU's
+    // request path for longer than the requests take).
+    const int site = (wave + 2 * (wave >> 2)) & 3;
+    f_request(cf, 0);
+    advance(cf);
+    if (cf.valid) {
+        f_request(cf, 1);
+        advance(cf);
+    }
+    bool pending = false;                                    // a requested stage waits in registers
+    bool need_prep = true;                                   // the stage to request next opens a tile
+    auto x_request = [&]() {
+        if (need_prep) {
+            prep_x(decode(cx.s));
+            need_prep = false;
+        }
+#pragma unroll
+        for (int i = 0; i < 8 * NTASK; ++i) x_piece(i);
+        pending = true;
+        xs += (size_t)16 * HW * 2;
+        advance(cx);
+        need_prep = cx.cs == 0;
+    };
+    x_request();
+    x_commit(0);
+    pending = false;
+    if (cx.valid) x_request();
+    wait_barrier(pending ? 8 * NTASK : 0);
+
+    int fslot = 0, xslot = 0;
+    const int ntiles = (send - s0 + sstep - 1) / sstep;
+    int s = s0, cs = 0;
+    const int total = ntiles * nst;
+#pragma unroll 1
+    for (int it = 0; it < total; ++it) {
+        if (cs == 0) {
+            prep_pix(decode(s));
+            zero_acc();
+        }
+        bool xreq = false, freq = false;
+        compute(fslot, xslot, site, [&]() {
+            if (pending) {
+                x_commit(xslot ^ 1);
+                pending = false;
+            }
+            if (cx.valid) {
+                x_request();
+                xreq = true;
+            }
+            freq = f_next(fslot);
+        });
+        const int newest = (xreq ? 8 * NTASK : 0) + (freq ? P::NF : 0);
+        if (cs == nst - 1) {
+            wait_only(newest);                               // before the stores: they would count as the newest requests
+            stores();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            wait_barrier(newest);
+        }
+        fslot = fslot == 2 ? 0 : fslot + 1;
+        xslot ^= 1;
+        if (++cs == nst) {
+            cs = 0;
+            s += sstep;
+        }
+    }
+}
+
+}  // namespace wino

@@ -53,10 +53,15 @@ template <> struct Mma<bf16_t> {
 // 16-bit MFMA rates the address arithmetic of these loads, vector or scalar, costs as much as the
 // multiplies of a stage, so the kernels keep one running address per load slot instead of
 // recomputing row * pitch products.
+// The instruction is written out rather than taken from the compiler's builtin: the compiler counts the builtin
+// as an access of unknown kind, and while one is in flight (in these kernels: always) it can no longer tell in
+// which order LDS reads return, so that every wait for an LDS read becomes a wait for ALL of them -- the read
+// issued one instruction earlier included, which leaves a wave's matrix pipe idle for an LDS round trip at
+// every step.  Written out, the load is invisible to that bookkeeping: every kernel that uses it waits for its
+// rows itself (s_waitcnt vmcnt before the workgroup's barrier), which they did already.
 __device__ __forceinline__ void dma_row(uint64_t sbase, unsigned lane_off, void* lds_dst) {
-    const char* src = reinterpret_cast<const char*>(sbase) + lane_off;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                     (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+    const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(sbase) : "memory");
 }
 
 constexpr int GEMM_BM = 128, GEMM_BN = 128;

@@ -13,6 +13,7 @@
 #include "fused.hpp"
 #include "direct.hpp"
 #include "direct16.hpp"
+#include "direct16_rows.hpp"
 #include "gemm.hpp"
 #include "transforms.hpp"
 #include "transforms_f4.hpp"
@@ -687,7 +688,53 @@ bool direct16_plan(const Geometry& g, int npg, bool rows, D16Geom* d) {
     return true;
 }
 
-size_t direct16_bank_bytes(const Geometry& g) { return (size_t)9 * round_up(g.C, 32) * round_up(g.K, D16_KT) * 2; }
+// The 8-wave kernel of direct16_rows.hpp: blocks of 32/WF rows x 32 columns whose waves own 4 consecutive rows of one
+// image.  WF = 2 (128 filters per tile) when that wastes no filters, else 1.
+template <int WF>
+bool direct16_rows_plan(const Geometry& g, D16Geom* d) {
+    typedef D16R<WF> P;
+    const long G = (long)g.N * g.Ho;
+    if (g.Ho % 4 != 0 || g.K % 64 != 0 || g.Wo % 2 != 0) return false;
+    // the block's waves (4 rows x 32 columns each) side by side until they span the image, the rest stacked
+    int WC = 1;
+    while (WC < P::WP && 32 * WC < g.Wo) WC *= 2;
+    const int BR = 4 * (P::WP / WC), BC = 32 * WC;
+    if (G < BR) return false;
+    const int maxcross = g.Ho % BR == 0 ? 0 : (g.Ho + BR - 2) / g.Ho;     // images a block's rows can span beyond the first
+    const int PW = std::min(BC, (g.Wo + 1) / 2 * 2) + 2;      // slots of an LDS row: the block's columns (or the image's) + 2
+    const int LR = BR + 2 + 2 * maxcross, PP = (PW - 2) / 2 + 1 + g.pad;
+    if (LR * PW > P::XPLANE || 2 * LR * PP > P::NTASK * 512 || LR > 255 || PW > 2048) return false;
+    d->N = g.N; d->C = g.C; d->K = g.K; d->H = g.H; d->W = g.W; d->pad = g.pad; d->Ho = g.Ho; d->Wo = g.Wo;
+    d->BR = BR; d->BC = BC; d->WC = WC; d->PW = PW; d->LR = LR; d->PP = PP;
+    d->colBlocks = (g.Wo + BC - 1) / BC;
+    d->rowBlocks = (int)((G + BR - 1) / BR);
+    d->maxcross = maxcross;
+    d->kTiles = (g.K + P::KT - 1) / P::KT;
+    d->CQ = (int)round_up(g.C, 16) / 8;
+    d->Kp = (int)round_up(g.K, P::KT);
+    d->G = G;
+    return (long)d->rowBlocks * d->colBlocks < (1L << 28);
+}
+inline int direct16_rows_wf(const Geometry& g) { return (g.K % 128 == 0 || g.K > 256) ? 2 : 1; }
+
+template <typename T, int WF>
+int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    D16R<WF>::LDS));
+        attr_set = true;
+    }
+    // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs
+    const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
+    const long blocks = std::max<long>(8, std::min<long>(device_cus(), (tiles + 7) / 8 * 8) / 8 * 8);
+    hipLaunchKernelGGL((direct16_rows_kernel<T, WF>), dim3((unsigned)blocks), dim3(512), D16R<WF>::LDS, st, (const T*)x,
+                       (const T*)W9, (T*)y, d, ep);
+    LAUNCH_CHECK("direct16_rows");
+    return WINO_OK;
+}
+
+size_t direct16_bank_bytes(const Geometry& g) { return (size_t)9 * round_up(g.C, 32) * round_up(g.K, 128) * 2; }
 
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
     D16Geom d;
@@ -719,11 +766,13 @@ int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry&
                     void* W9, void* y, hipStream_t st) {
     if (misaligned(x, 4)) return fail(WINO_ERR_UNSUPPORTED, "the 16-bit direct path loads column pairs: x must be 4-byte aligned");
     D16Geom d;
-    // pixels per tile: 512, fewer when that leaves the chip short of tiles; blocks of whole rows when the layer allows
-    int npg = 4;
-    const bool rows = direct16_plan(g, 4, true, &d) &&
-                      (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
-    if (!rows) {
+    // large layers: the 8-wave kernel, one workgroup per CU; else tiles of 512 pixels, fewer pixels when that leaves
+    // the chip short of tiles
+    int npg = 4, wf = direct16_rows_wf(g);
+    const bool big = !misaligned(y, 4) && (wf == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d)) &&
+               (long)d.rowBlocks * d.colBlocks * d.kTiles >= device_cus();
+    const bool rows = !big && direct16_plan(g, 4, true, &d) && (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
+    if (!big && !rows) {
         for (; npg > 1; npg >>= 1) {
             if (!direct16_plan(g, npg, false, &d)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: no block shape for this layer");
             if ((long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus()) break;
@@ -736,6 +785,8 @@ int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry&
 #define D16_GO(T)                                                                                                  \
     hipLaunchKernelGGL(direct16_pack_kernel<T>, pgrid, dim3(256), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
     LAUNCH_CHECK("direct16_pack");                                                                                 \
+    if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, st);                                  \
+    if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, st);                                             \
     if (rows) return launch_direct16_t<T, 4, true>(d, ep, x, W9, y, st);                                           \
     if (npg == 4) return launch_direct16_t<T, 4, false>(d, ep, x, W9, y, st);                                      \
     if (npg == 2) return launch_direct16_t<T, 2, false>(d, ep, x, W9, y, st);                                      \

@@ -32,6 +32,40 @@ def test_integers_round_once(oracle, shape, dtype):
         assert np.array_equal(host(got), rounded(want, dtype, oracle)), pad
 
 
+# Layers with at least one tile per CU, output heights that are multiples of 4, even widths and filter counts that
+# are multiples of 64 run on the 8-wave kernel (one workgroup per CU, tiles of 64 or 128 filters x 4-row strips):
+# (N, C, K, H, W, pad)
+#   * 128-filter tiles, a block as wide as the image, 4 stages per tile;
+#   * 64-filter tiles (K = 64), 200 columns in a block of 256, a last stage whose second channel vector lies past C;
+#   * K = 192 (64-filter tiles, three of them), no padding, blocks of 8 rows x 128 columns;
+#   * 12-row images under blocks of 16 rows: a block spans three images;
+#   * two column blocks, the second one half empty.
+BIG_SHAPES = [(32, 64, 128, 112, 112, 1), (16, 24, 64, 64, 200, 1), (12, 16, 192, 66, 130, 0), (192, 16, 256, 12, 24, 1),
+              (16, 32, 128, 32, 160, 1)]
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", BIG_SHAPES)
+def test_integers_round_once_one_tile_per_cu_and_more(oracle, shape, dtype):
+    """Whole tensors against the staged Winograd pipeline (exact on these integers as well: every transformed value
+    is a multiple of 1/4 far inside the 16-bit formats' exact range), the first and the last image's planes of
+    three filters against the oracle, twice (the kernel's workgroups are persistent: the second run must not depend
+    on what the first left in LDS)."""
+    N, C, K, H, W, pad = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -1, 1).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    xd, wd, bd = dev(x, dtype), dev(w, dtype), dev(bias, dtype)
+    ref = ops.conv(xd, wd, pad, algo=ops.ALGO_STAGED, relu=True, bias=bd)
+    ks = sorted({0, K // 2, K - 1})
+    for rep in range(2):
+        got = ops.conv(xd, wd, pad, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+        assert torch.equal(got, ref), rep
+        for n in (0, N - 1):
+            want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], pad) + bias[ks][None, :, None, None], 0)
+            assert np.array_equal(host(got[n:n + 1][:, ks]), rounded(want.astype(np.float32), dtype, oracle)), (rep, n)
+
+
 @pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
 @pytest.mark.parametrize("shape", [(2, 64, 64, 56, 56), (1, 128, 256, 28, 28), (3, 256, 64, 14, 14)])
 def test_floats_within_tolerance(oracle, shape, dtype):
