@@ -770,7 +770,7 @@ int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry&
     // the chip short of tiles
     int npg = 4, wf = direct16_rows_wf(g);
     const bool big = !misaligned(y, 4) && (wf == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d)) &&
-               (long)d.rowBlocks * d.colBlocks * d.kTiles >= device_cus();
+               (long)d.rowBlocks * d.colBlocks * d.kTiles >= device_cus() / 2;
     const bool rows = !big && direct16_plan(g, 4, true, &d) && (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
     if (!big && !rows) {
         for (; npg > 1; npg >>= 1) {
