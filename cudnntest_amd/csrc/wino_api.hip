@@ -837,11 +837,16 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
 }
 
 // Where AUTO leaves the Winograd kernels: layers with C <= 4 (direct.hpp), and 2-byte NCHW layers with large images
-// and enough tiles for the whole chip (direct16.hpp; measured on the VGG-16 shapes at N = 32 in bf16: 222 against
-// 373 us at C = K = 64, H = 224; 150 against 245 us at C = K = 128, H = 112; 148 against 164 us at C = K = 256, H = 56;
-// from 28 x 28 down the Winograd pipelines are faster).  x: the input tensor if known (its alignment decides).
+// and enough tiles for the whole chip (direct16.hpp, direct16_rows.hpp; measured on the VGG-16 shapes at N = 32 in
+// bf16, direct against the fastest Winograd pipeline: 175 against 373 us at C = K = 64, H = 224; 138 against 245 us
+// at C = K = 128, H = 112; 130 against 164 us at C = K = 256, H = 56; 75 against 79 and 127 against 135 us for the
+// two 28 x 28 shapes, which only the 8-wave kernel wins; at 14 x 14 the Winograd pipelines are faster, 55 against
+// 98 us).  x: the input tensor if known (its alignment decides).
 bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x) {
     if (!direct16_ok(src, dst, dtype, flags, g) || misaligned(x, 4)) return false;
+    D16Geom d;
+    const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d);
+    if (plan8 && g.Ho >= 28 && g.Wo >= 28 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus()) return true;
     if (g.Ho < 48 || g.Wo < 48) return false;
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
     return tiles >= 2L * device_cus();
