@@ -51,31 +51,44 @@ struct D16Geom {
 };
 
 // ---- filter bank -> W9[tap][Cp/8][Kp][8] (zero padded) --------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void direct16_pack_kernel(const T* __restrict__ w, T* __restrict__ W9, FltStrides s,
-                                                            int K, int C, int Kp, int CQ) {
-    const int k = blockIdx.x * 256 + threadIdx.x, cq = blockIdx.y;
+// One thread per (filter, channel vector).  VEC: the bank is [K][C][3][3] with C a multiple of 8 and a 16-byte
+// aligned base, so the 72 values of a thread are 144 contiguous, aligned bytes: nine 16-byte loads instead of 72
+// two-byte ones a filter apart.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(64) void direct16_pack_kernel(const T* __restrict__ w, T* __restrict__ W9, FltStrides s,
+                                                           int K, int C, int Kp, int CQ) {
+    const int k = blockIdx.x * 64 + threadIdx.x, cq = blockIdx.y;
     if (k >= Kp) return;
-    T raw[8][9];
+    unsigned short raw[72];                                  // [channel of the vector][tap]
+    const bool kin = k < K;
+    if (VEC) {
+        uint4 v[9];
+        const uint4* src = reinterpret_cast<const uint4*>(w + ((size_t)(kin ? k : K - 1) * C + (cq * 8 < C ? cq * 8 : 0)) * 9);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const int c = cq * 8 + e;
-        const T* wp = w + (k < K ? k : K - 1) * s.k + (c < C ? c : C - 1) * s.c;
+        for (int i = 0; i < 9; ++i) v[i] = src[i];
+        __builtin_memcpy(raw, v, sizeof(raw));
+    } else {
 #pragma unroll
-        for (int t = 0; t < 9; ++t) raw[e][t] = wp[(t / 3) * s.r + (t % 3) * s.s];
+        for (int e = 0; e < 8; ++e) {
+            const int c = cq * 8 + e;
+            const T* wp = w + (kin ? k : K - 1) * s.k + (c < C ? c : C - 1) * s.c;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const T val = wp[(t / 3) * s.r + (t % 3) * s.s];
+                __builtin_memcpy(&raw[e * 9 + t], &val, 2);
+            }
+        }
     }
 #pragma unroll
     for (int t = 0; t < 9; ++t) {
-        Pack16<T> pk;
+        unsigned short pk[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const bool ok = k < K && cq * 8 + e < C;
-            pk.e[e] = ok ? raw[e][t] : from_f32<T>(0.f);
-        }
-        *reinterpret_cast<Pack16<T>*>(W9 + (((size_t)t * CQ + cq) * Kp + k) * 8) = pk;
+        for (int e = 0; e < 8; ++e) pk[e] = (kin && cq * 8 + e < C) ? raw[e * 9 + t] : (unsigned short)0;    // +0.0 in both formats
+        uint4 out;
+        __builtin_memcpy(&out, pk, 16);
+        *reinterpret_cast<uint4*>(W9 + (((size_t)t * CQ + cq) * Kp + k) * 8) = out;
     }
 }
-
 
 // v with its lanes swapped pairwise (0 <-> 1, 2 <-> 3, ...)
 __device__ __forceinline__ float swap_lane_pairs(float v) {

@@ -781,9 +781,11 @@ int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry&
     }
     const Epilogue ep = make_epilogue(flags, bias);
     const FltStrides fs = flt_strides(WINO_NCHW, g.K, g.C);
-    dim3 pgrid((d.Kp + 255) / 256, d.CQ);
+    dim3 pgrid((d.Kp + 63) / 64, d.CQ);
+    const bool pvec = g.C % 8 == 0 && !misaligned(w, 16);
 #define D16_GO(T)                                                                                                  \
-    hipLaunchKernelGGL(direct16_pack_kernel<T>, pgrid, dim3(256), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
+    if (pvec) hipLaunchKernelGGL((direct16_pack_kernel<T, true>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
+    else hipLaunchKernelGGL((direct16_pack_kernel<T, false>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
     LAUNCH_CHECK("direct16_pack");                                                                                 \
     if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, st);                                  \
     if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, st);                                             \
