@@ -380,10 +380,11 @@ def main():
     }
 
     # ---- the same K steps with the filter bank transformed beforehand (filter transform excluded) ----
-    if not multi and stack is None and resolved[0] in ("staged", "epilogue", "fused"):
+    if not multi and stack is None and resolved[0] in ("staged", "epilogue", "fused", "staged_f4"):
         x0, w0, y0 = tensors[0]
-        U0 = ops.filter_transform(w0, layout)
-        a0 = {"staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE, "fused": ops.ALGO_FUSED}[resolved[0]]
+        U0 = ops.f4_filter_transform(w0, layout) if resolved[0] == "staged_f4" else ops.filter_transform(w0, layout)
+        a0 = {"staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE, "fused": ops.ALGO_FUSED,
+              "staged_f4": ops.ALGO_STAGED_F4}[resolved[0]]
         out["ms_per_step_filters_prepared"] = round(
             timed(lambda: ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0), args.steps, args.warmup)[0], 4)
 

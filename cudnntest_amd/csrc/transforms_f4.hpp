@@ -164,11 +164,13 @@ __global__ __launch_bounds__(256) void input_transform_f4_generic_kernel(const T
 // ---- output transform ------------------------------------------------------------------------------
 // PK = false: Mo[36][Kp][Pp], thread per (tile p, filter k), p fastest
 // PK = true : Mo[36][Pp][Kp], thread per (filter k, tile p), k fastest
+// Bias, ReLU and 2x2 max pooling as in the F(2x2) output stage: with pooling, s describes the pooled tensor
+// (Ho/2 x Wo/2) and a tile gives 2x2 pooled values; a window cut by the border is dropped.
 template <typename T, bool PK>
 __global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* __restrict__ Mo, T* __restrict__ y,
                                                                    ActStrides s, int N, int K, int Ho, int Wo, int th,
                                                                    int tw, long P, long Pp, int Kp, int order,
-                                                                   int relu) {
+                                                                   Epilogue ep) {
     long p;
     int k;
     if (PK) {
@@ -188,13 +190,27 @@ __global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* _
     output_tile_transform_f4(m, o);
     int n, ty, tx;
     decode_tile(p, order, N, th, tw, n, ty, tx);
-    if (relu) {
+    const float bv = bias_of<T>(ep, k);
 #pragma unroll
-        for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) o[a][b] = fmaxf(o[a][b], 0.f);
-    }
+        for (int b = 0; b < 4; ++b) {
+            o[a][b] += bv;
+            if (ep.relu) o[a][b] = fmaxf(o[a][b], 0.f);
+        }
     T* yp = y + n * s.n + k * s.c;
+    if (ep.pool) {
+        const int Hq = Ho / 2, Wq = Wo / 2;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int ph = 2 * ty + a, pw = 2 * tx + b;
+                const float v = fmaxf(fmaxf(o[2 * a][2 * b], o[2 * a][2 * b + 1]), fmaxf(o[2 * a + 1][2 * b], o[2 * a + 1][2 * b + 1]));
+                if (ph < Hq && pw < Wq) yp[ph * s.h + pw * s.w] = from_f32<T>(v);
+            }
+        return;
+    }
     if (s.w == 1 && (Wo & 3) == 0 && (s.h & 3) == 0 && (s.c & 3) == 0 && (s.n & 3) == 0 &&
         (reinterpret_cast<uintptr_t>(y) & (4 * sizeof(T) - 1)) == 0) {
         // W-contiguous destination, rows a multiple of 4 wide: one 4-element store per output row

@@ -544,20 +544,21 @@ int launch_f4_input(int layout, int order, const Geometry& g, const void* x, voi
 }
 
 template <typename T>
-int launch_f4_output(int layout, int order, int porder, unsigned flags, int N, int K, int Ho, int Wo, int Kp, long P,
-                     long Pp, const float* Mo, void* y, hipStream_t st) {
+int launch_f4_output(int layout, int order, int porder, unsigned flags, const void* bias, int N, int K, int Ho, int Wo,
+                     int Kp, long P, long Pp, const float* Mo, void* y, hipStream_t st) {
     const int th = (Ho + 3) / 4, tw = (Wo + 3) / 4;
-    const int relu = (flags & WINO_FLAG_RELU) ? 1 : 0;
+    const Epilogue ep = make_epilogue(flags, bias);
+    const ActStrides ys = out_strides(layout, flags, N, K, Ho, Wo);
     if (porder == WINO_PRODUCT_PK) {
         int bx = 64;
         while (bx < K && bx < 256) bx *= 2;
         dim3 block(bx, 256 / bx), grid((K + bx - 1) / bx, (unsigned)((P + block.y - 1) / block.y));
-        hipLaunchKernelGGL((output_transform_f4_kernel<T, true>), grid, block, 0, st, Mo, (T*)y,
-                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+        hipLaunchKernelGGL((output_transform_f4_kernel<T, true>), grid, block, 0, st, Mo, (T*)y, ys, N, K, Ho, Wo, th, tw, P,
+                           Pp, Kp, order, ep);
     } else {
         dim3 grid((unsigned)((P + 255) / 256), K), block(256);
-        hipLaunchKernelGGL((output_transform_f4_kernel<T, false>), grid, block, 0, st, Mo, (T*)y,
-                           act_strides(layout, N, K, Ho, Wo), N, K, Ho, Wo, th, tw, P, Pp, Kp, order, relu);
+        hipLaunchKernelGGL((output_transform_f4_kernel<T, false>), grid, block, 0, st, Mo, (T*)y, ys, N, K, Ho, Wo, th, tw, P,
+                           Pp, Kp, order, ep);
     }
     LAUNCH_CHECK("f4_output_transform");
     return WINO_OK;
@@ -853,14 +854,27 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
     return tiles >= 2L * device_cus();
 }
+// fp32 layers with a long reduction and enough 4x4 tiles run faster through the F(4x4,3x3) pipeline, product tensor
+// and all: 2.25 multiplies per output instead of 4, and a transformed input of 2.25x the tensor instead of 4x.
+// Measured at N = 32, NCHW, against the fastest F(2x2) pipeline: C = K = 256, H = 56: 0.42 against 0.53 ms;
+// C = 256, K = 512, H = 28: 0.22 against 0.28; C = K = 512, H = 28: 0.38 against 0.50; C = K = 512, H = 14 (512
+// tiles): 0.18 against 0.16, N = 64 (1024 tiles): 0.28 against 0.30; C = K = 128, H = 112: 0.58 against 0.56.
+// Its rounding error is about four times that of F(2x2) (3e-6 to 5e-6 relative L2 on these layers).
+bool auto_f4(int src, int dtype, const Geometry& g) {
+    // (from an NHWC source the layout-generic F(4x4) input transform is the slowest stage: no gain there yet)
+    if (dtype != WINO_F32 || src == WINO_NHWC || g.C < 256 || g.K < 128) return false;
+    const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
+    return tiles4 >= 1024;
+}
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, bool have_w) {
     if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x)) return WINO_ALGO_DIRECT;
+    if (have_w && auto_f4(src, dtype, g)) return WINO_ALGO_STAGED_F4;
     return pick_algo(src, dtype, g);
 }
 
-int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned flags, int N, int C, int K, int H, int W,
-                 int pad, const void* x, const void* w, const void* Upre, void* y, void* stream) {
+int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned flags, const void* bias, int N, int C, int K,
+                 int H, int W, int pad, const void* x, const void* w, const void* Upre, void* y, void* stream) {
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g, 4))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
@@ -893,7 +907,7 @@ int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned 
         if (rc) return rc;
     }
     StageScope t(WINO_STAGE_OUTPUT, st);
-    return wino_f4_output_transform(dst, dtype, order, porder, flags, N, K, g.Ho, g.Wo, Mo, y, stream);
+    DISPATCH_DTYPE(dtype, launch_f4_output<T>(dst, order, porder, flags, bias, N, K, g.Ho, g.Wo, g.Kp, g.P, g.Pp, Mo, y, st));
 }
 
 int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
@@ -912,7 +926,10 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     if (flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)) return fail(WINO_ERR_INVALID, "unknown flags 0x%x", flags);
     if ((flags & WINO_FLAG_POOL2) && (g.Ho < 2 || g.Wo < 2))
         return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", g.Ho, g.Wo);
-    if (algo == WINO_ALGO_AUTO) algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
+    if (algo == WINO_ALGO_AUTO) {
+        algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
+        if (algo == WINO_ALGO_STAGED_F4) Upre = nullptr;      // transformed filters handed in alongside w are F(2x2) ones
+    }
     if (algo == WINO_ALGO_DIRECT) {
         if (!w) return fail(WINO_ERR_INVALID, "the direct path needs the filter bank, not its Winograd transform");
         if (direct_ok(dst, flags, g)) {
@@ -928,11 +945,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
         return launch_direct16(dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
     }
-    if (algo == WINO_ALGO_STAGED_F4) {
-        if (bias || (flags & WINO_FLAG_POOL2))
-            return fail(WINO_ERR_UNSUPPORTED, "bias and pooling are not built for the F(4x4,3x3) mode");
-    }
-    if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(ss, src, dst, dtype, flags, N, C, K, H, W, pad, x, w, Upre, y, stream);
+    if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(ss, src, dst, dtype, flags, bias, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype, algo);
@@ -1042,7 +1055,10 @@ int conv_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     int passes = 1;
     if (valid_layout(src) && valid_layout(dst) && valid_dtype(dtype) && x && y && (w || Upre) &&
         make_geometry(dtype, N, C, K, H, W, pad, &g) && algo >= WINO_ALGO_AUTO && algo <= WINO_ALGO_DIRECT) {
-        if (algo == WINO_ALGO_AUTO) algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
+        if (algo == WINO_ALGO_AUTO) {
+            algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
+            if (algo == WINO_ALGO_STAGED_F4) Upre = nullptr;  // transformed filters handed in alongside w are F(2x2) ones
+        }
         passes = batch_passes(src, dst, dtype, algo, g);
     }
     if (passes <= 1) return conv_pass(ss, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, Upre, bias, y, stream);
@@ -1138,7 +1154,10 @@ size_t wino_workspace_bytes(int dtype, int N, int C, int K, int H, int W, int pa
         fail(WINO_ERR_INVALID, "bad shape or dtype");
         return 0;
     }
-    return scratch_layout(g, dtype).total;
+    Geometry g4;
+    size_t need = scratch_layout(g, dtype).total;
+    if (make_geometry(dtype, N, C, K, H, W, pad, &g4, 4)) need = std::max(need, scratch_layout(g4, dtype).total);
+    return need;
 }
 
 int wino_set_workspace(void* ptr, size_t bytes) {
@@ -1347,8 +1366,10 @@ int wino_f4_output_transform(int layout, int dtype, int tile_order, int product_
     const long P = (long)N * ((Ho + 3) / 4) * ((Wo + 3) / 4);
     const int Kp = (int)round_up(K, kKPad);
     const long Pp = round_up(P, kPPad);
-    DISPATCH_DTYPE(dtype, launch_f4_output<T>(layout, tile_order, product_order, flags, N, K, Ho, Wo, Kp, P, Pp, Mo, y,
-                                              (hipStream_t)stream));
+    if (flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)) return fail(WINO_ERR_INVALID, "unknown flags 0x%x", flags);
+    if ((flags & WINO_FLAG_POOL2) && (Ho < 2 || Wo < 2)) return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", Ho, Wo);
+    DISPATCH_DTYPE(dtype, launch_f4_output<T>(layout, tile_order, product_order, flags, nullptr, N, K, Ho, Wo, Kp, P, Pp, Mo,
+                                              y, (hipStream_t)stream));
 }
 
 int wino_stage_timing(int enable) {

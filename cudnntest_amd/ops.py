@@ -364,11 +364,11 @@ def f4_batched_gemm(U, V, C, K, P, product_order=PRODUCT_KP):
 
 
 def f4_output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False,
-                        dtype=torch.float32, product_order=PRODUCT_KP):
-    y = torch.empty(act_shape(layout, N, K, Ho, Wo), dtype=dtype, device=Mo.device)
+                        dtype=torch.float32, product_order=PRODUCT_KP, pool=False):
+    y = torch.empty(act_shape(layout, N, K, Ho // 2 if pool else Ho, Wo // 2 if pool else Wo), dtype=dtype, device=Mo.device)
     _lib.check(_lib.load().wino_f4_output_transform(int(layout), _DTYPES[dtype], tile_order, product_order,
-                                                    FLAG_RELU if relu else 0, N, K, Ho, Wo, _ptr(Mo), _ptr(y),
-                                                    _stream()), "wino_f4_output_transform")
+                                                    (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0), N, K, Ho, Wo,
+                                                    _ptr(Mo), _ptr(y), _stream()), "wino_f4_output_transform")
     return y
 
 

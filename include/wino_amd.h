@@ -55,8 +55,12 @@ typedef enum {
     WINO_ALGO_FUSED = 3,    /* one kernel: input transform, multiply-accumulate and output transform
                                (the structure of fusedTest/winotrans.cuh:1452 Winofuse4433) */
     WINO_ALGO_STAGED_F4 = 4, /* the staged pipeline in F(4x4,3x3) -- 6x6 tiles, 36 coordinates, the reference's
-                               own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101).
-                               Never chosen by WINO_ALGO_AUTO. */
+                               own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101):
+                               2.25 multiplies per output instead of 4, about four times the rounding error of
+                               F(2x2) (3e-6 to 5e-6 relative L2 in fp32 on the VGG layers).  WINO_ALGO_AUTO takes it
+                               for fp32 layers with C >= 256 and at least 1024 tiles from NCHW and CHWN sources when
+                               it is given the filter bank itself; transformed filters handed to this algorithm by
+                               name must come from wino_f4_filter_transform. */
     WINO_ALGO_DIRECT = 5     /* no Winograd at all, the convolution itself on the matrix cores.  Two kernels:
                                layers with C <= 4 (the network's first layer, which the reference runs through
                                the same wrappers: comparison/layoutCompare.cu:38-46): the 9*C <= 36 products of an
@@ -123,7 +127,7 @@ int wino_conv_prepared(int src, int dst, int dtype, int algo, unsigned flags, in
  * in the output stage of whichever algorithm runs, instead of the separate passes over y of
  *   addBias_CHWN / relu_CHWN / maxPool_CHWN
  *   netTest/cudnn_test_0124/VGG_Batched/CHWN_support.cuh:107,512,248
- * (the fused form is what fusedTest/winotrans.cuh:380-400 sketches).  Not built for WINO_ALGO_STAGED_F4.
+ * (the fused form is what fusedTest/winotrans.cuh:380-400 sketches).
  */
 int wino_conv_ex(int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
                  int W, int pad, const void *x, const void *w, const void *bias, void *y, void *stream);

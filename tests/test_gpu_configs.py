@@ -69,7 +69,7 @@ def test_n64_c512_every_pipeline(oracle, H, layout):
     ks, want = oracle_planes(oracle, x, w)
     xl, wl = to_layout(x, layout), to_layout(w, layout)
     base = None
-    for algo in (ops.ALGO_AUTO, ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED):
+    for algo in (ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_STAGED_F4, ops.ALGO_AUTO):
         y = from_layout(ops.conv(xl, wl, 1, layout, algo=algo), layout)
         assert tuple(y.shape) == (N, K, H, H)
         err = oracle.rel_l2(host(y[-1:][:, ks]), want)
@@ -77,16 +77,21 @@ def test_n64_c512_every_pipeline(oracle, H, layout):
         if base is None:
             base = y.clone()
         else:
-            assert rel(y, base) <= 1e-6, algo
-    # the filter bank transformed once, then the automatic choice again: the same bits as with the bank itself
+            # the F(2x2) pipelines differ by summation order; F(4x4) -- by name, or as the automatic choice for
+            # these long reductions -- has other transforms and three to four times the rounding error
+            assert rel(y, base) <= (1e-6 if algo in (ops.ALGO_EPILOGUE, ops.ALGO_FUSED) else 2e-5), algo
+    # the filter bank transformed once (F(2x2)), then the automatic choice among the F(2x2) pipelines: the same bits
+    # as that pipeline gives with the bank itself
     U = ops.filter_transform(wl, layout)
     yp = from_layout(ops.conv_prepared(xl, U, K, 1, layout), layout)
-    assert torch.equal(yp, base)
+    assert rel(yp, base) <= 1e-6
+    assert any(torch.equal(yp, from_layout(ops.conv(xl, wl, 1, layout, algo=a), layout))
+               for a in (ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED))
     # and in the other two destination layouts (the cross-layout entry points)
     for dst in LAYOUTS:
         if dst != layout:
             yd = from_layout(ops.conv(xl, wl, 1, layout, dst), dst)
-            assert rel(yd, base) <= 1e-6, dst
+            assert rel(yd, base) <= 2e-5, dst
 
 
 def test_n64_c512_h14_cut_rounds_repeat_bit_for_bit():

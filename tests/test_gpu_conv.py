@@ -95,9 +95,13 @@ def test_properties_at_full_size():
     x2 = torch.rand((N, C, H, H), device="cuda", generator=g) * 2 - 1
     w = torch.randn((K, C, 3, 3), device="cuda", generator=g) * (2.0 / (9 * C)) ** 0.5
     y1, y2 = ops.conv(x1, w), ops.conv(x2, w)
-    for algo in ALGOS[1:]:
+    # the F(2x2) pipelines agree to summation order; the automatic choice may be the F(4x4) pipeline (other
+    # transforms, three to four times the rounding error of F(2x2), still a twentieth of the 1e-4 layer tolerance)
+    ys = ops.conv(x1, w, algo=ALGOS[1])
+    for algo in ALGOS[2:]:
         ya = ops.conv(x1, w, algo=algo)
-        assert ((ya - y1).norm() / y1.norm()).item() < 1e-6, algo
+        assert ((ya - ys).norm() / ys.norm()).item() < 1e-6, algo
+    assert ((y1 - ys).norm() / ys.norm()).item() < 1e-5
     y12 = ops.conv(x1 + x2, w)
     rel = ((y12 - (y1 + y2)).norm() / y12.norm()).item()
     assert rel < 1e-5, rel
@@ -108,8 +112,8 @@ def test_properties_at_full_size():
     assert ((yd - x1).norm() / x1.norm()).item() < 1e-6
     y_nhwc = ops.conv(x1.permute(0, 2, 3, 1).contiguous(), w.permute(0, 2, 3, 1).contiguous(), src=ops.NHWC)
     y_chwn = ops.conv(x1.permute(1, 2, 3, 0).contiguous(), w.permute(1, 2, 3, 0).contiguous(), src=ops.CHWN)
-    assert ((y_nhwc.permute(0, 3, 1, 2) - y1).norm() / y1.norm()).item() < 1e-6
-    assert ((y_chwn.permute(3, 0, 1, 2) - y1).norm() / y1.norm()).item() < 1e-6
+    assert ((y_nhwc.permute(0, 3, 1, 2) - y1).norm() / y1.norm()).item() < 1e-5
+    assert ((y_chwn.permute(3, 0, 1, 2) - y1).norm() / y1.norm()).item() < 1e-5
 
 
 def test_caller_owned_workspace(oracle):

@@ -4,7 +4,8 @@ The joint identity  A^T[(G g G^T) . (B^T d B)]A == valid correlation(d, g)  is
 exact in rationals; for F(2x2,3x3) every constant is a power of two, so on small
 integers it must hold bit-for-bit in fp32 -- a wrong sign, a transposed matrix
 or a wrong tile origin breaks it.  Single-stage closed forms pin each stage on
-its own, and the tile geometry is checked against the instances the
+its own, for F(2x2) and for F(4x4) (one-hot taps, pixels and products against outer products of the columns of
+G, B^T and A^T), and the tile geometry is checked against the instances the
 reference's notebooks print (layoutTest/NCHW/data/ConvTest_V3_NCHW-Mar18.ipynb
 cell 2: inside=22 -> blockn=6, M=2304 at N=64).
 """
@@ -112,6 +113,84 @@ def test_input_transform_tiling_and_padding(oracle):
         assert np.array_equal(V[:, c, (n * 3 + ty) * 3 + tx], one)
     for layout in LAYOUTS:
         assert np.array_equal(oracle.wino_input_transform(synth.act_to_layout(x, layout), 1, layout, m=2), V)
+
+
+# F(4x4,3x3): the matrices of comparison/wrapedConv_NCHW.cuh:836-855 (B^T), :879-899 (G), :1084-1101 (A^T), written
+# out here as data and used only as the expected values of one-hot probes
+BT4 = np.array([[4, 0, -5, 0, 1, 0], [0, -4, -4, 1, 1, 0], [0, 4, -4, -1, 1, 0],
+                [0, -2, -1, 2, 1, 0], [0, 2, -1, -2, 1, 0], [0, 4, 0, -5, 0, 1]], np.float64)
+G4 = np.array([[1 / 4, 0, 0], [-1 / 6, -1 / 6, -1 / 6], [-1 / 6, 1 / 6, -1 / 6],
+               [1 / 24, 1 / 12, 1 / 6], [1 / 24, -1 / 12, 1 / 6], [0, 0, 1]], np.float64)
+AT4 = np.array([[1, 1, 1, 1, 1, 0], [0, 1, -1, 2, -2, 0], [0, 1, 1, 4, 4, 0], [0, 1, -1, 8, -8, 1]], np.float64)
+
+
+def test_f4_filter_transform_one_hot_taps(oracle):
+    # a single 1 at tap (r, s) gives outer(G[:, r], G[:, s]): nine probes pin every column of G on both sides
+    for r, s in itertools.product(range(3), range(3)):
+        w = np.zeros((1, 1, 3, 3), np.float32)
+        w[0, 0, r, s] = 1.0
+        U = oracle.wino_filter_transform(w, m=4).reshape(6, 6)
+        assert np.allclose(U, np.outer(G4[:, r], G4[:, s]), rtol=0, atol=1e-7), (r, s)
+    # multiples of 24 make every entry an integer: exact
+    w = np.zeros((1, 1, 3, 3), np.float32)
+    w[0, 0, 0, 2] = 576.0
+    assert np.array_equal(oracle.wino_filter_transform(w, m=4).reshape(6, 6), np.outer(24 * G4[:, 0], 24 * G4[:, 2]).astype(np.float32))
+    # index order U[xi][c][k] as for F(2x2)
+    K, C = 3, 2
+    w = synth.small_ints(K * C * 9, 8).reshape(K, C, 3, 3)
+    base = oracle.wino_filter_transform(w, 0, m=4)
+    assert base.shape == (36, C, K)
+    for k, c in itertools.product(range(K), range(C)):
+        assert np.array_equal(base[:, c, k], oracle.wino_filter_transform(w[k:k + 1, c:c + 1].copy(), 0, m=4)[:, 0, 0])
+
+
+def test_f4_input_transform_one_hot_pixels_and_tiling(oracle):
+    # B^T of F(4x4) is integral: a single 1 at d[r][s] of one 6x6 tile gives outer(B^T[:, r], B^T[:, s]) exactly
+    for r, s in itertools.product(range(6), range(6)):
+        x = np.zeros((1, 1, 6, 6), np.float32)
+        x[0, 0, r, s] = 1
+        V = oracle.wino_input_transform(x, pad=0, m=4).reshape(6, 6)
+        assert np.array_equal(V, np.outer(BT4[:, r], BT4[:, s]).astype(np.float32)), (r, s)
+    # a tile of ones: the row sums of B^T are (0, -6, 0, 0, 0, 0) -> only V[1][1] = 36
+    V = oracle.wino_input_transform(np.ones((1, 1, 6, 6), np.float32), pad=0, m=4).reshape(6, 6)
+    want = np.zeros((6, 6), np.float32)
+    want[1, 1] = 36
+    assert np.array_equal(V, want)
+    # pad 1, H = W = 7 -> 2x2 tiles of 4x4 outputs with origin (4ty-1, 4tx-1), zeros outside the image;
+    # tile (ty, tx) of image n is column p = (n*2 + ty)*2 + tx
+    N, C, H = 2, 2, 7
+    x = synth.small_ints(N * C * H * H, 23).reshape(N, C, H, H)
+    V = oracle.wino_input_transform(x, pad=1, m=4)
+    assert V.shape == (36, C, N * 4)
+    xp = np.pad(x, [(0, 0), (0, 0), (1, 4), (1, 4)])
+    for n, c, ty, tx in itertools.product(range(N), range(C), range(2), range(2)):
+        d = xp[n, c, 4 * ty:4 * ty + 6, 4 * tx:4 * tx + 6].copy().reshape(1, 1, 6, 6)
+        assert np.array_equal(V[:, c, (n * 2 + ty) * 2 + tx], oracle.wino_input_transform(d, pad=0, m=4).reshape(36))
+    for layout in LAYOUTS:
+        assert np.array_equal(oracle.wino_input_transform(synth.act_to_layout(x, layout), 1, layout, m=4), V)
+
+
+def test_f4_output_transform_one_hot_products(oracle):
+    # Mo = one-hot at (i, j) -> Y = outer(A^T[:, i], A^T[:, j]), exactly (A^T is integral)
+    for i, j in itertools.product(range(6), range(6)):
+        Mo = np.zeros((36, 1, 1), np.float32)
+        Mo[i * 6 + j] = 1
+        y = oracle.wino_output_transform(Mo, 1, 4, 4, m=4).reshape(4, 4)
+        assert np.array_equal(y, np.outer(AT4[:, i], AT4[:, j]).astype(np.float32)), (i, j)
+    # Ho = Wo = 6 -> 2x2 tiles, the last two rows and columns of the second tiles clipped
+    Mo = synth.small_ints(36 * 2 * 4, 5).reshape(36, 2, 4)
+    y = oracle.wino_output_transform(Mo, 1, 6, 6, m=4)
+    assert y.shape == (1, 2, 6, 6)
+    for k, ty, tx in itertools.product(range(2), range(2), range(2)):
+        tile = AT4 @ Mo[:, k, ty * 2 + tx].reshape(6, 6).astype(np.float64) @ AT4.T
+        hh, ww = min(4, 6 - 4 * ty), min(4, 6 - 4 * tx)
+        assert np.array_equal(y[0, k, 4 * ty:4 * ty + hh, 4 * tx:4 * tx + ww], tile[:hh, :ww].astype(np.float32))
+
+
+def test_f4_gemm_matches_einsum(oracle):
+    U = synth.small_ints(36 * 5 * 7, 1).reshape(36, 5, 7)
+    V = synth.small_ints(36 * 5 * 11, 2).reshape(36, 5, 11)
+    assert np.array_equal(oracle.wino_gemm(U, V, m=4), np.einsum("xck,xcp->xkp", U, V))
 
 
 def test_gemm_matches_einsum(oracle):
