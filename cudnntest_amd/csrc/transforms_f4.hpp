@@ -161,6 +161,77 @@ __global__ __launch_bounds__(256) void input_transform_f4_generic_kernel(const T
     for (int xi = 0; xi < 36; ++xi) vp[xi * plane] = from_f32<T>(v[xi]);
 }
 
+// ---- input transform, fp32 NHWC source, batch-major tiles: a row of tiles staged in LDS ------------------------
+// In NHWC the channels of a pixel are contiguous and the pixels of a tile are not: a thread per (tile, channel)
+// gathers 4-byte pieces 4 pixels apart.  Here a workgroup takes one image, one tile row, a block of at most 14 tile
+// columns and 32 channels: the 6 x (4*tiles + 2) pixels it needs are loaded 16 bytes per lane, 8 lanes per pixel
+// (128 contiguous bytes; every load unconditional from a clamped address and masked afterwards, twelve of them in
+// flight per lane), and stored to LDS with a pixel pitch of 33 words.  Then one thread per (channel of a vector,
+// tile, channel vector), channel fastest as in the layout-generic kernel: its 36 LDS reads hit distinct banks across
+// the wave (bank = 4*tile + channel + const), and the 4 lanes of a vector and the 16 tiles of a wave write 256
+// contiguous bytes of each coordinate plane of V.
+constexpr int F4N_CC = 32, F4N_PITCH = 33, F4N_TCB = 14;
+__global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const float* __restrict__ x, float* __restrict__ V,
+                                                                       int N, int C, int H, int W, int pad, int th,
+                                                                       int tw, long Pp, int Cp, int colBlocks) {
+    __shared__ float sm[6 * (4 * F4N_TCB + 2) * F4N_PITCH];
+    const int tid = threadIdx.x;
+    const int ty = blockIdx.x / colBlocks, cb = blockIdx.x - ty * colBlocks;
+    const int c0 = blockIdx.y * F4N_CC, n = blockIdx.z;
+    const int tx0 = cb * F4N_TCB, ntx = min(F4N_TCB, tw - tx0);
+    const int wlb = 4 * ntx + 2;                             // pixel columns of the block
+    const int h0 = 4 * ty - pad, w0 = 4 * tx0 - pad;
+    // ---- pixels -> LDS
+    const int npix = 6 * wlb;                                // <= 348: twelve passes of 32 pixels at most
+    const int ch4 = tid & 7, pl = tid >> 3;                  // 16-byte piece of the 32 channels; pixel of a pass
+    float4 raw[12];
+#pragma unroll
+    for (int q = 0; q < 12; ++q) {
+        const int pix = min(pl + 32 * q, npix - 1);
+        const int r = pix / wlb, col = pix - r * wlb;
+        const int ih = h0 + r, iw = w0 + col, c = c0 + 4 * ch4;
+        const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
+        const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - 1);
+        const unsigned keep = ok ? 0xFFFFFFFFu : 0u;
+        const float* src = x + (((size_t)n * H + ihc) * W + iwc) * C;
+        if ((C & 3) == 0 && c + 3 < C) {                     // wave-uniform unless C is not a multiple of 32
+            const float4 v = *reinterpret_cast<const float4*>(src + c);
+            raw[q] = make_float4(mask_keep(v.x, keep), mask_keep(v.y, keep), mask_keep(v.z, keep), mask_keep(v.w, keep));
+        } else {
+            float e[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) e[k] = mask_keep(src[min(c + k, C - 1)], c + k < C ? keep : 0u);
+            raw[q] = make_float4(e[0], e[1], e[2], e[3]);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 12; ++q) {
+        const int pix = pl + 32 * q;
+        if (pix < npix) {
+            float* d = sm + pix * F4N_PITCH + 4 * ch4;
+            d[0] = raw[q].x; d[1] = raw[q].y; d[2] = raw[q].z; d[3] = raw[q].w;
+        }
+    }
+    __syncthreads();
+    // ---- tiles
+    const size_t vplane = (size_t)Cp * Pp;
+    const int nvec = min(F4N_CC, Cp - c0) / 4;               // channel vectors of this workgroup (Cp is a multiple of 16)
+    const long p0 = ((long)n * th + ty) * tw + tx0;
+    for (int idx = tid; idx < nvec * ntx * 4; idx += 256) {
+        const int e = idx & 3, t = (idx >> 2) % ntx, ql = (idx >> 2) / ntx;
+        const float* src = sm + (4 * t) * F4N_PITCH + 4 * ql + e;
+        float d[6][6], v[36];
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+#pragma unroll
+            for (int j = 0; j < 6; ++j) d[i][j] = src[(i * wlb + j) * F4N_PITCH];
+        input_tile_transform_f4(d, v);
+        float* vp = V + ((size_t)(c0 / 4 + ql) * Pp + p0 + t) * 4 + e;
+#pragma unroll
+        for (int xi = 0; xi < 36; ++xi) vp[xi * vplane] = v[xi];
+    }
+}
+
 // ---- output transform ------------------------------------------------------------------------------
 // PK = false: Mo[36][Kp][Pp], thread per (tile p, filter k), p fastest
 // PK = true : Mo[36][Pp][Kp], thread per (filter k, tile p), k fastest

@@ -535,6 +535,14 @@ int launch_f4_filter(int layout, int K, int C, int Kp, int Cp, const void* w, vo
 template <typename T>
 int launch_f4_input(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st) {
     constexpr int CV = ChanVec<T>::n;
+    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && sizeof(T) == 4 && g.N <= 65535 && g.Cp / F4N_CC < 65535) {
+        const int colBlocks = (g.tw + F4N_TCB - 1) / F4N_TCB;
+        dim3 grid((unsigned)(g.th * colBlocks), (g.Cp + F4N_CC - 1) / F4N_CC, g.N);
+        hipLaunchKernelGGL(input_transform_f4_nhwc_kernel, grid, dim3(256), 0, st, (const float*)x, (float*)V, g.N, g.C, g.H, g.W,
+                           g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks);
+        LAUNCH_CHECK("f4_input_transform_nhwc");
+        return WINO_OK;
+    }
     dim3 grid((unsigned)((g.P * CV + 255) / 256), g.Cp / CV), block(256);
     hipLaunchKernelGGL(input_transform_f4_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
                        act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
@@ -859,17 +867,17 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
 // Measured at N = 32, NCHW, against the fastest F(2x2) pipeline: C = K = 256, H = 56: 0.42 against 0.53 ms;
 // C = 256, K = 512, H = 28: 0.22 against 0.28; C = K = 512, H = 28: 0.38 against 0.50; C = K = 512, H = 14 (512
 // tiles): 0.18 against 0.16, N = 64 (1024 tiles): 0.28 against 0.30; C = K = 128, H = 112: 0.58 against 0.56.
-// Its rounding error is about four times that of F(2x2) (3e-6 to 5e-6 relative L2 on these layers).
-bool auto_f4(int src, int dtype, const Geometry& g) {
-    // (from an NHWC source the layout-generic F(4x4) input transform is the slowest stage: no gain there yet)
-    if (dtype != WINO_F32 || src == WINO_NHWC || g.C < 256 || g.K < 128) return false;
+// (NHWC: 0.43 against 0.53 on the first of these, CHWN 0.41 against 0.52.)  Its rounding error is about four times that
+// of F(2x2) (3e-6 to 5e-6 relative L2 on these layers).
+bool auto_f4(int dtype, const Geometry& g) {
+    if (dtype != WINO_F32 || g.C < 256 || g.K < 128) return false;
     const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
     return tiles4 >= 1024;
 }
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, bool have_w) {
     if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x)) return WINO_ALGO_DIRECT;
-    if (have_w && auto_f4(src, dtype, g)) return WINO_ALGO_STAGED_F4;
+    if (have_w && auto_f4(dtype, g)) return WINO_ALGO_STAGED_F4;
     return pick_algo(src, dtype, g);
 }
 
