@@ -409,7 +409,11 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
     };
     const int xi = blockIdx.y;
     const int b = blockIdx.x;
-    const int xcd = xcd_map ? b & 7 : 0, jj = xcd_map ? b >> 3 : b;     // as in gemm_rows_kernel
+    // as in gemm_rows_kernel, but the XCD that takes slot s of a group of 8 tile columns moves on by one with every
+    // coordinate: with pTiles not a multiple of 8 the last group is partly empty, and the XCDs whose slots are filled
+    // there would otherwise carry a whole tile column more than the others in every one of the 16 or 36 planes
+    // (49 tile columns: 7 against 6, the kernel's duration is the 7)
+    const int xcd = xcd_map ? (b + xi) & 7 : 0, jj = xcd_map ? b >> 3 : b;
     const int ktile = jj % kTiles;
     const int ptile = (jj / kTiles) * (xcd_map ? 8 : 1) + xcd;
     if (ptile >= pTiles) return;

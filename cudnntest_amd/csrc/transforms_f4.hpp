@@ -88,33 +88,44 @@ __device__ __forceinline__ void output_tile_transform_f4(const float m[36], floa
     for (int a = 0; a < 4; ++a) at6(t[a], y[a]);
 }
 
-// ---- filter transform: thread per (filter k, channel c), k fastest --------------------------
-// One channel per thread (36 live values); the CV channels of a vector are written by CV
-// different threads, 4 or 2 bytes each -- the filter bank is small and transformed once.
+// ---- filter transform: thread per (filter k, channel vector), k fastest -----------------------------------
+// The CV channels of a vector one after the other (36 live values each), their results gathered into one
+// 16-byte store per coordinate: a wave writes 1 KB runs of U.
 template <typename T>
-__global__ __launch_bounds__(256) void filter_transform_f4_kernel(const T* __restrict__ w, T* __restrict__ U,
-                                                                   FltStrides s, int K, int C, int Kp, int Cp) {
+__global__ __launch_bounds__(64) void filter_transform_f4_kernel(const T* __restrict__ w, T* __restrict__ U,
+                                                                  FltStrides s, int K, int C, int Kp, int Cp) {
     constexpr int CV = ChanVec<T>::n;
     const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    const int c = blockIdx.y;
+    const int cq = blockIdx.y;
     if (k >= Kp) return;
-    float u[36];
-    if (k < K && c < C) {
-        float g[3][3];
-        const T* wp = w + k * s.k + c * s.c;
+    T out[36][CV];
 #pragma unroll
-        for (int r = 0; r < 3; ++r)
+    for (int e = 0; e < CV; ++e) {
+        const int c = cq * CV + e;
+        float u[36];
+        if (k < K && c < C) {
+            float g[3][3];
+            const T* wp = w + k * s.k + c * s.c;
 #pragma unroll
-            for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
-        filter_tile_transform_f4(g, u);
-    } else {
+            for (int r = 0; r < 3; ++r)
 #pragma unroll
-        for (int i = 0; i < 36; ++i) u[i] = 0.f;
+                for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
+            filter_tile_transform_f4(g, u);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 36; ++i) u[i] = 0.f;
+        }
+#pragma unroll
+        for (int xi = 0; xi < 36; ++xi) out[xi][e] = from_f32<T>(u[xi]);
     }
     const size_t plane = (size_t)Cp * Kp;
-    T* up = U + ((size_t)(c / CV) * Kp + k) * CV + (c % CV);
+    T* up = U + ((size_t)cq * Kp + k) * CV;
 #pragma unroll
-    for (int xi = 0; xi < 36; ++xi) up[xi * plane] = from_f32<T>(u[xi]);
+    for (int xi = 0; xi < 36; ++xi) {
+        uint4 v;
+        __builtin_memcpy(&v, out[xi], 16);
+        *reinterpret_cast<uint4*>(up + xi * plane) = v;
+    }
 }
 
 // ---- input transform, layout-generic -------------------------------------------------------
