@@ -2,8 +2,8 @@
 """Benchmark of the Winograd 3x3 convolution hot path on one MI355X.
 
 A step is one whole layer through the drop-in entry point (wino_conv: filter
-transform + input transform + 16-way GEMM + output transform, or their fused
-forms; inputs already in HBM).  The default workload is the VGG-16 conv3-style
+transform + input transform + 16- or 36-way GEMM + output transform, or their fused
+forms, as the library's automatic choice resolves; inputs already in HBM).  The default workload is the VGG-16 conv3-style
 layer the headline metric is quoted on: 3x3, stride 1, pad 1, N=32, C=K=256,
 H=W=56, fp32, NCHW.  `--workload vgg16_all13` makes a step the thirteen VGG-16
 convolutions (ReLU fused into the output stage) on synthetic activations of each
@@ -67,15 +67,26 @@ WORKLOADS = {
 # script (the summary file holds the counters and the copy-kernel scale factor), keyed by
 # (workload, layout, dtype, resolved algo): (bytes, summary under profiles/).
 MEASURED_TRAFFIC = {
-    # 596.1 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
+    # gemm_128x128_kernel of the F(4x4) pipeline: 314.5 MB fetched + 231.2 MB written
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged_f4"):
+        (545.7e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # 635.7 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"):
-        (707.3e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt"),
-    # 449.1 MB fetched + 411.0 MB written
+        (746.9e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # 454.1 MB fetched + 411.0 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"):
-        (860.1e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_hbm_traffic.txt"),
-    # 596.4 MB fetched + 411.0 MB written
+        (865.1e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # 578.9 MB fetched + 411.0 MB written
     ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"):
-        (1007.4e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_hbm_traffic.txt"),
+        (989.9e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # direct16_rows_kernel: 83.1 + 51.4 MB; 325.3 + 208.9 MB
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "direct"):
+        (134.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv3_N32_counters.txt"),
+    ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "bf16", "direct"):
+        (534.2e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # gemm_rows_kernel in bf16: 271.7 MB fetched + 56.9 MB written
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "epilogue"):
+        (328.6e6, "profiles/epilogue_bf16_nchw_vgg16_conv3_N32_counters.txt"),
 }
 # what the default run also times, after the headline's timed region: (name, workload, dtype)
 OTHER_CONFIGS = [
@@ -87,7 +98,7 @@ OTHER_CONFIGS = [
     ("cfg5_vgg16_all13_N32_bf16", "vgg16_all13", "bf16"),
 ]
 KERNEL_OF = {"staged": "gemm_128x128_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
-             "staged_f4": "gemm_128x128_kernel", "direct": "direct conv kernel"}
+             "staged_f4": "gemm_128x128_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel"}
 
 
 def main():
