@@ -516,4 +516,163 @@ __global__ __launch_bounds__(256) void gemm_128x128_kernel(const T* __restrict__
             }
 }
 
+// =============================================================================
+// The same GEMM as one resident set of workgroups that WALK the (coordinate, tile column) pairs.
+//
+// gemm_128x128_kernel starts and ends a workgroup per (tile, coordinate): three stages of loads in flight before
+// its first multiply, 64 KB of product stores after its last -- about 6 us of a 33 us workgroup when the reduction
+// is 256 channels long.  Here the grid is the resident set (two workgroups per CU).  The pairs, tile column fastest,
+// are dealt round-robin to GROUPS of kTiles workgroups -- the filter tiles of a pair, on one XCD, so that its L2
+// serves the shared V slab; at any time the whole chip works on a few neighbouring coordinates, whose U planes stay
+// in the L2s -- and a workgroup runs its pairs as ONE pipeline: the load ring moves on to the next pair's rows when
+// the current pair's last stage has been requested, and at the end of a pair's reduction the workgroup stores the
+// product and clears its accumulators while those loads are in flight.
+// =============================================================================
+template <typename T, int NV, bool PK, int RING>
+__global__ __launch_bounds__(256, 2) void gemm_128x128_walk_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                                   float* __restrict__ Mo, int Cp, int Kp, long Pp,
+                                                                   int kTiles, int pTiles, int nxi, int groups) {
+    typedef typename Mma<T>::vec vec;
+    constexpr int CV = ChanVec<T>::n;
+    static_assert(RING >= 3 && RING <= 4, "ring depth");
+    __shared__ vec As0[NV][GEMM_BM], As1[NV][GEMM_BM], As2[NV][GEMM_BM], As3[RING > 3 ? NV : 1][GEMM_BM];
+    __shared__ vec Bs0[NV][GEMM_BN], Bs1[NV][GEMM_BN], Bs2[NV][GEMM_BN], Bs3[RING > 3 ? NV : 1][GEMM_BN];
+    auto aslot = [&](auto sl) -> vec(*)[GEMM_BM] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return As0; else if constexpr (S == 1) return As1; else if constexpr (S == 2) return As2; else return As3;
+    };
+    auto bslot = [&](auto sl) -> vec(*)[GEMM_BN] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return Bs0; else if constexpr (S == 1) return Bs1; else if constexpr (S == 2) return Bs2; else return Bs3;
+    };
+    const int b = blockIdx.x;
+    const int xcd = b & 7, v = b >> 3;                   // ids go round-robin to the XCDs
+    const int gl = v / kTiles, ktile = v - gl * kTiles;
+    const int grp = gl * 8 + xcd;
+    const int units = pTiles * nxi;                      // pairs, q = xi * pTiles + tile column
+    if (grp >= groups || grp >= units) return;
+    const int mine = (units - grp + groups - 1) / groups;    // pairs grp, grp + groups, ...
+    const int k0 = ktile * GEMM_BM;
+    const int CQ = Cp / CV, nch = CQ / NV;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const unsigned lane_off = lane * 16;
+    const uint64_t stepU = (uint64_t)NV * Kp * 16, stepV = (uint64_t)NV * Pp * 16;
+    constexpr int WV = (RING - 2) * NV;
+    constexpr int WAIT_IMM = (WV & 0xF) | (0x7 << 4) | (0xF << 8) | ((WV >> 4) << 14);
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // ---- load side: the pair whose rows are being requested
+    uint64_t sptr[NV];
+    int lq = grp, lst = 0;                               // pair and stage of it to request next
+    auto point_at = [&](int q) {
+        const int xi = q / pTiles, ptile = q - xi * pTiles;
+        const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
+        const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + (size_t)ptile * GEMM_BN;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int piece = wave + 4 * i;
+            const int opnd = i / (NV / 2);
+            const int row = (piece >> 1) % NV, half = piece & 1;
+            sptr[i] = opnd ? reinterpret_cast<uint64_t>(Vb + (size_t)row * Pp + half * 64)
+                           : reinterpret_cast<uint64_t>(Ub + (size_t)row * Kp + half * 64);
+        }
+    };
+    point_at(lq);
+    auto stage_load = [&](auto sl) {
+        // past the last pair: the last stage again (never read)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int piece = wave + 4 * i;
+            const int opnd = i / (NV / 2);
+            const int row = (piece >> 1) % NV, half = piece & 1;
+            dma_row(sptr[i], lane_off, opnd ? &bslot(sl)[row][half * 64] : &aslot(sl)[row][half * 64]);
+        }
+        if (++lst == nch) {
+            lst = 0;
+            if (lq + groups < units) {
+                lq += groups;
+                point_at(lq);
+            } else {
+                lst = nch - 1;                           // stay on the last stage
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) sptr[i] += (i / (NV / 2)) ? stepV : stepU;
+        }
+    };
+    // ---- compute side
+    int cq = grp, cst = 0;
+    auto iteration = [&](auto sl) {
+        __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        stage_load(std::integral_constant<int, (decltype(sl)::value + RING - 1) % RING>{});
+        __builtin_amdgcn_sched_barrier(0);
+        vec a[2][2], bq[2][2];
+        auto frag_load = [&](int g) {
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
+                const vec fa = aslot(sl)[2 * g + lh][(PK ? wn : wm) * 64 + qq * 32 + l32];
+                const vec fb = bslot(sl)[2 * g + lh][(PK ? wm : wn) * 64 + qq * 32 + l32];
+                a[g & 1][qq] = PK ? fb : fa;
+                bq[g & 1][qq] = PK ? fa : fb;
+            }
+        };
+        frag_load(0);
+#pragma unroll
+        for (int g = 0; g < NV / 2; ++g) {
+            if (g + 1 < NV / 2) frag_load(g + 1);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) Mma<T>::run(a[g & 1][i], bq[g & 1][j], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (++cst == nch) {                              // the pair's reduction is complete: store it, start the next
+            cst = 0;
+            const int xi = cq / pTiles, ptile = cq - xi * pTiles;
+            cq += groups;
+            const long p0 = (long)ptile * GEMM_BN;
+            // (the row pitch is made opaque here: the 64 store addresses of a thread would otherwise be computed
+            // ahead of the loop and kept in registers across it -- 300 registers, one workgroup per CU)
+            long pitch = PK ? (long)Kp : Pp;
+            asm volatile("" : "+s"(pitch));
+            float* Mb = Mo + (size_t)xi * Kp * Pp +
+                        (PK ? (size_t)(p0 + wm * 64 + 4 * lh) * pitch + k0 + wn * 64 + l32
+                            : (size_t)(k0 + wm * 64 + 4 * lh) * pitch + p0 + wn * 64 + l32);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float* row = Mb + (size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * pitch;      // MFMA row; lanes: columns
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        row[j * 32] = acc[i][j][r];
+                        acc[i][j][r] = 0.f;
+                    }
+                }
+        }
+    };
+    const int total = mine * nch;
+    for_each_const(std::make_integer_sequence<int, RING - 1>{}, stage_load);
+    int s = 0;
+    for (; s + RING <= total; s += RING) for_each_const(std::make_integer_sequence<int, RING>{}, iteration);
+    if (s < total) iteration(std::integral_constant<int, 0>{});
+    if (s + 1 < total) iteration(std::integral_constant<int, 1>{});
+    if (RING > 3 && s + 2 < total) iteration(std::integral_constant<int, 2>{});
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  // the surplus requests of the last stages
+}
+
 }  // namespace wino
