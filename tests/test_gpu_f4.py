@@ -65,6 +65,34 @@ def test_f4_batched_gemm(oracle, porder):
     assert np.array_equal(Mo[:, :K, :P], want)
 
 
+@pytest.mark.parametrize("porder", [ops.PRODUCT_KP, ops.PRODUCT_PK])
+@pytest.mark.parametrize("C,K,P", [(16, 70, 128 * 70), (80, 200, 128 * 22 - 5), (380, 600, 128 * 9)])
+def test_f4_batched_gemm_walking_workgroups(oracle, porder, C, K, P):
+    """Products with work for three and more rounds of the resident workgroups and a reduction of at most 24 stages run
+    on the kernel whose workgroups walk the (coordinate, tile column) pairs in one pipeline: one, two and five filter
+    tiles (groups of workgroups that do and do not divide an XCD's share), reductions of 1, 5 and 24 stages, a ragged
+    last tile column; bit-exact on integers, twice (nothing may depend on what a previous launch left in LDS)."""
+    g = ops.f4_geometry(ops.F32, 1, C, K, 6, 6, 1)
+    Cp, Kp, Pp = g["Cp"], g["Kp"], (P + 127) // 128 * 128
+    U = np.zeros((36, Cp, Kp), np.float32)
+    V = np.zeros((36, Cp, Pp), np.float32)
+    U[:, :C, :K] = synth.small_ints(36 * C * K, 13, -2, 2).reshape(36, C, K)
+    V[:, :C, :P] = synth.small_ints(36 * C * P, 14, -3, 3).reshape(36, C, P)
+    Ud, Vd = pack_operand(U), pack_operand(V)
+    want = np.einsum("xck,xcp->xkp", U[:, :C, :K], V[:, :C, :P], optimize=True)
+    pins = [(0, 0, 0), (35, K - 1, P - 1), (17, K // 2, P // 3)]
+    ref = oracle.wino_gemm(np.ascontiguousarray(U[:, :C, :K]), np.ascontiguousarray(V[:, :C, :P]), m=4) if C * K * P < 2e8 else None
+    for rep in range(2):
+        Mo = host(ops.f4_batched_gemm(Ud, Vd, C, K, P, porder))
+        if porder == ops.PRODUCT_PK:
+            Mo = Mo.transpose(0, 2, 1)
+        assert np.array_equal(Mo[:, :K, :P], want), rep
+    if ref is not None:
+        assert np.array_equal(ref, want)
+    for xi, k, p_ in pins:                       # the einsum itself against a plain dot product
+        assert want[xi, k, p_] == float(np.dot(U[xi, :C, k].astype(np.float64), V[xi, :C, p_].astype(np.float64)))
+
+
 @pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("order", [ops.TILES_BATCH_MAJOR, ops.TILES_BATCH_MINOR])
 @pytest.mark.parametrize("porder", [ops.PRODUCT_KP, ops.PRODUCT_PK])
