@@ -781,9 +781,13 @@ int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const
     return WINO_OK;
 }
 
-// W9: room for direct16_bank_bytes(g), 16-byte aligned
+// W9: room for direct16_bank_bytes(g), 16-byte aligned.  The order of the bank depends on the kernel that reads it,
+// and that on the layer and on the alignment of x and y, so packing and running take the same arguments:
+// D16_PACK_RUN both, D16_PACK only the bank (x and y are looked at, not touched), D16_RUN with a bank packed earlier
+// for tensors of the same alignment.
+enum { D16_PACK_RUN = 0, D16_PACK = 1, D16_RUN = 2 };
 int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
-                    void* W9, void* y, hipStream_t st) {
+                    void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN) {
     if (misaligned(x, 4)) return fail(WINO_ERR_UNSUPPORTED, "the 16-bit direct path loads column pairs: x must be 4-byte aligned");
     D16Geom d;
     // large layers: the 8-wave kernel, one workgroup per CU; else tiles of 512 pixels, fewer pixels when that leaves
@@ -804,9 +808,12 @@ int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry&
     dim3 pgrid((d.Kp + 63) / 64, d.CQ);
     const bool pvec = g.C % 8 == 0 && !misaligned(w, 16);
 #define D16_GO(T)                                                                                                  \
-    if (pvec) hipLaunchKernelGGL((direct16_pack_kernel<T, true>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
-    else hipLaunchKernelGGL((direct16_pack_kernel<T, false>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
-    LAUNCH_CHECK("direct16_pack");                                                                                 \
+    if (mode != D16_RUN) {                                                                                         \
+        if (pvec) hipLaunchKernelGGL((direct16_pack_kernel<T, true>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
+        else hipLaunchKernelGGL((direct16_pack_kernel<T, false>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
+        LAUNCH_CHECK("direct16_pack");                                                                             \
+    }                                                                                                              \
+    if (mode == D16_PACK) return WINO_OK;                                                                          \
     if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, st);                                  \
     if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, st);                                             \
     if (rows) return launch_direct16_t<T, 4, true>(d, ep, x, W9, y, st);                                           \
@@ -1442,6 +1449,8 @@ struct wino_stack {
         unsigned flags;
         void* U = nullptr;         // cached transformed filters
         void* wraw = nullptr;      // layers with C <= 4: a copy of the filter bank itself, for the direct path
+        void* U4 = nullptr;        // fp32 layers AUTO runs through F(4x4): their filters transformed for it
+        void* W9 = nullptr;        // 2-byte NCHW layers AUTO runs directly: the bank in the direct kernel's order
         void* bias = nullptr;
         bool set = false, has_bias = false;
     };
@@ -1463,8 +1472,22 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
     for (int l = 0; l < n; ++l) {
         const auto& L = s->layers[l];
         void* out = l + 1 == n ? y : s->act[l & 1];
-        int rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
-                           L.wraw, L.U, L.has_bias ? L.bias : nullptr, out, stream);
+        const void* bias = L.has_bias ? L.bias : nullptr;
+        int rc;
+        Geometry g;
+        make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g);
+        if (L.U4) {
+            rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, WINO_ALGO_STAGED_F4, L.flags, s->N, L.C, L.K, L.H,
+                           L.W, 1, in, nullptr, L.U4, bias, out, stream);
+        } else if (L.W9 && !misaligned(in, 4) && !misaligned(out, 4) &&
+                   auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in)) {
+            // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
+            StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
+            rc = launch_direct16(s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
+        } else {
+            rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
+                           L.wraw, L.U, bias, out, stream);
+        }
         if (rc) return rc;
         in = out;
     }
@@ -1528,6 +1551,15 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         const bool direct16_layer = dtype != WINO_F32 && L.layout_in == WINO_NCHW && L.layout_out == WINO_NCHW &&
                                     L.C % 8 == 0 && !(L.flags & WINO_FLAG_POOL2);
         if (e == hipSuccess && (L.C <= 4 || direct16_layer)) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
+        // what AUTO runs outside the F(2x2) kernels gets its filters prepared once as well
+        if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && auto_f4(dtype, g)) {
+            Geometry g4;
+            make_geometry(dtype, N, L.C, L.K, L.H, L.W, 1, &g4, 4);
+            e = hipMalloc(&L.U4, (size_t)36 * g4.Cp * g4.Kp * es);
+        }
+        if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && direct16_layer &&
+            auto_direct16(L.layout_in, L.layout_out, dtype, L.flags, g, nullptr))
+            e = hipMalloc(&L.W9, direct16_bank_bytes(g));
         if (e != hipSuccess) return bail(e);
     }
     for (int i = 0; i < 2 && raw->act_bytes; ++i) {
@@ -1549,6 +1581,16 @@ int wino_stack_set_layer(wino_stack_t* s, int layer, const void* w, const void* 
     if (L.wraw)
         HIP_TRY(hipMemcpyAsync(L.wraw, w, (size_t)9 * L.K * L.C * dtype_size(s->dtype), hipMemcpyDeviceToDevice,
                                (hipStream_t)stream));
+    if (L.U4) {
+        rc = wino_f4_filter_transform(L.layout_in, s->dtype, L.K, L.C, w, L.U4, stream);
+        if (rc) return rc;
+    }
+    if (L.W9) {
+        Geometry g;
+        make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g);
+        rc = launch_direct16(s->dtype, L.flags, nullptr, g, L.W9, w, L.W9, L.W9, (hipStream_t)stream, D16_PACK);   // (x, y: any aligned address)
+        if (rc) return rc;
+    }
     L.has_bias = bias != nullptr;
     if (bias)
         HIP_TRY(hipMemcpyAsync(L.bias, bias, (size_t)L.K * dtype_size(s->dtype), hipMemcpyDeviceToDevice,
@@ -1583,6 +1625,8 @@ int wino_stack_forward_graph(wino_stack_t* s, const void* x, void* y, void* stre
         Geometry g;
         if (!make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g)) return fail(WINO_ERR_INVALID, "bad layer shape");
         need = std::max(need, scratch_layout(g, s->dtype).total);
+        Geometry g4;
+        if (L.U4 && make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4)) need = std::max(need, scratch_layout(g4, s->dtype).total);
     }
     void* base = nullptr;
     int rc = arena_get(need, &base);
@@ -1616,6 +1660,8 @@ int wino_stack_destroy(wino_stack_t* s) {
     for (auto& L : s->layers) {
         if (L.U) (void)hipFree(L.U);
         if (L.wraw) (void)hipFree(L.wraw);
+        if (L.U4) (void)hipFree(L.U4);
+        if (L.W9) (void)hipFree(L.W9);
         if (L.bias) (void)hipFree(L.bias);
     }
     for (int i = 0; i < 2; ++i)

@@ -156,3 +156,46 @@ def test_stack_graph_follows_a_change_of_bias(oracle):
     with pytest.raises(ValueError):
         st.set_layer(0, dev(params[0][0]), torch.zeros(7, device="cuda"))
     st.close()
+
+
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
+def test_stack_layers_on_the_f4_pipeline(oracle, layout):
+    """fp32 layers that the automatic choice runs through F(4x4,3x3) (C, K >= 128, one of them 256, 512 tiles and
+    more): the stack transforms their filters for that pipeline when they are set; the pass gives the bits of the
+    layers run one by one with the algorithm named, and the oracle's planes within the fp32 tolerance."""
+    N, C, H = 32, 128, 32
+    layers = [dict(K=256, relu=True, pool=True, layout_in=layout, layout_out=layout),
+              dict(K=128, relu=True, pool=False, layout_in=layout, layout_out=layout)]
+    assert ops.pick_algo(layout, ops.F32, N, C, 256, H, H, 1) == ops.ALGO_STAGED_F4
+    assert ops.pick_algo(layout, ops.F32, N, 256, 128, H // 2, H // 2, 1) == ops.ALGO_STAGED_F4
+    st = ops.ConvStack(torch.float32, N, C, H, H, layers)
+    g = torch.Generator(device="cuda").manual_seed(0xF4)
+    x = torch.rand((N, C, H, H), device="cuda", generator=g) * 2 - 1
+    ws, bs = [], []
+    c = C
+    for i, L in enumerate(layers):
+        ws.append(torch.randn((L["K"], c, 3, 3), device="cuda", generator=g) * (2.0 / (9 * c)) ** 0.5)
+        bs.append(torch.randn((L["K"],), device="cuda", generator=g) * 0.1)
+        c = L["K"]
+
+    def lay(t, flt=False):
+        if layout == ops.NCHW:
+            return t.contiguous()
+        return (t.permute(0, 2, 3, 1) if layout == ops.NHWC else t.permute(1, 2, 3, 0)).contiguous()
+
+    for i in range(2):
+        st.set_layer(i, lay(ws[i]), bs[i])
+    got = st.forward(lay(x)).clone()
+    a = lay(x)
+    for i, L in enumerate(layers):
+        a = ops.conv(a, lay(ws[i]), 1, layout, algo=ops.ALGO_STAGED_F4, relu=True, pool=L["pool"], bias=bs[i])
+    assert torch.equal(got, a)
+    got_nchw = got if layout == ops.NCHW else (got.permute(0, 3, 1, 2) if layout == ops.NHWC else got.permute(3, 0, 1, 2))
+    want = reference_chain(oracle, host(x[-1:]), [(host(w), host(b)) for w, b in zip(ws, bs)], layers)
+    assert oracle.rel_l2(host(got_nchw[-1:]), want) <= TOL[ops.F32]
+    out = torch.empty_like(got)
+    for rep in range(2):
+        out.zero_()
+        st.forward(lay(x), out=out, graph=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out, got), rep
