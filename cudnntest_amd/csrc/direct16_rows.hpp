@@ -197,6 +197,14 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             yoff[j] = (rowok && colok) ? (int)((((long)(t.n0 + dn) * g.K + k0c) * g.Ho + oh + j) * g.Wo + t.c0 + col) : -1;
+        if (ep.pool && rowok && colok) {
+            // 2x2 pooling: the wave's rows are two pooling rows (Ho is a multiple of 4), a lane pair is one pooling
+            // column (Wo is even); yoff[0], yoff[1]: the two pooled rows, this pair's column
+            const int Hq = g.Ho >> 1, Wq = g.Wo >> 1;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                yoff[j] = (int)((((long)(t.n0 + dn) * g.K + k0c) * Hq + (oh >> 1) + j) * Wq + ((t.c0 + col) >> 1));
+        }
     };
 
     floatx16 acc[2][4];
@@ -254,7 +262,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     // that each stores one 4-byte pair -- the even lane for filter r, the odd lane for filter r+1.
     // K is a multiple of 64 (the host checks), so a wave's 64 filters exist or the wave has none.  The four rows of
     // a wave exist together, so a lane stores all its values or none.
-    const unsigned kstride2 = (unsigned)(g.Ho * g.Wo) * 2u;  // bytes between the planes of two filters
+    const unsigned kstride2 = (ep.pool ? (unsigned)((g.Ho >> 1) * (g.Wo >> 1)) : (unsigned)(g.Ho * g.Wo)) * 2u;   // bytes between the planes of two filters
     const bool odd = lane & 1;
     auto stores = [&]() {
         if (k0c >= g.K || yoff[0] < 0) return;
@@ -263,6 +271,36 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         unsigned ks = kstride2;
         asm volatile("" : "+s"(ks));
         char* const yb = reinterpret_cast<char*>(y);
+        if (ep.pool) {
+            // with pooling: the maximum over the two rows in registers, over the two columns with the neighbouring lane;
+            // the even lane stores the pooled value of filter r, the odd lane that of filter r+1 (2 bytes each)
+            unsigned q[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) q[j] = (unsigned)yoff[j] * 2u + (unsigned)(4 * lh + (odd ? 1 : 0)) * ks;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int r2 = 0; r2 < 16; r2 += 2) {
+                    const int kk = 32 * i + 8 * (r2 >> 2) + 4 * lh + (r2 & 3);
+                    float b0 = 0.f, b1 = 0.f;
+                    if (ep.bias) {
+                        b0 = bias_of<T>(ep, k0c + kk);
+                        b1 = bias_of<T>(ep, k0c + kk + 1);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        float v0 = fmaxf(acc[i][2 * j][r2], acc[i][2 * j + 1][r2]) + b0;
+                        float v1 = fmaxf(acc[i][2 * j][r2 + 1], acc[i][2 * j + 1][r2 + 1]) + b1;
+                        if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
+                        v0 = fmaxf(v0, swap_lane_pairs(v0));
+                        v1 = fmaxf(v1, swap_lane_pairs(v1));
+                        *reinterpret_cast<T*>(yb + q[j]) = from_f32<T>(odd ? v1 : v0);
+                        q[j] += ((r2 & 2) ? 6u : 2u) * ks;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            return;
+        }
         unsigned o[4];                                       // byte offsets: a scalar base and a 32-bit offset per store
 #pragma unroll
         for (int j = 0; j < 4; ++j) o[j] = ((unsigned)yoff[j] - (odd ? 1u : 0u)) * 2u + (unsigned)(4 * lh + (odd ? 1 : 0)) * ks;

@@ -756,11 +756,19 @@ int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, 
 
 size_t direct16_bank_bytes(const Geometry& g) { return (size_t)9 * round_up(g.C, 32) * round_up(g.K, 128) * 2; }
 
+// whether a layer runs on the 8-wave kernel (given 4-byte aligned tensors)
+bool direct16_big(const Geometry& g, D16Geom* d) {
+    const bool plan = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, d) : direct16_rows_plan<1>(g, d);
+    return plan && (long)d->rowBlocks * d->colBlocks * d->kTiles >= device_cus() / 2;
+}
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
     D16Geom d;
-    return dtype != WINO_F32 && src == WINO_NCHW && dst == WINO_NCHW && g.C % 8 == 0 && g.W % 2 == 0 &&
-           !(flags & WINO_FLAG_POOL2) && (long)g.N * g.K * g.Ho * g.Wo < (1L << 31) &&
-           (long)g.C * g.H * g.W * 2 * 8 < (1L << 32) && direct16_plan(g, 4, false, &d);
+    if (!(dtype != WINO_F32 && src == WINO_NCHW && dst == WINO_NCHW && g.C % 8 == 0 && g.W % 2 == 0 &&
+          (long)g.N * g.K * g.Ho * g.Wo < (1L << 31) && (long)g.C * g.H * g.W * 2 * 8 < (1L << 32) &&
+          direct16_plan(g, 4, false, &d)))
+        return false;
+    // 2x2 pooling lives in the stores of the 8-wave kernel only
+    return !(flags & WINO_FLAG_POOL2) || direct16_big(g, &d);
 }
 
 template <typename T, int NPG, bool ROWS>
@@ -793,8 +801,9 @@ int launch_direct16(int dtype, unsigned flags, const void* bias, const Geometry&
     // large layers: the 8-wave kernel, one workgroup per CU; else tiles of 512 pixels, fewer pixels when that leaves
     // the chip short of tiles
     int npg = 4, wf = direct16_rows_wf(g);
-    const bool big = !misaligned(y, 4) && (wf == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d)) &&
-               (long)d.rowBlocks * d.colBlocks * d.kTiles >= device_cus() / 2;
+    const bool pool = (flags & WINO_FLAG_POOL2) != 0;        // (pooled values are stored one by one: no alignment asked of y)
+    const bool big = (pool || !misaligned(y, 4)) && direct16_big(g, &d);
+    if (pool && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: pooling needs the 8-wave kernel's layer shapes");
     const bool rows = !big && direct16_plan(g, 4, true, &d) && (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
     if (!big && !rows) {
         for (; npg > 1; npg >>= 1) {
@@ -965,7 +974,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         }
         if (!direct16_ok(src, dst, dtype, flags, g))
             return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for C <= 4, and for 2-byte NCHW tensors with "
-                                              "C a multiple of 8 and an even width; no pooling");
+                                              "C a multiple of 8 and an even width (pooling: output height a multiple of 4, K a multiple of 64, a large layer)");
         void* base = nullptr;
         const int rcb = ss.get(kCounterBytes + direct16_bank_bytes(g), &base);
         if (rcb) return rcb;
@@ -1479,7 +1488,7 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
         if (L.U4) {
             rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, WINO_ALGO_STAGED_F4, L.flags, s->N, L.C, L.K, L.H,
                            L.W, 1, in, nullptr, L.U4, bias, out, stream);
-        } else if (L.W9 && !misaligned(in, 4) && !misaligned(out, 4) &&
+        } else if (L.W9 && !misaligned(in, 4) && (!misaligned(out, 4) || (L.flags & WINO_FLAG_POOL2)) &&
                    auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in)) {
             // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
@@ -1548,8 +1557,7 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
         // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte NCHW layers)
-        const bool direct16_layer = dtype != WINO_F32 && L.layout_in == WINO_NCHW && L.layout_out == WINO_NCHW &&
-                                    L.C % 8 == 0 && !(L.flags & WINO_FLAG_POOL2);
+        const bool direct16_layer = dtype != WINO_F32 && L.layout_in == WINO_NCHW && L.layout_out == WINO_NCHW && L.C % 8 == 0;
         if (e == hipSuccess && (L.C <= 4 || direct16_layer)) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         // what AUTO runs outside the F(2x2) kernels gets its filters prepared once as well
         if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && auto_f4(dtype, g)) {

@@ -71,7 +71,9 @@ typedef enum {
                                direct product by nothing but the multiplies (the stage it replaces is
                                comparison/GEMM.cuh:124-253; the reference's own direct kernel in tile geometry is
                                Conv_fuse, fusedTest/winotrans.cuh:1868).
-                               Bias and ReLU, no pooling; needs the filter bank itself (not wino_conv_prepared).
+                               Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (output
+                               height a multiple of 4, K a multiple of 64, at least a tile for every other CU), not
+                               for C <= 4; needs the filter bank itself (not wino_conv_prepared).
                                What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW layers. */
 } wino_algo_t;
 

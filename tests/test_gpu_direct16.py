@@ -39,7 +39,8 @@ def test_integers_round_once(oracle, shape, dtype):
 #   * 64-filter tiles (K = 64), 200 columns in a block of 256, a last stage whose second channel vector lies past C;
 #   * K = 192 (64-filter tiles, three of them), no padding, blocks of 8 rows x 128 columns;
 #   * 12-row images under blocks of 16 rows: a block spans three images;
-#   * two column blocks, the second one half empty.
+#   * two column blocks, the second one half empty (this one stays on the 4-wave kernel: its block does not fit the
+#     8-wave kernel's LDS plane).
 BIG_SHAPES = [(32, 64, 128, 112, 112, 1), (16, 24, 64, 64, 200, 1), (12, 16, 192, 66, 130, 0), (192, 16, 256, 12, 24, 1),
               (16, 32, 128, 32, 160, 1)]
 
@@ -64,6 +65,19 @@ def test_integers_round_once_one_tile_per_cu_and_more(oracle, shape, dtype):
         for n in (0, N - 1):
             want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], pad) + bias[ks][None, :, None, None], 0)
             assert np.array_equal(host(got[n:n + 1][:, ks]), rounded(want.astype(np.float32), dtype, oracle)), (rep, n)
+    # 2x2 max pooling in the kernel's stores: the maximum of values that are rounded afterwards is the maximum of the
+    # rounded values (rounding is monotonic), so the pooled tensor is the pooling of the unpooled one, bit for bit
+    Ho, Wo = got.shape[2], got.shape[3]
+    if shape == BIG_SHAPES[4]:
+        # (130 columns of a 128-filter block x 6 rows do not fit the 8-wave kernel's LDS plane: this layer runs on the
+        # 4-wave kernel, which has no pooling)
+        with pytest.raises(_lib.WinoError):
+            ops.conv(xd, wd, pad, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+        return
+    pooled = ops.conv(xd, wd, pad, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+    assert tuple(pooled.shape) == (N, K, Ho // 2, Wo // 2)
+    assert torch.equal(pooled, torch.nn.functional.max_pool2d(got.float(), 2).to(got.dtype))
+    assert torch.equal(pooled, ops.conv(xd, wd, pad, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True))
 
 
 @pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
