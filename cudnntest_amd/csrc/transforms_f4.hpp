@@ -92,12 +92,9 @@ __device__ __forceinline__ void output_tile_transform_f4(const float m[36], floa
 // The CV channels of a vector one after the other (36 live values each), their results gathered into one
 // 16-byte store per coordinate: a wave writes 1 KB runs of U.
 template <typename T>
-__global__ __launch_bounds__(64) void filter_transform_f4_kernel(const T* __restrict__ w, T* __restrict__ U,
-                                                                  FltStrides s, int K, int C, int Kp, int Cp) {
+__device__ __forceinline__ void filter_transform_f4_thread(const T* __restrict__ w, T* __restrict__ U, const FltStrides& s, int K,
+                                                           int C, int Kp, int Cp, int k, int cq) {
     constexpr int CV = ChanVec<T>::n;
-    const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    const int cq = blockIdx.y;
-    if (k >= Kp) return;
     T out[36][CV];
 #pragma unroll
     for (int e = 0; e < CV; ++e) {
@@ -128,6 +125,25 @@ __global__ __launch_bounds__(64) void filter_transform_f4_kernel(const T* __rest
     }
 }
 
+template <typename T>
+__global__ __launch_bounds__(64) void filter_transform_f4_kernel(const T* __restrict__ w, T* __restrict__ U,
+                                                                  FltStrides s, int K, int C, int Kp, int Cp) {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k < Kp) filter_transform_f4_thread<T>(w, U, s, K, C, Kp, Cp, k, blockIdx.y);
+}
+
+// A whole-layer call gives the filter bank's transform to the input transform's launch (the FilterJob of the
+// F(2x2) kernels): one more z-slice of its grid -- slice 0, which is dispatched first, so the job runs beside the
+// input's workgroups and not after them -- whose workgroups share the Kp x Cp/CV threads of the job, filters
+// fastest, and leave at once when there is none left for them.
+template <typename T>
+__device__ __forceinline__ void filter_job_f4(const FilterJob& fj) {
+    constexpr int CV = ChanVec<T>::n;
+    const long id = ((long)blockIdx.y * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= (long)fj.Kp * (fj.Cp / CV)) return;
+    filter_transform_f4_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, (int)(id % fj.Kp), (int)(id / fj.Kp));
+}
+
 // ---- input transform, layout-generic -------------------------------------------------------
 // Thread per (channel-in-vector e, tile p, channel vector cq) with e fastest: the CV lanes of
 // one tile write the CV elements of one 16-byte vector, so a wave's store is one contiguous
@@ -137,8 +153,12 @@ template <typename T>
 __global__ __launch_bounds__(256) void input_transform_f4_generic_kernel(const T* __restrict__ x, T* __restrict__ V,
                                                                           ActStrides s, int N, int C, int H, int W,
                                                                           int pad, int th, int tw, long P, long Pp,
-                                                                          int Cp, int order) {
+                                                                          int Cp, int order, FilterJob fj) {
     constexpr int CV = ChanVec<T>::n;
+    if (gridDim.z == 2 && blockIdx.z == 0) {                 // dispatched first: the job runs under the input's workgroups
+        filter_job_f4<T>(fj);
+        return;
+    }
     const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const int e = (int)(gid % CV);
     const long p = gid / CV;
@@ -184,11 +204,16 @@ __global__ __launch_bounds__(256) void input_transform_f4_generic_kernel(const T
 constexpr int F4N_CC = 32, F4N_PITCH = 33, F4N_TCB = 14;
 __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const float* __restrict__ x, float* __restrict__ V,
                                                                        int N, int C, int H, int W, int pad, int th,
-                                                                       int tw, long Pp, int Cp, int colBlocks) {
+                                                                       int tw, long Pp, int Cp, int colBlocks, FilterJob fj) {
     __shared__ float sm[6 * (4 * F4N_TCB + 2) * F4N_PITCH];
+    const int zjob = gridDim.z - N;                          // 1 with a filter job: slice 0, dispatched first
+    if (zjob && blockIdx.z == 0) {
+        filter_job_f4<float>(fj);
+        return;
+    }
     const int tid = threadIdx.x;
     const int ty = blockIdx.x / colBlocks, cb = blockIdx.x - ty * colBlocks;
-    const int c0 = blockIdx.y * F4N_CC, n = blockIdx.z;
+    const int c0 = blockIdx.y * F4N_CC, n = blockIdx.z - zjob;
     const int tx0 = cb * F4N_TCB, ntx = min(F4N_TCB, tw - tx0);
     const int wlb = 4 * ntx + 2;                             // pixel columns of the block
     const int h0 = 4 * ty - pad, w0 = 4 * tx0 - pad;

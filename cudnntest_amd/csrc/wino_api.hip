@@ -543,21 +543,37 @@ int launch_f4_filter(int layout, int K, int C, int Kp, int Cp, const void* w, vo
     return WINO_OK;
 }
 
+// fj: a filter job to ride in the launch (its w is null for none).  Its threads are Kp x Cp/CV; the extra z-slice of
+// the grid has at least that many (the input side has P x Cp/CV x CV or more), or the job gets a launch of its own.
 template <typename T>
-int launch_f4_input(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st) {
+int launch_f4_input(int layout, int order, const Geometry& g, const void* x, void* V, hipStream_t st,
+                    const FilterJob& fj = FilterJob{}) {
     constexpr int CV = ChanVec<T>::n;
-    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && sizeof(T) == 4 && g.N <= 65535 && g.Cp / F4N_CC < 65535) {
+    const long job = fj.w ? (long)fj.Kp * (fj.Cp / CV) : 0;
+    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && sizeof(T) == 4 && g.N < 65535 && g.Cp / F4N_CC < 65535) {
         const int colBlocks = (g.tw + F4N_TCB - 1) / F4N_TCB;
         dim3 grid((unsigned)(g.th * colBlocks), (g.Cp + F4N_CC - 1) / F4N_CC, g.N);
+        const bool ride = job > 0 && (long)grid.x * grid.y * 256 >= job;
+        if (job > 0 && !ride) {
+            const int rc = launch_f4_filter<T>(layout, fj.K, fj.C, fj.Kp, fj.Cp, fj.w, fj.U, st);
+            if (rc) return rc;
+        }
+        if (ride) grid.z += 1;
         hipLaunchKernelGGL(input_transform_f4_nhwc_kernel, grid, dim3(256), 0, st, (const float*)x, (float*)V, g.N, g.C, g.H, g.W,
-                           g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks);
+                           g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, ride ? fj : FilterJob{});
         LAUNCH_CHECK("f4_input_transform_nhwc");
         return WINO_OK;
     }
     dim3 grid((unsigned)((g.P * CV + 255) / 256), g.Cp / CV), block(256);
+    const bool ride = job > 0 && (long)grid.x * grid.y * 256 >= job;
+    if (job > 0 && !ride) {
+        const int rc = launch_f4_filter<T>(layout, fj.K, fj.C, fj.Kp, fj.Cp, fj.w, fj.U, st);
+        if (rc) return rc;
+    }
+    if (ride) grid.z = 2;
     hipLaunchKernelGGL(input_transform_f4_generic_kernel<T>, grid, block, 0, st, (const T*)x, (T*)V,
                        act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp,
-                       g.Cp, order);
+                       g.Cp, order, ride ? fj : FilterJob{});
     LAUNCH_CHECK("f4_input_transform");
     return WINO_OK;
 }
@@ -925,16 +941,19 @@ int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned 
     float* Mo = (float*)(b + sc.m_off);
     const int order = tile_order_for(src, dst);
     const int porder = dst == WINO_NHWC ? WINO_PRODUCT_PK : WINO_PRODUCT_KP;
+    // the filter transform rides in the input transform's launch, unless the stages are being timed one by one
+    const bool ride = !Upre && !g_timing;
     if (Upre) {
         U = const_cast<void*>(Upre);
-    } else {
+    } else if (!ride) {
         StageScope t(WINO_STAGE_FILTER, st);
         rc = wino_f4_filter_transform(src, dtype, K, C, w, U, stream);
         if (rc) return rc;
     }
     {
         StageScope t(WINO_STAGE_INPUT, st);
-        rc = wino_f4_input_transform(src, dtype, order, N, C, H, W, pad, x, V, stream);
+        const FilterJob fj = ride ? FilterJob{w, U, flt_strides(src, K, C), K, C, g.Kp, g.Cp} : FilterJob{};
+        DISPATCH_DTYPE_RC(rc, dtype, launch_f4_input<T>(src, order, g, x, V, st, fj));
         if (rc) return rc;
     }
     {
