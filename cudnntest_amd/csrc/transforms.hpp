@@ -69,12 +69,11 @@ __device__ __forceinline__ void output_tile_transform(const float m[16], float& 
 // is a 16-byte vector and a wave's stores are contiguous.  The grid covers the
 // padded (Cp/CV) x Kp rectangle and the padding is written as zeros, which is
 // what lets the GEMM run without masks on the reduction dimension.
+// The 3x3 taps of filter k for the CV channels of vector cq, as fp32; zeros where the filter or a channel does not exist.
 template <typename T>
-__device__ __forceinline__ void filter_transform_thread(const T* __restrict__ w, T* __restrict__ U, FltStrides s,
-                                                        int K, int C, int Kp, int Cp, int k, int cq) {
+__device__ __forceinline__ void filter_taps_load(const T* __restrict__ w, const FltStrides& s, int K, int C, int k, int cq,
+                                                 float (&g)[ChanVec<T>::n][3][3]) {
     constexpr int CV = ChanVec<T>::n;
-    float u[CV][16];
-    float g[CV][3][3];
     // all CV channels of this vector exist, and the filter bank allows 16-byte loads
     const bool full = k < K && (cq + 1) * CV <= C && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
     if (full && s.c == 9 && s.s == 1 && (C * 9) % CV == 0) {
@@ -118,6 +117,15 @@ __device__ __forceinline__ void filter_transform_thread(const T* __restrict__ w,
             for (int t = 0; t < 9; ++t) g[e][t / 3][t % 3] = mask_keep(to_f32(raw[e][t]), m);
         }
     }
+}
+
+template <typename T>
+__device__ __forceinline__ void filter_transform_thread(const T* __restrict__ w, T* __restrict__ U, FltStrides s,
+                                                        int K, int C, int Kp, int Cp, int k, int cq) {
+    constexpr int CV = ChanVec<T>::n;
+    float u[CV][16];
+    float g[CV][3][3];
+    filter_taps_load<T>(w, s, K, C, k, cq, g);
 #pragma unroll
     for (int e = 0; e < CV; ++e) filter_tile_transform(g[e], u[e]);
     const size_t plane = (size_t)Cp * Kp;   // elements per coordinate
@@ -298,7 +306,15 @@ __device__ __forceinline__ void tile_from_lds_store(const T* base, int per_ch, i
     }
 }
 
-template <typename T, int VEC>
+// the F(4x4,3x3) pieces the tiled NCHW kernel uses with M = 4 (transforms_f4.hpp)
+template <typename T>
+__device__ __forceinline__ void filter_transform_f4_thread(const T* __restrict__ w, T* __restrict__ U, const FltStrides& s, int K,
+                                                           int C, int Kp, int Cp, int k, int cq);
+__device__ __forceinline__ void tile_from_lds_store_f4(const float* base, int per_ch, int ldsW, float* vp, size_t plane);
+
+// M = 2: F(2x2,3x3) tiles, 4x4 pixels every 2.  M = 4: F(4x4,3x3) tiles, 6x6 pixels every 4 (fp32 only); the halo
+// copy is the same code, the filter job and the tile arithmetic are the F(4x4) ones.
+template <typename T, int VEC, int M = 2>
 __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __restrict__ x, T* __restrict__ V, int N,
                                                                    int C, int H, int W, int pad, int th, int tw,
                                                                    long Pp, int Cp, int TR, int TC, int colBlocks,
@@ -308,16 +324,18 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     T* in_smem = reinterpret_cast<T*>(in_smem_raw);   // [CV][rows][ldsW], the storage type
     if (fj.w && blockIdx.z == 0) {
         // the first z-slice transforms the filter bank: channel vector blockIdx.y (the layer's C), filters strided
-        for (int k = blockIdx.x * 256 + threadIdx.x; k < fj.Kp; k += gridDim.x * 256)
-            filter_transform_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, k, blockIdx.y);
+        for (int k = blockIdx.x * 256 + threadIdx.x; k < fj.Kp; k += gridDim.x * 256) {
+            if constexpr (M == 4) filter_transform_f4_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, k, blockIdx.y);
+            else filter_transform_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, k, blockIdx.y);
+        }
         return;
     }
     const int cq = blockIdx.y, n = fj.w ? blockIdx.z - 1 : blockIdx.z;
     const int rb = blockIdx.x / colBlocks, cb = blockIdx.x % colBlocks;
     const int ty0 = rb * TR, tx0 = cb * TC;
-    const int rows = 2 * TR + 2;
-    const int ldsW = 2 * TC + 2;          // even
-    const int h0 = 2 * ty0 - pad, w0 = 2 * tx0 - pad;
+    const int rows = M * TR + 2;
+    const int ldsW = M * TC + 2;          // even
+    const int h0 = M * ty0 - pad, w0 = M * tx0 - pad;
     const int tid = threadIdx.x;
 
     const int per_ch = rows * ldsW;
@@ -392,7 +410,13 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
     const long p = ((long)n * th + ty) * tw + tx;
     const size_t plane = (size_t)Cp * Pp;
     T* vp = V + ((size_t)cq * Pp + p) * CV;
-    tile_from_lds_store<T>(in_smem + (2 * tr) * ldsW + 2 * tc, per_ch, ldsW, vp, plane);
+    if constexpr (M == 4) {
+        static_assert(M != 4 || sizeof(T) == 4, "the F(4x4) tiles of this kernel are fp32");
+        tile_from_lds_store_f4(reinterpret_cast<const float*>(in_smem) + (4 * tr) * ldsW + 4 * tc, per_ch, ldsW,
+                               reinterpret_cast<float*>(vp), plane);
+    } else {
+        tile_from_lds_store<T>(in_smem + (2 * tr) * ldsW + 2 * tc, per_ch, ldsW, vp, plane);
+    }
 }
 
 // ---- input transform, NCHW source, small images -------------------------------------
@@ -402,8 +426,8 @@ __global__ __launch_bounds__(256) void input_transform_nchw_kernel(const T* __re
 // and scattered into LDS planes [ch][2*th+2][2*tw+2] whose zero padding was written beforehand; thread
 // (channel vector, tile) then builds its tile as in the tiled kernel.  A thread walks the run 256 words at a
 // time; (stepC, stepH, stepW) is that stride split into planes, rows and words by the host, so the position of a
-// word costs two compares instead of two divisions.
-template <typename T, int VEC>
+// word costs two compares instead of two divisions.  M as in the tiled kernel.
+template <typename T, int VEC, int M = 2>
 __global__ __launch_bounds__(256) void input_transform_nchw_small_kernel(const T* __restrict__ x, T* __restrict__ V,
                                                                          int C, int H, int W, int pad, int th, int tw,
                                                                          long Pp, int Cp, int NQ, int groups,
@@ -412,7 +436,18 @@ __global__ __launch_bounds__(256) void input_transform_nchw_small_kernel(const T
     constexpr int CV = ChanVec<T>::n;
     constexpr int NB = 8;                              // loads in flight per thread
     extern __shared__ __attribute__((aligned(16))) unsigned char in_smem_raw[];
-    if (fj.w && (int)blockIdx.x >= in_blocks) {
+    int bid = blockIdx.x;
+    if constexpr (M == 4) {
+        // the filter job's workgroups come first: they run beside the input's, not after them
+        const int job_blocks = gridDim.x - in_blocks;
+        if (bid < job_blocks) {
+            const long id = (long)bid * 256 + threadIdx.x;
+            if (id < (long)fj.Kp * (fj.Cp / CV))
+                filter_transform_f4_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, (int)(id % fj.Kp), (int)(id / fj.Kp));
+            return;
+        }
+        bid -= job_blocks;
+    } else if (fj.w && bid >= in_blocks) {
         filter_job_blocks<T, 256>(fj, in_blocks);
         return;
     }
@@ -421,11 +456,11 @@ __global__ __launch_bounds__(256) void input_transform_nchw_small_kernel(const T
     T* in_smem = reinterpret_cast<T*>(in_smem_raw);
     elem_t* smem_bits = reinterpret_cast<elem_t*>(in_smem_raw);
     const int tid = threadIdx.x;
-    const int n = blockIdx.x / groups, cq0 = (blockIdx.x - n * groups) * NQ;
+    const int n = bid / groups, cq0 = (bid - n * groups) * NQ;
     const int nq = min(NQ, Cp / CV - cq0);             // channel vectors of this workgroup
     const int c0 = cq0 * CV;
     const int nch = max(min(nq * CV, C - c0), 0);      // channels that exist; the others stay zero
-    const int rows = 2 * th + 2, ldsW = 2 * tw + 2, per_ch = rows * ldsW;
+    const int rows = M * th + 2, ldsW = M * tw + 2, per_ch = rows * ldsW;
     const int Ww = W / VEC;
     const int words = nch * H * Ww;
     const raw_t* xw = reinterpret_cast<const raw_t*>(x + ((size_t)n * C + c0) * H * W);
@@ -474,7 +509,13 @@ __global__ __launch_bounds__(256) void input_transform_nchw_small_kernel(const T
     const int ty = t / tw, tx = t - ty * tw;
     const long p = (long)n * tiles + t;
     T* vp = V + ((size_t)(cq0 + q) * Pp + p) * CV;
-    tile_from_lds_store<T>(in_smem + q * CV * per_ch + (2 * ty) * ldsW + 2 * tx, per_ch, ldsW, vp, (size_t)Cp * Pp);
+    if constexpr (M == 4) {
+        static_assert(M != 4 || sizeof(T) == 4, "the F(4x4) tiles of this kernel are fp32");
+        tile_from_lds_store_f4(reinterpret_cast<const float*>(in_smem) + q * CV * per_ch + (4 * ty) * ldsW + 4 * tx, per_ch, ldsW,
+                               reinterpret_cast<float*>(vp), (size_t)Cp * Pp);
+    } else {
+        tile_from_lds_store<T>(in_smem + q * CV * per_ch + (2 * ty) * ldsW + 2 * tx, per_ch, ldsW, vp, (size_t)Cp * Pp);
+    }
 }
 
 // ---- input transform, NHWC source, LDS-transposed ---------------------------------------

@@ -96,22 +96,12 @@ __device__ __forceinline__ void filter_transform_f4_thread(const T* __restrict__
                                                            int C, int Kp, int Cp, int k, int cq) {
     constexpr int CV = ChanVec<T>::n;
     T out[36][CV];
+    float g[CV][3][3];
+    filter_taps_load<T>(w, s, K, C, k, cq, g);                // 16-byte loads where the bank's layout has them
 #pragma unroll
     for (int e = 0; e < CV; ++e) {
-        const int c = cq * CV + e;
         float u[36];
-        if (k < K && c < C) {
-            float g[3][3];
-            const T* wp = w + k * s.k + c * s.c;
-#pragma unroll
-            for (int r = 0; r < 3; ++r)
-#pragma unroll
-                for (int q = 0; q < 3; ++q) g[r][q] = to_f32(wp[r * s.r + q * s.s]);
-            filter_tile_transform_f4(g, u);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 36; ++i) u[i] = 0.f;
-        }
+        filter_tile_transform_f4(g[e], u);
 #pragma unroll
         for (int xi = 0; xi < 36; ++xi) out[xi][e] = from_f32<T>(u[xi]);
     }
@@ -142,6 +132,29 @@ __device__ __forceinline__ void filter_job_f4(const FilterJob& fj) {
     const long id = ((long)blockIdx.y * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= (long)fj.Kp * (fj.Cp / CV)) return;
     filter_transform_f4_thread<T>((const T*)fj.w, (T*)fj.U, fj.s, fj.K, fj.C, fj.Kp, fj.Cp, (int)(id % fj.Kp), (int)(id / fj.Kp));
+}
+
+// ---- input transform, fp32 NCHW source: the tiled kernel of transforms.hpp with M = 4 ------------------------------
+// Its second phase: the 6x6 pixels of one tile for the 4 channels of a vector, from LDS planes [ch][rows][ldsW]
+// (`base`: the tile's first pixel in the first plane, at an even column: 8-byte reads), to 36 vectors of V.
+__device__ __forceinline__ void tile_from_lds_store_f4(const float* base, int per_ch, int ldsW, float* vp, size_t plane) {
+    float v[4][36];
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch) {
+        float d[6][6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const float2 a = *reinterpret_cast<const float2*>(base + ch * per_ch + i * ldsW + 2 * j);
+                d[i][2 * j] = a.x;
+                d[i][2 * j + 1] = a.y;
+            }
+        input_tile_transform_f4(d, v[ch]);
+    }
+#pragma unroll
+    for (int xi = 0; xi < 36; ++xi)
+        *reinterpret_cast<float4*>(vp + xi * plane) = make_float4(v[0][xi], v[1][xi], v[2][xi], v[3][xi]);
 }
 
 // ---- input transform, layout-generic -------------------------------------------------------

@@ -564,6 +564,42 @@ int launch_f4_input(int layout, int order, const Geometry& g, const void* x, voi
         LAUNCH_CHECK("f4_input_transform_nhwc");
         return WINO_OK;
     }
+    if constexpr (sizeof(T) == 4) {
+        // NCHW rows with at least 128 tiles to an image: TR x TC tiles per workgroup through an LDS halo of 4 channels
+        // (<= 64 KB), the tiled kernel of the F(2x2) pipeline with 6x6 tiles every 4 pixels
+        if (layout == WINO_NCHW && order == WINO_TILES_BATCH_MAJOR && g.th * g.tw >= 128 && g.tw <= 252 && g.N < 65535) {
+            const int TC = g.tw < 64 ? g.tw : 64;
+            int TR = std::min(256 / TC, g.th);
+            while (TR > 1 && (size_t)CV * (4 * TR + 2) * (4 * TC + 2) * 4 > 65536) --TR;
+            const int colBlocks = (g.tw + TC - 1) / TC, rowBlocks = (g.th + TR - 1) / TR;
+            const int ldsW = 4 * TC + 2;
+            int chunkLog2 = 0;
+            while ((64 << chunkLog2) < ldsW) ++chunkLog2;
+            const size_t lds = (size_t)CV * (4 * TR + 2) * ldsW * 4;
+            dim3 grid(rowBlocks * colBlocks, g.Cp / CV, g.N + (job ? 1 : 0));
+            hipLaunchKernelGGL((input_transform_nchw_kernel<float, 1, 4>), grid, dim3(256), lds, st, (const float*)x, (float*)V,
+                               g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, TR, TC, colBlocks, chunkLog2, fj);
+            LAUNCH_CHECK("f4_input_transform_nchw");
+            return WINO_OK;
+        }
+        // smaller images: one image and NQ channel vectors per workgroup (LDS planes of 4 NQ channels, <= 64 KB)
+        if (layout == WINO_NCHW && order == WINO_TILES_BATCH_MAJOR && g.th * g.tw < 128) {
+            const int tiles = g.th * g.tw, CQ = g.Cp / CV;
+            const int plane = (4 * g.th + 2) * (4 * g.tw + 2) * CV * 4;          // bytes of a channel vector's planes
+            const int NQ = std::max(1, std::min(std::min(256 / tiles, 65536 / plane), CQ));
+            const int groups = (CQ + NQ - 1) / NQ;
+            const long in_blocks = (long)g.N * groups, extra = (job + 255) / 256;
+            if (in_blocks + extra < (1L << 31) && (size_t)NQ * plane <= 65536) {
+                const int stepC = 256 / (g.H * g.W), stepH = (256 - stepC * g.H * g.W) / g.W,
+                          stepW = 256 - stepC * g.H * g.W - stepH * g.W;
+                hipLaunchKernelGGL((input_transform_nchw_small_kernel<float, 1, 4>), dim3((unsigned)(in_blocks + extra)), dim3(256),
+                                   (size_t)NQ * plane, st, (const float*)x, (float*)V, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp,
+                                   NQ, groups, (int)in_blocks, stepC, stepH, stepW, fj);
+                LAUNCH_CHECK("f4_input_transform_nchw_small");
+                return WINO_OK;
+            }
+        }
+    }
     dim3 grid((unsigned)((g.P * CV + 255) / 256), g.Cp / CV), block(256);
     const bool ride = job > 0 && (long)grid.x * grid.y * 256 >= job;
     if (job > 0 && !ride) {
