@@ -117,9 +117,12 @@ struct Geometry {
 
 __host__ inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
 
+// Zero padding beyond one row/column is honoured arithmetically, like the reference does
+// (comparison/wrapedConv_NCHW.cuh:346-362), by the layout-generic transforms of the staged pipelines.
+constexpr int kMaxPad = 1024;
 __host__ inline bool make_geometry(int dtype, int N, int C, int K, int H, int W, int pad, Geometry* g, int m = 2) {
     g->m = m;
-    if (N <= 0 || C <= 0 || K <= 0 || H <= 0 || W <= 0 || pad < 0 || pad > 1) return false;
+    if (N <= 0 || C <= 0 || K <= 0 || H <= 0 || W <= 0 || pad < 0 || pad > kMaxPad) return false;
     g->N = N; g->C = C; g->K = K; g->H = H; g->W = W; g->pad = pad;
     g->Ho = H + 2 * pad - 2;
     g->Wo = W + 2 * pad - 2;

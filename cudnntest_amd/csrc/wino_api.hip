@@ -665,7 +665,7 @@ int tile_order_for(int src, int /*dst*/) {
 // Winograd path
 bool direct_ok(int dst, unsigned flags, const Geometry& g) {
     const size_t lds = direct_lds_bytes(g.C, g.K);
-    return lds != 0 && lds <= 64 * 1024 && !(flags & WINO_FLAG_POOL2) &&
+    return lds != 0 && lds <= 64 * 1024 && !(flags & WINO_FLAG_POOL2) && g.pad <= 1 &&
            (long)g.N * g.C * g.H * g.W < (1L << 30) && (long)g.N * g.K * g.Ho * g.Wo < (1L << 30);   // 32-bit byte offsets
 }
 
@@ -815,7 +815,7 @@ bool direct16_big(const Geometry& g, D16Geom* d) {
 }
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
     D16Geom d;
-    if (!(dtype != WINO_F32 && src == WINO_NCHW && dst == WINO_NCHW && g.C % 8 == 0 && g.W % 2 == 0 &&
+    if (!(dtype != WINO_F32 && src == WINO_NCHW && dst == WINO_NCHW && g.C % 8 == 0 && g.W % 2 == 0 && g.pad <= 1 &&
           (long)g.N * g.K * g.Ho * g.Wo < (1L << 31) && (long)g.C * g.H * g.W * 2 * 8 < (1L << 32) &&
           direct16_plan(g, 4, false, &d)))
         return false;
@@ -958,7 +958,8 @@ int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g,
     if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x)) return WINO_ALGO_DIRECT;
     if (have_w && auto_f4(dtype, g)) return WINO_ALGO_STAGED_F4;
-    return pick_algo(src, dtype, g);
+    const int algo = pick_algo(src, dtype, g);
+    return algo == WINO_ALGO_FUSED && g.pad > 1 ? WINO_ALGO_EPILOGUE : algo;   // the single kernel masks one ring of padding
 }
 
 int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned flags, const void* bias, int N, int C, int K,
@@ -1028,7 +1029,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
             return launch_direct(src, dst, dtype, flags, bias, g, x, w, y, (hipStream_t)stream);
         }
         if (!direct16_ok(src, dst, dtype, flags, g))
-            return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for C <= 4, and for 2-byte NCHW tensors with "
+            return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for pad 0 and 1: for C <= 4, and for 2-byte NCHW tensors with "
                                               "C a multiple of 8 and an even width (pooling: output height a multiple of 4, K a multiple of 64, a large layer)");
         void* base = nullptr;
         const int rcb = ss.get(kCounterBytes + direct16_bank_bytes(g), &base);
@@ -1060,6 +1061,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (rc) return rc;
     }
     if (algo == WINO_ALGO_FUSED) {
+        if (g.pad > 1) return fail(WINO_ERR_UNSUPPORTED, "the single-kernel path is built for pad 0 and 1 (pad=%d)", g.pad);
         StageScope t(WINO_STAGE_GEMM, st);
         return launch_fused(src, dst, dtype, order, flags, bias, g, x, U, y, st);
     }

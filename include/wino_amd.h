@@ -14,6 +14,10 @@
  *   CHWN     [C][H][W][N]                [C][3][3][K]   comparison/wrapedConv_CHWN.cuh:288
  * The convolution is a stride-1 cross-correlation with `pad` rows/columns of
  * zeros on every side; the output is Ho x Wo = (H+2*pad-2) x (W+2*pad-2).
+ * pad is 0 .. 1024 (the reference takes it arithmetically,
+ * comparison/wrapedConv_NCHW.cuh:346-362, and its drivers pass 1).  The staged
+ * and epilogue pipelines and WINO_ALGO_AUTO take any of these; WINO_ALGO_FUSED and
+ * WINO_ALGO_DIRECT are built for 0 and 1 and answer WINO_ERR_UNSUPPORTED beyond.
  *
  * Alignment: x, w, bias and y need only the alignment of their element type (any
  * view of a device allocation works).  The Winograd-domain operands U, V and the

@@ -25,7 +25,7 @@ def torch_conv(x_nchw, w_kcrs, pad):
 
 
 @pytest.mark.parametrize("shape", SHAPES)
-@pytest.mark.parametrize("pad", [0, 1])
+@pytest.mark.parametrize("pad", [0, 1, 2, 3])
 def test_direct_vs_library_all_layout_pairs(oracle, shape, pad):
     N, C, K, H, W = shape
     if pad == 0 and min(H, W) < 3:

@@ -230,3 +230,21 @@ def test_tile_geometry(oracle):
     assert oracle.wino_tiles(4, 22, 22, 1) == (6, 6)
     assert oracle.wino_tiles(4, 224, 224, 1) == (56, 56)
     assert oracle.wino_tiles(4, 14, 14, 1) == (4, 4)
+
+
+@pytest.mark.parametrize("m", [2, 4])
+@pytest.mark.parametrize("pad", [2, 3, 5])
+def test_wide_padding_is_a_padded_image(oracle, m, pad):
+    """The reference takes `padding` arithmetically (comparison/wrapedConv_NCHW.cuh:346-362): a transform with padding
+    p is the transform without padding of the image with p rings of zeros around it, and the whole Winograd
+    convolution is the direct one."""
+    N, C, K, H, W = 2, 3, 4, 6, 5
+    x = synth.small_ints(N * C * H * W, 40 + pad).reshape(N, C, H, W)
+    xp = np.pad(x, [(0, 0), (0, 0), (pad, pad), (pad, pad)])
+    assert oracle.wino_tiles(m, H, W, pad) == oracle.wino_tiles(m, H + 2 * pad, W + 2 * pad, 0)
+    for layout in LAYOUTS:
+        got = oracle.wino_input_transform(synth.act_to_layout(x, layout), pad, layout, m=m)
+        assert np.array_equal(got, oracle.wino_input_transform(synth.act_to_layout(xp, layout), 0, layout, m=m))
+    w = synth.small_ints(K * C * 9, 41 + pad).reshape(K, C, 3, 3) * (576 if m == 4 else 1)
+    assert np.array_equal(oracle.wino_conv(x, w, pad, m=m), oracle.direct_conv(x, w, pad))
+    assert np.array_equal(oracle.direct_conv(x, w, pad), oracle.direct_conv(xp, w, 0))
