@@ -64,10 +64,11 @@ def test_invalid_arguments_are_rejected_without_a_gpu():
     assert L.wino_conv(7, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1, one, one, one, None) == -1
     assert L.wino_conv(0, 0, 9, 0, 0, 1, 1, 1, 4, 4, 1, one, one, one, None) == -1
     assert L.wino_conv(0, 0, 0, 12, 0, 1, 1, 1, 4, 4, 1, one, one, one, None) == -1
-    # bad shapes: zero batch, image too small for pad 0, unsupported pad
+    # bad shapes: zero batch, image too small for pad 0, negative and absurd pad
     assert L.wino_conv(0, 0, 0, 0, 0, 0, 1, 1, 4, 4, 1, one, one, one, None) == -1
     assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 2, 2, 0, one, one, one, None) == -1
-    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 2, one, one, one, None) == -1
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, -1, one, one, one, None) == -1
+    assert L.wino_conv(0, 0, 0, 0, 0, 1, 1, 1, 4, 4, 1025, one, one, one, None) == -1
     assert b"bad shape" in L.wino_last_error()
     assert L.wino_filter_transform(0, 0, 0, 4, one, one, None) == -1
     assert L.wino_input_transform(0, 0, 5, 1, 1, 4, 4, 1, one, one, None) == -1
