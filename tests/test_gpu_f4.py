@@ -33,7 +33,12 @@ def test_f4_filter_transform(oracle, layout, K, C):
 @pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("order", [ops.TILES_BATCH_MAJOR, ops.TILES_BATCH_MINOR])
 @pytest.mark.parametrize("shape,pad", [((2, 3, 5, 5), 1), ((3, 17, 9, 6), 1), ((1, 64, 14, 14), 1), ((2, 5, 8, 7), 0),
-                                       ((2, 16, 22, 22), 1)])
+                                       ((2, 16, 22, 22), 1),
+                                       # the NCHW LDS-halo kernels: a whole 56x56 image per workgroup, row blocks with a
+                                       # ragged last one (112 wide), two column blocks (tw = 68), odd sizes without padding,
+                                       # small images with several channel vectors to a workgroup and a ragged last group
+                                       ((2, 9, 56, 56), 1), ((1, 5, 112, 110), 1), ((1, 4, 10, 270), 1), ((2, 6, 47, 51), 0),
+                                       ((3, 44, 14, 14), 1), ((2, 21, 28, 26), 1)])
 def test_f4_input_transform(oracle, layout, order, shape, pad):
     N, C, H, W = shape
     x = synth.small_ints(N * C * H * W, 77 + sum(shape), -8, 8).reshape(N, C, H, W)

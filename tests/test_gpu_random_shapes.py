@@ -1,0 +1,75 @@
+"""Seeded random layer shapes through every pipeline and layout against the CPU oracle's direct convolution: odd
+extents, channel counts around the vector and tile sizes, both paddings, batch sizes that leave ragged tile blocks.
+The fixed-shape tests name the cases the kernels were designed around; this sweep is for the ones nobody named."""
+import numpy as np
+import pytest
+
+from cudnntest_amd import ops, synth
+from cudnntest_amd._lib import WinoError
+from gpu_util import TOL, dev, host, rounded
+
+pytestmark = pytest.mark.gpu
+LAYOUTS = [ops.NCHW, ops.NHWC, ops.CHWN]
+
+
+def _shapes(seed, count, cmax, hmax):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        N = int(rng.integers(1, 6))
+        C = int(rng.choice([1, 3, 4, 5, 8, 16, 17, 31, 32, 40, 64, 72, cmax]))
+        K = int(rng.choice([1, 2, 7, 16, 33, 64, 65, 96, 130]))
+        H = int(rng.integers(3, hmax))
+        W = int(rng.integers(3, hmax))
+        out.append((N, C, K, H, W, int(rng.integers(0, 3))))
+    return out
+
+
+@pytest.mark.parametrize("shape", _shapes(20260, 24, 130, 40))
+def test_fp32_integers_bit_exact_every_pipeline(oracle, shape):
+    N, C, K, H, W, pad = shape
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=sum(shape), integer=True)
+    for src in LAYOUTS:
+        dst = LAYOUTS[(src + N) % 3]
+        xs, ws = synth.act_to_layout(x, src), synth.flt_to_layout(w, src)
+        want = oracle.direct_conv(xs, ws, pad, src, dst)
+        for algo in (ops.ALGO_AUTO, ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_DIRECT):
+            try:
+                got = host(ops.conv(dev(xs), dev(ws), pad, src, dst, algo))
+            except WinoError as e:
+                assert e.code == -2 and algo in (ops.ALGO_FUSED, ops.ALGO_DIRECT), (algo, str(e))   # built for fewer cases, and says so
+                continue
+            assert np.array_equal(got, want), (src, dst, algo)
+
+
+@pytest.mark.parametrize("shape", _shapes(77, 16, 200, 64))
+def test_fp32_floats_f4_and_auto(oracle, shape):
+    N, C, K, H, W, pad = shape
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=sum(shape) + 1)
+    bias = synth.normal(K, 5, 0.3)
+    for src in LAYOUTS:
+        xs, ws = synth.act_to_layout(x, src), synth.flt_to_layout(w, src)
+        want = synth.act_from_layout(oracle.direct_conv(xs, ws, pad, src), src) + bias[None, :, None, None]
+        want = synth.act_to_layout(np.maximum(want, 0).astype(np.float32), src)
+        for algo in (ops.ALGO_STAGED_F4, ops.ALGO_AUTO):
+            got = host(ops.conv(dev(xs), dev(ws), pad, src, algo=algo, relu=True, bias=dev(bias)))
+            assert oracle.rel_l2(got, want) <= 2e-5, (src, algo)
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", _shapes(4242, 12, 136, 72))
+def test_two_byte_integers_round_once(oracle, dtype, shape):
+    """Small integers: every product and partial sum is exact in fp32, so the only rounding is the final store."""
+    N, C, K, H, W, pad = shape
+    x, w = synth.conv_inputs(N, C, K, H, W, seed=sum(shape) + 2, integer=True)
+    for src in LAYOUTS:
+        xs, ws = synth.act_to_layout(x, src), synth.flt_to_layout(w, src)
+        want = rounded(oracle.direct_conv(xs, ws, pad, src), dtype, oracle)
+        for algo in (ops.ALGO_AUTO, ops.ALGO_EPILOGUE, ops.ALGO_DIRECT):
+            try:
+                got = host(ops.conv(dev(xs, dtype), dev(ws, dtype), pad, src, algo=algo))
+            except WinoError as e:
+                assert e.code == -2 and algo == ops.ALGO_DIRECT, (algo, str(e))
+                continue
+            assert np.array_equal(got, want), (src, algo)
+    assert TOL[dtype] > 0
