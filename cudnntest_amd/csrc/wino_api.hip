@@ -943,14 +943,14 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
 }
 // fp32 layers with a long reduction and enough 4x4 tiles run faster through the F(4x4,3x3) pipeline, product tensor
 // and all: 2.25 multiplies per output instead of 4, and a transformed input of 2.25x the tensor instead of 4x.
-// Measured at N = 32, NCHW, against the fastest F(2x2) pipeline: C = K = 256, H = 56: 0.39 against 0.51 ms;
-// C = 256, K = 512, H = 28: 0.20 against 0.28; C = K = 512, H = 28: 0.34 against 0.50; C = K = 512, H = 14 (512
-// tiles): 0.14 against 0.16; C = 128, K = 256, H = 56: 0.26 against 0.28; C = K = 128, H = 112: 0.57 against 0.55
-// (the single-kernel path); C = 64, K = 128, H = 112: 0.41 against 0.31.  (NHWC: 0.42 against 0.53 on the first of
-// these, CHWN 0.40 against 0.52.)  Its rounding error is about four times that of F(2x2) (3e-6 to 5e-6 relative L2
-// on these layers).
+// Measured at N = 32, NCHW, against the fastest F(2x2) pipeline: C = K = 256, H = 56: 0.37 against 0.54 ms;
+// C = 256, K = 512, H = 28: 0.19 against 0.28; C = K = 512, H = 28: 0.34 against 0.52; C = K = 512, H = 14 (512
+// tiles): 0.13 against 0.17; C = 128, K = 256, H = 56: 0.24 against 0.28; C = K = 128, H = 112: 0.52 against 0.57
+// (the single-kernel path); C = K = 128, H = 56: 0.14 against 0.18; C = 64, K = 128, H = 112: 0.36 against 0.31.
+// (NHWC: 0.40 against 0.53 on the first of these, CHWN 0.38 against 0.52.)  Its rounding error is about four times
+// that of F(2x2) (3e-6 to 5e-6 relative L2 on these layers).
 bool auto_f4(int dtype, const Geometry& g) {
-    if (dtype != WINO_F32 || g.C < 128 || g.K < 128 || (g.C < 256 && g.K < 256)) return false;
+    if (dtype != WINO_F32 || g.C < 128 || g.K < 128) return false;
     const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
     return tiles4 >= 512;
 }

@@ -62,7 +62,7 @@ typedef enum {
                                own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101):
                                2.25 multiplies per output instead of 4, about four times the rounding error of
                                F(2x2) (3e-6 to 5e-6 relative L2 in fp32 on the VGG layers).  WINO_ALGO_AUTO takes it
-                               for fp32 layers with C, K >= 128, one of them >= 256, and at least 512 tiles when it is
+                               for fp32 layers with C, K >= 128 and at least 512 tiles when it is
                                given the filter bank itself; transformed filters handed to this algorithm by
                                name must come from wino_f4_filter_transform. */
     WINO_ALGO_DIRECT = 5     /* no Winograd at all, the convolution itself on the matrix cores.  Two kernels:
