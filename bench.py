@@ -67,26 +67,26 @@ WORKLOADS = {
 # script (the summary file holds the counters and the copy-kernel scale factor), keyed by
 # (workload, layout, dtype, resolved algo): (bytes, summary under profiles/).
 MEASURED_TRAFFIC = {
-    # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_kernel): 320.4 MB fetched + 231.2 MB written
+    # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_kernel): 320.7 MB fetched + 231.2 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged_f4"):
-        (551.6e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
-    # 635.9 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
+        (551.9e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # 636.1 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"):
-        (747.1e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_counters.txt"),
-    # 482.8 MB fetched + 411.0 MB written
+        (747.2e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # 483.1 MB fetched + 411.0 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"):
-        (893.8e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_counters.txt"),
-    # 580.1 MB fetched + 411.0 MB written
+        (894.1e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # 581.5 MB fetched + 411.0 MB written
     ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"):
-        (991.1e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_counters.txt"),
-    # direct16_rows_kernel: 83.1 + 51.4 MB; 325.3 + 208.8 MB
+        (992.6e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # direct16_rows_kernel: 83.1 + 51.4 MB; 325.3 + 209.2 MB
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "direct"):
         (134.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv3_N32_counters.txt"),
     ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "bf16", "direct"):
-        (534.1e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv1_2_N32_counters.txt"),
-    # gemm_rows_kernel in bf16: 271.6 MB fetched + 56.9 MB written
+        (534.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # gemm_rows_kernel in bf16: 271.5 MB fetched + 56.9 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "epilogue"):
-        (328.5e6, "profiles/epilogue_bf16_nchw_vgg16_conv3_N32_counters.txt"),
+        (328.4e6, "profiles/epilogue_bf16_nchw_vgg16_conv3_N32_counters.txt"),
 }
 # what the default run also times, after the headline's timed region: (name, workload, dtype)
 OTHER_CONFIGS = [
