@@ -51,17 +51,29 @@ struct D16Geom {
 };
 
 // ---- filter bank -> W9[tap][Cp/8][Kp][8] (zero padded) --------------------------------------------------
-// One thread per (filter, channel vector).  VEC: the bank is [K][C][3][3] with C a multiple of 8 and a 16-byte
+// One thread per (filter, channel vector).  VEC = 1: the bank is [K][C][3][3] with C a multiple of 8 and a 16-byte
 // aligned base, so the 72 values of a thread are 144 contiguous, aligned bytes: nine 16-byte loads instead of 72
-// two-byte ones a filter apart.
-template <typename T, bool VEC>
+// two-byte ones a filter apart.  VEC = 2: [K][3][3][C], same conditions: a tap's 8 channels are one 16-byte load and
+// go out as they are.
+template <typename T, int VEC>
 __global__ __launch_bounds__(64) void direct16_pack_kernel(const T* __restrict__ w, T* __restrict__ W9, FltStrides s,
                                                            int K, int C, int Kp, int CQ) {
     const int k = blockIdx.x * 64 + threadIdx.x, cq = blockIdx.y;
     if (k >= Kp) return;
     unsigned short raw[72];                                  // [channel of the vector][tap]
     const bool kin = k < K;
-    if (VEC) {
+    if (VEC == 2) {
+        const bool in = kin && cq * 8 < C;
+        const uint4* src = reinterpret_cast<const uint4*>(w + (size_t)(kin ? k : K - 1) * 9 * C + (cq * 8 < C ? cq * 8 : 0));
+        uint4 v[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) v[t] = src[(size_t)t * (C / 8)];
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+            *reinterpret_cast<uint4*>(W9 + (((size_t)t * CQ + cq) * Kp + k) * 8) = in ? v[t] : make_uint4(0, 0, 0, 0);
+        return;
+    }
+    if (VEC == 1) {
         uint4 v[9];
         const uint4* src = reinterpret_cast<const uint4*>(w + ((size_t)(kin ? k : K - 1) * C + (cq * 8 < C ? cq * 8 : 0)) * 9);
 #pragma unroll

@@ -1,4 +1,5 @@
-// Direct 3x3 convolution of 2-byte NCHW tensors, the kernel for large images (see direct16.hpp for the method):
+// Direct 3x3 convolution of 2-byte NCHW (and, with the template flag further down, NHWC) tensors, the kernel for large
+// images (see direct16.hpp for the method):
 // one workgroup of 8 waves per CU, tiles of 64*WF filters x 8/WF waves of 4 rows x 32 columns of output pixels, the
 // waves side by side until they span the image's width (then stacked).
 //
@@ -38,12 +39,18 @@ template <int WF> struct D16R {
     static constexpr int NTASK = WF == 2 ? 2 : 3;            // input tasks per thread and stage
 };
 
-template <typename T, int WF>
+// NHWC: x and y are [N][H][W][C] / [N][Ho][Wo][K].  The 8 channels of a pixel's vector are 16 contiguous bytes of x:
+// an input task is one pixel slot of one channel vector (a 16-byte load, a 16-byte LDS write, zeros where the slot
+// lies outside the image), the two vectors of a pixel on neighbouring lanes.  The multiplies take the pixel fragment
+// as the first operand, so a lane holds one FILTER and its registers the pixels: the 32 filters of a wave's half are
+// 64 contiguous bytes of a pixel of y.
+template <typename T, int WF, bool NHWC = false>
 __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restrict__ x, const T* __restrict__ W9,
                                                                T* __restrict__ y, D16Geom g, Epilogue ep) {
     typedef typename Mma<T>::vec vec;
     typedef D16R<WF> P;
-    constexpr int NTASK = P::NTASK;
+    constexpr int NTASK = NHWC ? (2 * P::XPLANE + 511) / 512 : P::NTASK;   // input tasks per thread and stage
+    constexpr int NX = NHWC ? NTASK : 8 * NTASK;                           // and the requests they make
     extern __shared__ __attribute__((aligned(16))) unsigned char d16r_smem[];     // [3][FB] filters, [2][XB] input
     unsigned char* const xsm = d16r_smem + 3 * P::FB;
     const int tid = threadIdx.x;
@@ -75,7 +82,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     };
 
     // ---- input tasks of this thread: (channel vector v, LDS row, column pair); what does not depend on the tile ----
-    const int ntask = 2 * g.LR * g.PP;
+    const int ntask = NHWC ? 2 * g.LR * g.PW : 2 * g.LR * g.PP;
     int tpk[NTASK];                                          // LDS row | (first column of the pair relative to c0, + 8) << 8 | v << 20
     int ldsw[NTASK];                                         // byte offset of the pair's first slot inside an input stage (a multiple of
                                                              // 16, -16 for the pair left of a row) | bit 0 / 1: slot 0 / 1 exists;
@@ -83,6 +90,13 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
     for (int q = 0; q < NTASK; ++q) {
         const int t = tid + 512 * q;
+        if constexpr (NHWC) {
+            // task t: channel vector t & 1 of pixel slot t >> 1 (row-major over the LR x PW slots of a plane)
+            // (tid + 512 q: the vector is the same for all tasks of a thread; row and column are recomputed per tile)
+            tpk[q] = 0;
+            ldsw[q] = t < ntask ? ((((t & 1) * P::XPLANE + (t >> 1)) * 16) | 1) : 0;
+            continue;
+        }
         const int m = t % g.PP, rr = t / g.PP;
         const int lr = rr % g.LR, v = min(rr / g.LR, 1);
         const int slot0 = 2 * m - g.pad;                     // the pair (c0 + 2m - 2 pad, + 1) sits in slots (2m - pad, + 1)
@@ -111,11 +125,20 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     auto prep_x = [&](const Tile& t) {
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
-            const int lr = tpk[q] & 0xFF, v = tpk[q] >> 20;
+            const int sl = min((tid + 512 * q) >> 1, g.LR * g.PW - 1);           // NHWC: the task's pixel slot
+            const int lr = NHWC ? sl / g.PW : tpk[q] & 0xFF, v = NHWC ? tid & 1 : tpk[q] >> 20;
             const int qq = t.oh0 + lr;                       // padded row index counted from image n0
             int dn = 0;
             for (int k = 1; k <= g.maxcross; ++k) dn += qq >= k * Hp ? 1 : 0;
             const int ih = qq - dn * Hp - g.pad;
+            if constexpr (NHWC) {
+                const int iw = t.c0 + (sl - lr * g.PW) - g.pad;
+                const bool in = (ldsw[q] & 3) != 0 && t.n0 + dn < g.N && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+                const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 1);
+                const int dnc = max(min(dn, g.N - 1 - t.n0), 0);
+                xoff[q] = ((unsigned)(((dnc * g.H + ihc) * g.W + iwc) * g.C + v * 8) * 2u) | (in ? 1u : 0u);   // a multiple of 16
+                continue;
+            }
             const int iw = t.c0 + ((tpk[q] >> 8) & 0xFFF) - 8;
             const bool in = (ldsw[q] & 3) != 0 && t.n0 + dn < g.N && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
             const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 2);
@@ -143,32 +166,44 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
         for (int q = 0; q < P::NF; ++q) dma_row(base + frow_src[q], lane_off, d16r_smem + slot * P::FB + frow_dst[q]);
     };
-    uint32_t raw[NTASK][8];
+    uint32_t raw[NHWC ? 1 : NTASK][8];
+    uint4 rawn[NHWC ? NTASK : 1];                            // NHWC: the 8 channels of a task's pixel
     unsigned poff[NTASK];
     int req_cs = 0;                                          // the stage (inside its tile) whose input was requested last
     // piece 8q + e of a stage's input requests: channel e of task q.  A stage's second channel vector may lie past
     // C: the first one is loaded instead, and masked when it is written
     auto x_piece = [&](int idx) {
-        const int q = idx >> 3, e = idx & 7;
         if (idx == 0) req_cs = cx.cs;
+        if constexpr (NHWC) {
+            const int v = tid & 1;
+            const bool vok = cx.cs * 16 + v * 8 < g.C;
+            rawn[NHWC ? idx : 0] = *reinterpret_cast<const uint4*>(xs + ((xoff[idx] & ~15u) - (vok ? 0u : (unsigned)v * 16u)));
+            return;
+        }
+        const int q = idx >> 3, e = idx & 7;
         if (e == 0) {
             const int v = tpk[q] >> 20;
             const bool vok = cx.cs * 16 + v * 8 < g.C;
             poff[q] = (xoff[q] & ~3u) - (vok ? 0u : (unsigned)v * 8u * hw2);
         }
-        raw[q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
+        raw[NHWC ? 0 : q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
         poff[q] += hw2;
     };
     auto x_commit = [&](int xslot) {                         // the stage requested through x_piece into input slot xslot
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
             if ((ldsw[q] & 3) == 0) continue;
-            const bool keep = (xoff[q] & 1u) && req_cs * 16 + (tpk[q] >> 20) * 8 < g.C;
+            const bool keep = (xoff[q] & 1u) && req_cs * 16 + (NHWC ? tid & 1 : tpk[q] >> 20) * 8 < g.C;
             const uint32_t km = keep ? 0xFFFFFFFFu : 0u;
+            if constexpr (NHWC) {
+                const uint4 r = rawn[NHWC ? q : 0];
+                *reinterpret_cast<uint4*>(xsm + xslot * P::XB + (ldsw[q] & ~15)) = make_uint4(r.x & km, r.y & km, r.z & km, r.w & km);
+                continue;
+            }
             uint32_t lo[4], hi[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t a = raw[q][2 * e] & km, b = raw[q][2 * e + 1] & km;
+                const uint32_t a = raw[NHWC ? 0 : q][2 * e] & km, b = raw[NHWC ? 0 : q][2 * e + 1] & km;
                 lo[e] = __builtin_amdgcn_perm(b, a, 0x05040100u);     // (a.lo16, b.lo16): the pair's first pixel
                 hi[e] = __builtin_amdgcn_perm(b, a, 0x07060302u);     // (a.hi16, b.hi16): its second pixel
             }
@@ -182,6 +217,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     int xw_off = 0;                                          // the wave's first input row, this lane's column: byte offset in an input stage
     int yoff[4];                                             // element offset of (n, k0, oh, ow) in y per row of the wave, < 0: no pixel
     int k0c = 0;                                             // first filter of this wave
+    int pc0 = 0;                                             // NHWC: first output column of this wave
     auto prep_pix = [&](const Tile& t) {
         k0c = t.k0 + wf * 64;
         const long g0 = (long)t.n0 * g.Ho + t.oh0;
@@ -194,6 +230,20 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         const bool rowok = g0 + 4 * wr < g.G;
         const int L = rowok ? dn * Hp + oh - t.oh0 : 0;
         xw_off = ((lh * P::XPLANE) + L * g.PW + (colok ? col : 0)) * 16;
+        if constexpr (NHWC) {
+            // element offset of (n, oh + j, the wave's first column, the wave's first filter); the lane's filter and
+            // the register's column are added at the stores
+            pc0 = t.c0 + 32 * wc;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                yoff[j] = rowok ? (int)((((long)(t.n0 + dn) * g.Ho + oh + j) * g.Wo + pc0) * g.K + k0c) : -1;
+            if (ep.pool && rowok) {                          // the two pooled rows of the wave, its first pooled column
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    yoff[j] = (int)((((long)(t.n0 + dn) * (g.Ho >> 1) + (oh >> 1) + j) * (g.Wo >> 1) + (pc0 >> 1)) * g.K + k0c);
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             yoff[j] = (rowok && colok) ? (int)((((long)(t.n0 + dn) * g.K + k0c) * g.Ho + oh + j) * g.Wo + t.c0 + col) : -1;
@@ -240,7 +290,10 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                 const int r = rho - j;
                 if (r < 0 || r > 2) continue;
 #pragma unroll
-                for (int i = 0; i < 2; ++i) Mma<T>::run(a[r][i], b[t % 3], acc[i][j]);
+                for (int i = 0; i < 2; ++i) {
+                    if constexpr (NHWC) Mma<T>::run(b[t % 3], a[r][i], acc[i][j]);
+                    else Mma<T>::run(a[r][i], b[t % 3], acc[i][j]);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         };
@@ -271,6 +324,65 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         unsigned ks = kstride2;
         asm volatile("" : "+s"(ks));
         char* const yb = reinterpret_cast<char*>(y);
+        if constexpr (NHWC) {
+            // register r of acc[i][j]: pixel column pc0 + 8*(r/4) + 4*lh + r%4 of row j, the lane's filter
+            // k0c + 32*i + l32.  Two neighbouring lanes hold neighbouring filters and exchange values, so that each
+            // stores one 4-byte pair of filters -- the even lane for the pixel of register r, the odd lane for that of
+            // register r+1: per instruction the 16 even (odd) lanes of a half write 64 contiguous bytes of one pixel.
+            unsigned kp = (unsigned)g.K * 2u;                // bytes between two pixels of y
+            asm volatile("" : "+s"(kp));
+            if (ep.pool) {
+                // a 2x2 window is two rows of the wave and two neighbouring registers of a lane: the maximum is taken in
+                // registers and the lane stores its filter's pooled value (2 bytes; 32 lanes: 64 contiguous bytes)
+                unsigned q[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) q[j] = ((unsigned)yoff[j] + (unsigned)l32) * 2u + (unsigned)(2 * lh) * kp;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const float bk = ep.bias ? bias_of<T>(ep, k0c + 32 * i + l32) : 0.f;
+#pragma unroll
+                    for (int r2 = 0; r2 < 16; r2 += 2) {
+                        const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) {
+                            float v = fmaxf(fmaxf(acc[i][2 * j][r2], acc[i][2 * j][r2 + 1]), fmaxf(acc[i][2 * j + 1][r2], acc[i][2 * j + 1][r2 + 1])) + bk;
+                            if (ep.relu) v = fmaxf(v, 0.f);
+                            if (pok) *reinterpret_cast<T*>(yb + q[j] + (unsigned)(i * 64)) = from_f32<T>(v);
+                            q[j] += ((r2 & 2) ? 3u : 1u) * kp;
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) q[j] -= 16u * kp;
+                }
+                return;
+            }
+            unsigned o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = ((unsigned)yoff[j] + (unsigned)(l32 - (odd ? 1 : 0))) * 2u + (unsigned)(4 * lh + (odd ? 1 : 0)) * kp;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float bk = ep.bias ? bias_of<T>(ep, k0c + 32 * i + l32) : 0.f;
+#pragma unroll
+                for (int r2 = 0; r2 < 16; r2 += 2) {
+                    const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;    // (Wo is even: the pair's pixels exist together)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float v0 = acc[i][j][r2] + bk, v1 = acc[i][j][r2 + 1] + bk;
+                        if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
+                        const float got = swap_lane_pairs(odd ? v0 : v1);
+                        const float lo = odd ? got : v0, hi = odd ? v1 : got;
+                        struct alignas(4) Pair { T a, b; };
+                        if (pok) *reinterpret_cast<Pair*>(yb + o[j] + (unsigned)(i * 64)) = Pair{from_f32<T>(lo), from_f32<T>(hi)};
+                        o[j] += ((r2 & 2) ? 6u : 2u) * kp;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] -= 32u * kp;                    // back to the first pixel for the other 32 filters
+            }
+            return;
+        }
         if (ep.pool) {
             // with pooling: the maximum over the two rows in registers, over the two columns with the neighbouring lane;
             // the even lane stores the pooled value of filter r, the odd lane that of filter r+1 (2 bytes each)
@@ -346,7 +458,6 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     // wait until at most `newest` of this wave's memory requests are outstanding (loads return in order, so those
     // are the ones issued last), and for its LDS writes; then the workgroup's barrier
     auto wait_only = [&](int newest) {
-        constexpr int NX = 8 * NTASK;
         if (newest == 0) __builtin_amdgcn_s_waitcnt(0x0070);
         else if (newest == P::NF) __builtin_amdgcn_s_waitcnt(0x0070 | P::NF);
         else if (newest == NX) __builtin_amdgcn_s_waitcnt(0x0070 | (NX & 0xF) | ((NX >> 4) << 14));
@@ -384,9 +495,9 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             need_prep = false;
         }
 #pragma unroll
-        for (int i = 0; i < 8 * NTASK; ++i) x_piece(i);
+        for (int i = 0; i < NX; ++i) x_piece(i);
         pending = true;
-        xs += (size_t)16 * HW * 2;
+        xs += NHWC ? (size_t)32 : (size_t)16 * HW * 2;                           // the next 16 channels
         advance(cx);
         need_prep = cx.cs == 0;
     };
@@ -394,7 +505,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     x_commit(0);
     pending = false;
     if (cx.valid) x_request();
-    wait_barrier(pending ? 8 * NTASK : 0);
+    wait_barrier(pending ? NX : 0);
 
     int fslot = 0, xslot = 0;
     const int ntiles = (send - s0 + sstep - 1) / sstep;
@@ -418,7 +529,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             }
             freq = f_next(fslot);
         });
-        const int newest = (xreq ? 8 * NTASK : 0) + (freq ? P::NF : 0);
+        const int newest = (xreq ? NX : 0) + (freq ? P::NF : 0);
         if (cs == nst - 1) {
             wait_only(newest);                               // before the stores: they would count as the newest requests
             stores();

@@ -75,10 +75,14 @@ typedef enum {
                                direct product by nothing but the multiplies (the stage it replaces is
                                comparison/GEMM.cuh:124-253; the reference's own direct kernel in tile geometry is
                                Conv_fuse, fusedTest/winotrans.cuh:1868).
-                               Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (output
-                               height a multiple of 4, K a multiple of 64, at least a tile for every other CU), not
-                               for C <= 4; needs the filter bank itself (not wino_conv_prepared).
-                               What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW layers. */
+                               2-byte NHWC -> NHWC layers ([K][3][3][C] filters) with C a multiple of 8 and a 16-byte
+                               aligned x run on the larger of its two kernels (the 8-wave one) when the layer has its
+                               shape: output height a multiple of 4, even output width, K a multiple of 64, at least a
+                               tile for every other CU; other NHWC layers are refused (WINO_ERR_UNSUPPORTED).
+                               Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (the
+                               shape just named), not for C <= 4; needs the filter bank itself (not
+                               wino_conv_prepared).
+                               What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW and NHWC layers. */
 } wino_algo_t;
 
 /* order of the tile index p inside the transformed operands */

@@ -52,19 +52,22 @@ def test_prepared_filters_and_passes(oracle):
     assert torch.equal(got, ref)
 
 
-def test_stack_with_multi_pass_layers_eager_and_graph(oracle):
-    """Two bf16 layers of the size that is cut into passes, as a conv stack: the eager pass equals the layers run
-    one by one through the one-pass staged pipeline, and graph replays equal the eager pass."""
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC])
+def test_stack_with_multi_pass_layers_eager_and_graph(oracle, layout):
+    """Two bf16 layers of the size that is cut into passes (and that AUTO runs on the 16-bit direct kernel, the second
+    one with pooling in its stores), as a conv stack: the eager pass equals the layers run one by one through the
+    one-pass staged pipeline, and graph replays equal the eager pass."""
     N, C, K, H = 32, 64, 128, 112
-    layers = [dict(K=K, relu=True, pool=False), dict(K=K, relu=True, pool=True)]
+    layers = [dict(K=K, relu=True, pool=False, layout_in=layout), dict(K=K, relu=True, pool=True)]
     st = ops.ConvStack(torch.bfloat16, N, C, H, H, layers)
-    w1, w2 = _ints((K, C, 3, 3), 31, -1, 1, ops.BF16), _ints((K, K, 3, 3), 32, -1, 1, ops.BF16)
+    perm = (lambda t: t.permute(0, 2, 3, 1).contiguous()) if layout == ops.NHWC else (lambda t: t)
+    w1, w2 = perm(_ints((K, C, 3, 3), 31, -1, 1, ops.BF16)), perm(_ints((K, K, 3, 3), 32, -1, 1, ops.BF16))
     b1, b2 = _ints((K,), 33, -2, 2, ops.BF16), _ints((K,), 34, -2, 2, ops.BF16)
     st.set_layer(0, w1, b1)
     st.set_layer(1, w2, b2)
-    x = _ints((N, C, H, H), 35, -1, 1, ops.BF16)
-    mid = ops.conv(x, w1, 1, ops.NCHW, algo=ops.ALGO_STAGED, relu=True, bias=b1)
-    ref = ops.conv(mid, w2, 1, ops.NCHW, algo=ops.ALGO_STAGED, relu=True, bias=b2, pool=True)
+    x = perm(_ints((N, C, H, H), 35, -1, 1, ops.BF16))
+    mid = ops.conv(x, w1, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=b1)
+    ref = ops.conv(mid, w2, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=b2, pool=True)
     want = st.forward(x).clone()
     assert torch.equal(want, ref)
     out = torch.empty(st.out_shape, dtype=torch.bfloat16, device="cuda")

@@ -81,6 +81,45 @@ def test_integers_round_once_one_tile_per_cu_and_more(oracle, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", BIG_SHAPES[:4] + [(64, 256, 256, 28, 28, 1), (8, 72, 320, 56, 60, 1)])
+def test_nhwc_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
+    """[N][H][W][C] tensors and [K][3][3][C] filters: the pixel's channel vectors are loaded as they lie, the
+    multiplies run with the operands exchanged and the stores are along the filters.  Whole tensors against the staged
+    Winograd pipeline from the same layout and against the NCHW direct kernel (same products, same order of
+    summation: the same bits), planes of the first and last image against the oracle; twice."""
+    N, C, K, H, W, pad = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -1, 1).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    xl, wl = synth.act_to_layout(x, ops.NHWC), synth.flt_to_layout(w, ops.NHWC)
+    xd, wd, bd = dev(xl, dtype), dev(wl, dtype), dev(bias, dtype)
+    if shape[:5] in ((64, 256, 256, 28, 28), (32, 64, 128, 112, 112)):                  # what AUTO takes for such layers
+        assert ops.pick_algo(ops.NHWC, dtype, N, C, K, H, W, pad) == ops.ALGO_DIRECT
+    ref = ops.conv(xd, wd, pad, ops.NHWC, algo=ops.ALGO_STAGED, relu=True, bias=bd)
+    nchw = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+    ks = sorted({0, K // 2, K - 1})
+    for rep in range(2):
+        got = ops.conv(xd, wd, pad, ops.NHWC, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+        assert torch.equal(got, ref), rep
+        assert torch.equal(got.permute(0, 3, 1, 2), nchw), rep
+        for n in (0, N - 1):
+            want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], pad) + bias[ks][None, :, None, None], 0)
+            assert np.array_equal(host(got[n:n + 1].permute(0, 3, 1, 2)[:, ks]), rounded(want.astype(np.float32), dtype, oracle)), (rep, n)
+    # 2x2 pooling in the stores (rounding is monotonic: the pooled tensor is the pooling of the unpooled one)
+    pooled = ops.conv(xd, wd, pad, ops.NHWC, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+    assert tuple(pooled.shape) == (N, got.shape[1] // 2, got.shape[2] // 2, K)
+    assert torch.equal(pooled.permute(0, 3, 1, 2), torch.nn.functional.max_pool2d(got.permute(0, 3, 1, 2).float(), 2).to(got.dtype))
+    assert torch.equal(pooled, ops.conv(xd, wd, pad, ops.NHWC, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True))
+    # floats: only the final rounding separates it from the oracle
+    xf, wf = synth.conv_inputs(min(N, 2), C, K, H, W, seed=5 + sum(shape))
+    xr, wr = rounded(xf, dtype, oracle), rounded(wf, dtype, oracle)
+    if ops.pick_algo(ops.NHWC, dtype, min(N, 2), C, K, H, W, pad) == ops.ALGO_DIRECT:
+        gotf = ops.conv(dev(synth.act_to_layout(xr, ops.NHWC), dtype), dev(synth.flt_to_layout(wr, ops.NHWC), dtype), pad, ops.NHWC)
+        err = oracle.rel_l2(host(gotf.permute(0, 3, 1, 2)), oracle.direct_conv(xr, wr, pad))
+        assert err <= (1e-3 if dtype == ops.F16 else 5e-3), err
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
 @pytest.mark.parametrize("shape", [(2, 64, 64, 56, 56), (1, 128, 256, 28, 28), (3, 256, 64, 14, 14)])
 def test_floats_within_tolerance(oracle, shape, dtype):
     N, C, K, H, W = shape
