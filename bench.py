@@ -88,14 +88,17 @@ MEASURED_TRAFFIC = {
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "epilogue"):
         (328.4e6, "profiles/epilogue_bf16_nchw_vgg16_conv3_N32_counters.txt"),
 }
-# what the default run also times, after the headline's timed region: (name, workload, dtype)
+# what the default run also times, after the headline's timed region: (name, workload, dtype, layout)
 OTHER_CONFIGS = [
-    ("cfg1_N1_C64_K64_H56_f32", "cfg1_N1_C64_K64_H56", "f32"),
-    ("cfg3a_N64_C512_K512_H28_f32", "vgg16_conv4_N64_C512_K512_H28", "f32"),
-    ("cfg3b_N64_C512_K512_H14_f32", "vgg16_conv5_N64_C512_K512_H14", "f32"),
-    ("cfg4_N32_C64_K64_H224_f32", "vgg16_conv1_2_N32_C64_K64_H224", "f32"),
-    ("cfg5_vgg16_all13_N32_f16", "vgg16_all13", "f16"),
-    ("cfg5_vgg16_all13_N32_bf16", "vgg16_all13", "bf16"),
+    ("cfg1_N1_C64_K64_H56_f32", "cfg1_N1_C64_K64_H56", "f32", "NCHW"),
+    ("cfg2_N32_C256_K256_H56_f32_NHWC", "vgg16_conv3_N32_C256_K256_H56", "f32", "NHWC"),
+    ("cfg2_N32_C256_K256_H56_f32_CHWN", "vgg16_conv3_N32_C256_K256_H56", "f32", "CHWN"),
+    ("cfg3a_N64_C512_K512_H28_f32", "vgg16_conv4_N64_C512_K512_H28", "f32", "NCHW"),
+    ("cfg3b_N64_C512_K512_H14_f32", "vgg16_conv5_N64_C512_K512_H14", "f32", "NCHW"),
+    ("cfg4_N32_C64_K64_H224_f32", "vgg16_conv1_2_N32_C64_K64_H224", "f32", "NCHW"),
+    ("cfg5_vgg16_all13_N32_f16", "vgg16_all13", "f16", "NCHW"),
+    ("cfg5_vgg16_all13_N32_bf16", "vgg16_all13", "bf16", "NCHW"),
+    ("cfg5_vgg16_all13_N32_bf16_NHWC", "vgg16_all13", "bf16", "NHWC"),
 ]
 KERNEL_OF = {"staged": "gemm_128x128_kernel / gemm_128x128_walk_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
              "staged_f4": "gemm_128x128_kernel / gemm_128x128_walk_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel"}
@@ -224,9 +227,9 @@ def main():
             out.append((x, w, y))
         return out
 
-    def other_config(workload, dtype):
-        """one of the other benchmark configurations, NCHW, the automatic choice of pipeline: a few steps"""
-        layout, layers = ops.NCHW, layers_of(workload)
+    def other_config(workload, dtype, layout_name="NCHW"):
+        """one of the other benchmark configurations, the automatic choice of pipeline: a few steps"""
+        layout, layers = LAYOUT[layout_name], layers_of(workload)
         many = len(layers) > 1
         tens = device_tensors(layers, layout, dtype, 0xBE7C)
 
@@ -235,15 +238,20 @@ def main():
                 ops.conv(x, w, 1, layout, relu=many, out=y)
         tiny = layers[0][0] == 1                      # N = 1: a step is a few tens of microseconds
         steps = 20 if many else (200 if tiny else 30)
+        # generating the tensors left the GPU idle: untimed steps for 100 ms bring the clock back up, as before the headline
+        r0 = time.perf_counter()
+        while time.perf_counter() - r0 < 0.1:
+            run(tens)
+            torch.cuda.synchronize()
         ms, wall = timed(lambda: run(tens), steps, 5, group=10 if tiny else 1)
         flops = sum(2.0 * N * K * C * H * H * 9 for (N, C, K, H) in layers)
         res = {"ms": round(ms, 4), "ms_wall_mean": round(wall, 4), "steps": steps,
-               "effective_tflops": round(flops / (ms * 1e-3) / 1e12, 2), "dtype": dtype, "layout": "NCHW"}
+               "effective_tflops": round(flops / (ms * 1e-3) / 1e12, 2), "dtype": dtype, "layout": layout_name}
         per_layer, k_flops, k_ms = [], 0.0, 0.0
         for (N, C, K, H), t in zip(layers, tens):
             a = ops.pick_algo(layout, DT[dtype], N, C, K, H, H)
             st = staged_pass(lambda: run([t]), 10)
-            r = kernel_roofline("NCHW", dtype, a, N, C, K, H, st["gemm"][0] / 10)
+            r = kernel_roofline(layout_name, dtype, a, N, C, K, H, st["gemm"][0] / 10)
             k_flops += r["flops"]
             k_ms += r["kernel_ms"]
             if many:
@@ -422,7 +430,7 @@ def main():
     if default_run and not args.no_other_configs:
         del tensors
         torch.cuda.empty_cache()
-        out["configs"] = {name: other_config(wl, dty) for (name, wl, dty) in OTHER_CONFIGS}
+        out["configs"] = {name: other_config(wl, dty, lay) for (name, wl, dty, lay) in OTHER_CONFIGS}
 
     if not args.no_cpu_baseline:
         import oracle
