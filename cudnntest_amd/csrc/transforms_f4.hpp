@@ -225,8 +225,22 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
         return;
     }
     const int tid = threadIdx.x;
-    const int ty = blockIdx.x / colBlocks, cb = blockIdx.x - ty * colBlocks;
-    const int c0 = blockIdx.y * F4N_CC, n = blockIdx.z - zjob;
+    // Workgroup ids go round-robin to the 8 XCDs, each with an L2 of its own.  Re-dealt so that an XCD takes a
+    // contiguous eighth of the (image, channel block, tile row) sequence: neighbouring tile rows share two of their
+    // six pixel rows, and their 224-byte runs of a coordinate plane of V lie next to each other.
+    int bx = blockIdx.x, by = blockIdx.y, n = blockIdx.z - zjob;
+    {
+        const unsigned total = gridDim.x * gridDim.y * (unsigned)N;
+        if ((total & 7u) == 0) {
+            const unsigned lin = bx + gridDim.x * (by + gridDim.y * (unsigned)n);
+            const unsigned re = (lin & 7u) * (total >> 3) + (lin >> 3);
+            bx = re % gridDim.x;
+            by = (re / gridDim.x) % gridDim.y;
+            n = re / (gridDim.x * gridDim.y);
+        }
+    }
+    const int ty = bx / colBlocks, cb = bx - ty * colBlocks;
+    const int c0 = by * F4N_CC;
     const int tx0 = cb * F4N_TCB, ntx = min(F4N_TCB, tw - tx0);
     const int wlb = 4 * ntx + 2;                             // pixel columns of the block
     const int h0 = 4 * ty - pad, w0 = 4 * tx0 - pad;
