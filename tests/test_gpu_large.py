@@ -1,7 +1,7 @@
 """Index arithmetic past 2^31: a layer whose transformed operands hold more than 2^31 elements (N=768, C=K=256,
 H=W=56 in fp32: x and y 617 M elements = 2.5 GB each, the transformed input V 2.47 G elements = 9.9 GB, the product
 tensor of the staged pipeline as much again, byte offsets past 2^33).  The oracle convolves the LAST image (the far
-end of every index space) with three filters; the two pipelines must agree with each other over the whole tensor."""
+end of every index space) with three filters; the pipelines must agree with each other over the whole tensor."""
 import pytest
 import torch
 
@@ -36,7 +36,7 @@ def test_more_than_2_31_elements_per_operand(oracle, layout):
     else:
         xl, wl = x, w
     ys = {}
-    for algo in (ops.ALGO_EPILOGUE, ops.ALGO_STAGED):
+    for algo in (ops.ALGO_EPILOGUE, ops.ALGO_STAGED, ops.ALGO_STAGED_F4):
         y = ops.conv(xl, wl, 1, layout, algo=algo)
         y_nchw = y.permute(0, 3, 1, 2) if layout == ops.NHWC else y
         assert tuple(y_nchw.shape) == (N, K, H, H)
@@ -44,6 +44,9 @@ def test_more_than_2_31_elements_per_operand(oracle, layout):
         assert err <= TOL[ops.F32], (algo, err)
         ys[algo] = y
     assert _rel(ys[ops.ALGO_STAGED], ys[ops.ALGO_EPILOGUE]) <= 1e-5
+    # the F(4x4) pipeline (what the automatic choice runs at this size): 5.5 GB of transformed input, as much product
+    assert ops.pick_algo(layout, ops.F32, N, C, K, H, H, 1) == ops.ALGO_STAGED_F4
+    assert _rel(ys[ops.ALGO_STAGED_F4], ys[ops.ALGO_STAGED]) <= 2e-5
     # leave the scratch arena at its usual size for the tests that follow
     del ys, y, xl
     torch.cuda.empty_cache()
