@@ -331,6 +331,12 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             // register r+1: per instruction the 16 even (odd) lanes of a half write 64 contiguous bytes of one pixel.
             unsigned kp = (unsigned)g.K * 2u;                // bytes between two pixels of y
             asm volatile("" : "+s"(kp));
+            // (the two filter halves of a pixel, 64 + 64 bytes of one 128-byte line, are stored one right after the other)
+            float bk[2] = {0.f, 0.f};
+            if (ep.bias) {
+                bk[0] = bias_of<T>(ep, k0c + l32);
+                bk[1] = bias_of<T>(ep, k0c + 32 + l32);
+            }
             if (ep.pool) {
                 // a 2x2 window is two rows of the wave and two neighbouring registers of a lane: the maximum is taken in
                 // registers and the lane stores its filter's pooled value (2 bytes; 32 lanes: 64 contiguous bytes)
@@ -338,22 +344,19 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
                 for (int j = 0; j < 2; ++j) q[j] = ((unsigned)yoff[j] + (unsigned)l32) * 2u + (unsigned)(2 * lh) * kp;
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    const float bk = ep.bias ? bias_of<T>(ep, k0c + 32 * i + l32) : 0.f;
+                for (int r2 = 0; r2 < 16; r2 += 2) {
+                    const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;
 #pragma unroll
-                    for (int r2 = 0; r2 < 16; r2 += 2) {
-                        const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;
+                    for (int j = 0; j < 2; ++j) {
 #pragma unroll
-                        for (int j = 0; j < 2; ++j) {
-                            float v = fmaxf(fmaxf(acc[i][2 * j][r2], acc[i][2 * j][r2 + 1]), fmaxf(acc[i][2 * j + 1][r2], acc[i][2 * j + 1][r2 + 1])) + bk;
+                        for (int i = 0; i < 2; ++i) {
+                            float v = fmaxf(fmaxf(acc[i][2 * j][r2], acc[i][2 * j][r2 + 1]), fmaxf(acc[i][2 * j + 1][r2], acc[i][2 * j + 1][r2 + 1])) + bk[i];
                             if (ep.relu) v = fmaxf(v, 0.f);
                             if (pok) *reinterpret_cast<T*>(yb + q[j] + (unsigned)(i * 64)) = from_f32<T>(v);
-                            q[j] += ((r2 & 2) ? 3u : 1u) * kp;
                         }
-                        __builtin_amdgcn_sched_barrier(0);
+                        q[j] += ((r2 & 2) ? 3u : 1u) * kp;
                     }
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) q[j] -= 16u * kp;
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 return;
             }
@@ -361,25 +364,22 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
             for (int j = 0; j < 4; ++j) o[j] = ((unsigned)yoff[j] + (unsigned)(l32 - (odd ? 1 : 0))) * 2u + (unsigned)(4 * lh + (odd ? 1 : 0)) * kp;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const float bk = ep.bias ? bias_of<T>(ep, k0c + 32 * i + l32) : 0.f;
+            for (int r2 = 0; r2 < 16; r2 += 2) {
+                const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;    // (Wo is even: the pair's pixels exist together)
 #pragma unroll
-                for (int r2 = 0; r2 < 16; r2 += 2) {
-                    const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;    // (Wo is even: the pair's pixels exist together)
+                for (int j = 0; j < 4; ++j) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float v0 = acc[i][j][r2] + bk, v1 = acc[i][j][r2 + 1] + bk;
+                    for (int i = 0; i < 2; ++i) {
+                        float v0 = acc[i][j][r2] + bk[i], v1 = acc[i][j][r2 + 1] + bk[i];
                         if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
                         const float got = swap_lane_pairs(odd ? v0 : v1);
                         const float lo = odd ? got : v0, hi = odd ? v1 : got;
                         struct alignas(4) Pair { T a, b; };
                         if (pok) *reinterpret_cast<Pair*>(yb + o[j] + (unsigned)(i * 64)) = Pair{from_f32<T>(lo), from_f32<T>(hi)};
-                        o[j] += ((r2 & 2) ? 6u : 2u) * kp;
                     }
-                    __builtin_amdgcn_sched_barrier(0);
+                    o[j] += ((r2 & 2) ? 6u : 2u) * kp;
                 }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] -= 32u * kp;                    // back to the first pixel for the other 32 filters
+                __builtin_amdgcn_sched_barrier(0);
             }
             return;
         }
