@@ -39,18 +39,18 @@ template <int WF> struct D16R {
     static constexpr int NTASK = WF == 2 ? 2 : 3;            // input tasks per thread and stage
 };
 
-// NHWC: x and y are [N][H][W][C] / [N][Ho][Wo][K].  The 8 channels of a pixel's vector are 16 contiguous bytes of x:
-// an input task is one pixel slot of one channel vector (a 16-byte load, a 16-byte LDS write, zeros where the slot
-// lies outside the image), the two vectors of a pixel on neighbouring lanes.  The multiplies take the pixel fragment
-// as the first operand, so a lane holds one FILTER and its registers the pixels: the 32 filters of a wave's half are
-// 64 contiguous bytes of a pixel of y.
-template <typename T, int WF, bool NHWC = false>
+// XN: x is [N][H][W][C].  The 8 channels of a pixel's vector are 16 contiguous bytes of x: an input task is one pixel
+// slot of one channel vector (a 16-byte load, a 16-byte LDS write, zeros where the slot lies outside the image), the
+// two vectors of a pixel on neighbouring lanes.  YN: y is [N][Ho][Wo][K].  The multiplies take the pixel fragment as
+// the first operand, so a lane holds one FILTER and its registers the pixels: the 32 filters of a wave's half are 64
+// contiguous bytes of a pixel of y.  The two are independent: a layer may read one layout and write the other.
+template <typename T, int WF, bool XN = false, bool YN = XN>
 __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restrict__ x, const T* __restrict__ W9,
                                                                T* __restrict__ y, D16Geom g, Epilogue ep) {
     typedef typename Mma<T>::vec vec;
     typedef D16R<WF> P;
-    constexpr int NTASK = NHWC ? (2 * P::XPLANE + 511) / 512 : P::NTASK;   // input tasks per thread and stage
-    constexpr int NX = NHWC ? NTASK : 8 * NTASK;                           // and the requests they make
+    constexpr int NTASK = XN ? (2 * P::XPLANE + 511) / 512 : P::NTASK;   // input tasks per thread and stage
+    constexpr int NX = XN ? NTASK : 8 * NTASK;                           // and the requests they make
     extern __shared__ __attribute__((aligned(16))) unsigned char d16r_smem[];     // [3][FB] filters, [2][XB] input
     unsigned char* const xsm = d16r_smem + 3 * P::FB;
     const int tid = threadIdx.x;
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     };
 
     // ---- input tasks of this thread: (channel vector v, LDS row, column pair); what does not depend on the tile ----
-    const int ntask = NHWC ? 2 * g.LR * g.PW : 2 * g.LR * g.PP;
+    const int ntask = XN ? 2 * g.LR * g.PW : 2 * g.LR * g.PP;
     int tpk[NTASK];                                          // LDS row | (first column of the pair relative to c0, + 8) << 8 | v << 20
     int ldsw[NTASK];                                         // byte offset of the pair's first slot inside an input stage (a multiple of
                                                              // 16, -16 for the pair left of a row) | bit 0 / 1: slot 0 / 1 exists;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
     for (int q = 0; q < NTASK; ++q) {
         const int t = tid + 512 * q;
-        if constexpr (NHWC) {
+        if constexpr (XN) {
             // task t: channel vector t & 1 of pixel slot t >> 1 (row-major over the LR x PW slots of a plane)
             // (tid + 512 q: the vector is the same for all tasks of a thread; row and column are recomputed per tile)
             tpk[q] = 0;
@@ -125,13 +125,13 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     auto prep_x = [&](const Tile& t) {
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
-            const int sl = min((tid + 512 * q) >> 1, g.LR * g.PW - 1);           // NHWC: the task's pixel slot
-            const int lr = NHWC ? sl / g.PW : tpk[q] & 0xFF, v = NHWC ? tid & 1 : tpk[q] >> 20;
+            const int sl = min((tid + 512 * q) >> 1, g.LR * g.PW - 1);           // NHWC source: the task's pixel slot
+            const int lr = XN ? sl / g.PW : tpk[q] & 0xFF, v = XN ? tid & 1 : tpk[q] >> 20;
             const int qq = t.oh0 + lr;                       // padded row index counted from image n0
             int dn = 0;
             for (int k = 1; k <= g.maxcross; ++k) dn += qq >= k * Hp ? 1 : 0;
             const int ih = qq - dn * Hp - g.pad;
-            if constexpr (NHWC) {
+            if constexpr (XN) {
                 const int iw = t.c0 + (sl - lr * g.PW) - g.pad;
                 const bool in = (ldsw[q] & 3) != 0 && t.n0 + dn < g.N && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
                 const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 1);
@@ -166,18 +166,18 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
         for (int q = 0; q < P::NF; ++q) dma_row(base + frow_src[q], lane_off, d16r_smem + slot * P::FB + frow_dst[q]);
     };
-    uint32_t raw[NHWC ? 1 : NTASK][8];
-    uint4 rawn[NHWC ? NTASK : 1];                            // NHWC: the 8 channels of a task's pixel
+    uint32_t raw[XN ? 1 : NTASK][8];
+    uint4 rawn[XN ? NTASK : 1];                            // NHWC source: the 8 channels of a task's pixel
     unsigned poff[NTASK];
     int req_cs = 0;                                          // the stage (inside its tile) whose input was requested last
     // piece 8q + e of a stage's input requests: channel e of task q.  A stage's second channel vector may lie past
     // C: the first one is loaded instead, and masked when it is written
     auto x_piece = [&](int idx) {
         if (idx == 0) req_cs = cx.cs;
-        if constexpr (NHWC) {
+        if constexpr (XN) {
             const int v = tid & 1;
             const bool vok = cx.cs * 16 + v * 8 < g.C;
-            rawn[NHWC ? idx : 0] = *reinterpret_cast<const uint4*>(xs + ((xoff[idx] & ~15u) - (vok ? 0u : (unsigned)v * 16u)));
+            rawn[XN ? idx : 0] = *reinterpret_cast<const uint4*>(xs + ((xoff[idx] & ~15u) - (vok ? 0u : (unsigned)v * 16u)));
             return;
         }
         const int q = idx >> 3, e = idx & 7;
@@ -186,24 +186,24 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             const bool vok = cx.cs * 16 + v * 8 < g.C;
             poff[q] = (xoff[q] & ~3u) - (vok ? 0u : (unsigned)v * 8u * hw2);
         }
-        raw[NHWC ? 0 : q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
+        raw[XN ? 0 : q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
         poff[q] += hw2;
     };
     auto x_commit = [&](int xslot) {                         // the stage requested through x_piece into input slot xslot
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
             if ((ldsw[q] & 3) == 0) continue;
-            const bool keep = (xoff[q] & 1u) && req_cs * 16 + (NHWC ? tid & 1 : tpk[q] >> 20) * 8 < g.C;
+            const bool keep = (xoff[q] & 1u) && req_cs * 16 + (XN ? tid & 1 : tpk[q] >> 20) * 8 < g.C;
             const uint32_t km = keep ? 0xFFFFFFFFu : 0u;
-            if constexpr (NHWC) {
-                const uint4 r = rawn[NHWC ? q : 0];
+            if constexpr (XN) {
+                const uint4 r = rawn[XN ? q : 0];
                 *reinterpret_cast<uint4*>(xsm + xslot * P::XB + (ldsw[q] & ~15)) = make_uint4(r.x & km, r.y & km, r.z & km, r.w & km);
                 continue;
             }
             uint32_t lo[4], hi[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t a = raw[NHWC ? 0 : q][2 * e] & km, b = raw[NHWC ? 0 : q][2 * e + 1] & km;
+                const uint32_t a = raw[XN ? 0 : q][2 * e] & km, b = raw[XN ? 0 : q][2 * e + 1] & km;
                 lo[e] = __builtin_amdgcn_perm(b, a, 0x05040100u);     // (a.lo16, b.lo16): the pair's first pixel
                 hi[e] = __builtin_amdgcn_perm(b, a, 0x07060302u);     // (a.hi16, b.hi16): its second pixel
             }
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         const bool rowok = g0 + 4 * wr < g.G;
         const int L = rowok ? dn * Hp + oh - t.oh0 : 0;
         xw_off = ((lh * P::XPLANE) + L * g.PW + (colok ? col : 0)) * 16;
-        if constexpr (NHWC) {
+        if constexpr (YN) {
             // element offset of (n, oh + j, the wave's first column, the wave's first filter); the lane's filter and
             // the register's column are added at the stores
             pc0 = t.c0 + 32 * wc;
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                 if (r < 0 || r > 2) continue;
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    if constexpr (NHWC) Mma<T>::run(b[t % 3], a[r][i], acc[i][j]);
+                    if constexpr (YN) Mma<T>::run(b[t % 3], a[r][i], acc[i][j]);
                     else Mma<T>::run(a[r][i], b[t % 3], acc[i][j]);
                 }
             }
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         unsigned ks = kstride2;
         asm volatile("" : "+s"(ks));
         char* const yb = reinterpret_cast<char*>(y);
-        if constexpr (NHWC) {
+        if constexpr (YN) {
             // register r of acc[i][j]: pixel column pc0 + 8*(r/4) + 4*lh + r%4 of row j, the lane's filter
             // k0c + 32*i + l32.  Two neighbouring lanes hold neighbouring filters and exchange values, so that each
             // stores one 4-byte pair of filters -- the even lane for the pixel of register r, the odd lane for that of
@@ -497,7 +497,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
         for (int i = 0; i < NX; ++i) x_piece(i);
         pending = true;
-        xs += NHWC ? (size_t)32 : (size_t)16 * HW * 2;                           // the next 16 channels
+        xs += XN ? (size_t)32 : (size_t)16 * HW * 2;                           // the next 16 channels
         advance(cx);
         need_prep = cx.cs == 0;
     };

@@ -789,18 +789,18 @@ bool direct16_rows_plan(const Geometry& g, D16Geom* d) {
 }
 inline int direct16_rows_wf(const Geometry& g) { return (g.K % 128 == 0 || g.K > 256) ? 2 : 1; }
 
-template <typename T, int WF, bool NHWC = false>
+template <typename T, int WF, bool XN = false, bool YN = XN>
 int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
     static bool attr_set = false;
     if (!attr_set) {
-        HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, NHWC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, XN, YN>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     D16R<WF>::LDS));
         attr_set = true;
     }
     // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs
     const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
     const long blocks = std::max<long>(8, std::min<long>(device_cus(), (tiles + 7) / 8 * 8) / 8 * 8);
-    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, NHWC>), dim3((unsigned)blocks), dim3(512), D16R<WF>::LDS, st, (const T*)x,
+    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN>), dim3((unsigned)blocks), dim3(512), D16R<WF>::LDS, st, (const T*)x,
                        (const T*)W9, (T*)y, d, ep);
     LAUNCH_CHECK("direct16_rows");
     return WINO_OK;
@@ -815,14 +815,16 @@ bool direct16_big(const Geometry& g, D16Geom* d) {
 }
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
     D16Geom d;
-    if (src == WINO_NHWC && dst == WINO_NHWC)
-        // NHWC tensors: the 8-wave kernel only; offsets inside a block's images and into y are 32-bit
-        return dtype != WINO_F32 && g.C % 8 == 0 && g.pad <= 1 && direct16_big(g, &d) &&
-               (long)g.N * g.K * g.Ho * g.Wo < (1L << 31) && (long)(d.maxcross + 1) * g.C * g.H * g.W * 2 < (1L << 32);
-    if (!(dtype != WINO_F32 && src == WINO_NCHW && dst == WINO_NCHW && g.C % 8 == 0 && g.W % 2 == 0 && g.pad <= 1 &&
-          (long)g.N * g.K * g.Ho * g.Wo < (1L << 31) && (long)g.C * g.H * g.W * 2 * 8 < (1L << 32) &&
-          direct16_plan(g, 4, false, &d)))
+    if (dtype == WINO_F32 || src == WINO_CHWN || dst == WINO_CHWN || g.C % 8 != 0 || g.pad > 1 ||
+        (long)g.N * g.K * g.Ho * g.Wo >= (1L << 31))
         return false;
+    if (src == WINO_NHWC || dst == WINO_NHWC) {
+        // an NHWC side: the 8-wave kernel only; offsets inside a block's images are 32-bit
+        if (!direct16_big(g, &d)) return false;
+        return src == WINO_NHWC ? (long)(d.maxcross + 1) * g.C * g.H * g.W * 2 < (1L << 32)
+                                : g.W % 2 == 0 && (long)g.C * g.H * g.W * 2 * 8 < (1L << 32);
+    }
+    if (!(g.W % 2 == 0 && (long)g.C * g.H * g.W * 2 * 8 < (1L << 32) && direct16_plan(g, 4, false, &d))) return false;
     // 2x2 pooling lives in the stores of the 8-wave kernel only
     return !(flags & WINO_FLAG_POOL2) || direct16_big(g, &d);
 }
@@ -850,9 +852,9 @@ int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const
 // D16_PACK_RUN both, D16_PACK only the bank (x and y are looked at, not touched), D16_RUN with a bank packed earlier
 // for tensors of the same alignment.
 enum { D16_PACK_RUN = 0, D16_PACK = 1, D16_RUN = 2 };
-int launch_direct16(int layout, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
-                    void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN) {
-    const bool nhwc = layout == WINO_NHWC;
+int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x,
+                    const void* w, void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN) {
+    const bool nhwc = layout == WINO_NHWC, ynhwc = dst == WINO_NHWC;
     if (misaligned(x, nhwc ? 16 : 4))
         return fail(WINO_ERR_UNSUPPORTED, "the 16-bit direct path loads column pairs (NHWC: channel vectors): x must be 4-byte (16-byte) aligned");
     D16Geom d;
@@ -861,7 +863,7 @@ int launch_direct16(int layout, int dtype, unsigned flags, const void* bias, con
     int npg = 4, wf = direct16_rows_wf(g);
     const bool pool = (flags & WINO_FLAG_POOL2) != 0;        // (pooled values are stored one by one: no alignment asked of y)
     const bool big = (pool || !misaligned(y, 4)) && direct16_big(g, &d);
-    if (nhwc && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of NHWC tensors: the 8-wave kernel's layer shapes, y 4-byte aligned");
+    if ((nhwc || ynhwc) && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of NHWC tensors: the 8-wave kernel's layer shapes, y 4-byte aligned");
     if (pool && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: pooling needs the 8-wave kernel's layer shapes");
     const bool rows = !big && direct16_plan(g, 4, true, &d) && (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
     if (!big && !rows) {
@@ -883,8 +885,12 @@ int launch_direct16(int layout, int dtype, unsigned flags, const void* bias, con
         LAUNCH_CHECK("direct16_pack");                                                                             \
     }                                                                                                              \
     if (mode == D16_PACK) return WINO_OK;                                                                          \
-    if (nhwc && wf == 2) return launch_direct16_rows_t<T, 2, true>(d, ep, x, W9, y, st);                           \
-    if (nhwc) return launch_direct16_rows_t<T, 1, true>(d, ep, x, W9, y, st);                                      \
+    if (nhwc && ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, true>(d, ep, x, W9, y, st);        \
+                         return launch_direct16_rows_t<T, 1, true, true>(d, ep, x, W9, y, st); }                   \
+    if (nhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, false>(d, ep, x, W9, y, st);                \
+                return launch_direct16_rows_t<T, 1, true, false>(d, ep, x, W9, y, st); }                           \
+    if (ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, true>(d, ep, x, W9, y, st);               \
+                 return launch_direct16_rows_t<T, 1, false, true>(d, ep, x, W9, y, st); }                          \
     if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, st);                                  \
     if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, st);                                             \
     if (rows) return launch_direct16_t<T, 4, true>(d, ep, x, W9, y, st);                                           \
@@ -948,7 +954,7 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     D16Geom d;
     const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d);
     if (plan8 && g.Ho >= 28 && g.Wo >= 28 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus()) return true;
-    if (src == WINO_NHWC || g.Ho < 48 || g.Wo < 48) return false;
+    if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 48 || g.Wo < 48) return false;
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
     return tiles >= 2L * device_cus();
 }
@@ -1046,7 +1052,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         const int rcb = ss.get(kCounterBytes + direct16_bank_bytes(g), &base);
         if (rcb) return rcb;
         StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-        return launch_direct16(src, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
+        return launch_direct16(src, dst, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
     }
     if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(ss, src, dst, dtype, flags, bias, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
@@ -1560,7 +1566,7 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
                    auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in)) {
             // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-            rc = launch_direct16(L.layout_in, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
+            rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
         } else {
             rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
                            L.wraw, L.U, bias, out, stream);
@@ -1625,7 +1631,7 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
         // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte NCHW and NHWC layers)
-        const bool direct16_layer = dtype != WINO_F32 && L.layout_in == L.layout_out && L.layout_in != WINO_CHWN && L.C % 8 == 0;
+        const bool direct16_layer = dtype != WINO_F32 && L.layout_in != WINO_CHWN && L.layout_out != WINO_CHWN && L.C % 8 == 0;
         if (e == hipSuccess && (L.C <= 4 || direct16_layer)) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         // what AUTO runs outside the F(2x2) kernels gets its filters prepared once as well
         if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && auto_f4(dtype, g)) {
@@ -1664,7 +1670,7 @@ int wino_stack_set_layer(wino_stack_t* s, int layer, const void* w, const void* 
     if (L.W9) {
         Geometry g;
         make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g);
-        rc = launch_direct16(L.layout_in, s->dtype, L.flags, nullptr, g, L.W9, w, L.W9, L.W9, (hipStream_t)stream, D16_PACK);   // (x, y: any aligned address)
+        rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, nullptr, g, L.W9, w, L.W9, L.W9, (hipStream_t)stream, D16_PACK);   // (x, y: any aligned address)
         if (rc) return rc;
     }
     L.has_bias = bias != nullptr;

@@ -75,9 +75,9 @@ typedef enum {
                                direct product by nothing but the multiplies (the stage it replaces is
                                comparison/GEMM.cuh:124-253; the reference's own direct kernel in tile geometry is
                                Conv_fuse, fusedTest/winotrans.cuh:1868).
-                               2-byte NHWC -> NHWC layers ([K][3][3][C] filters) with C a multiple of 8 and a 16-byte
-                               aligned x run on the larger of its two kernels (the 8-wave one) when the layer has its
-                               shape: output height a multiple of 4, even output width, K a multiple of 64, at least a
+                               2-byte layers with an NHWC side (NHWC -> NHWC, NCHW -> NHWC, NHWC -> NCHW; the filters in
+                               the source's layout), C a multiple of 8 and, from NHWC, a 16-byte aligned x run on the
+                               larger of its two kernels (the 8-wave one) when the layer has its shape: output height a multiple of 4, even output width, K a multiple of 64, at least a
                                tile for every other CU; other NHWC layers are refused (WINO_ERR_UNSUPPORTED).
                                Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (the
                                shape just named), not for C <= 4; needs the filter bank itself (not

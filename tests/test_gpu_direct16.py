@@ -105,6 +105,13 @@ def test_nhwc_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
         for n in (0, N - 1):
             want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], pad) + bias[ks][None, :, None, None], 0)
             assert np.array_equal(host(got[n:n + 1].permute(0, 3, 1, 2)[:, ks]), rounded(want.astype(np.float32), dtype, oracle)), (rep, n)
+    # the two sides are independent: NCHW in and NHWC out, NHWC in and NCHW out (the filters in the source's layout)
+    cross = ops.conv(dev(x, dtype), dev(w, dtype), pad, ops.NCHW, ops.NHWC, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+    assert torch.equal(cross, got)
+    cross = ops.conv(xd, wd, pad, ops.NHWC, ops.NCHW, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+    assert torch.equal(cross, nchw)
+    cross = ops.conv(xd, wd, pad, ops.NHWC, ops.NCHW, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+    assert torch.equal(cross, torch.nn.functional.max_pool2d(nchw.float(), 2).to(nchw.dtype))
     # 2x2 pooling in the stores (rounding is monotonic: the pooled tensor is the pooling of the unpooled one)
     pooled = ops.conv(xd, wd, pad, ops.NHWC, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
     assert tuple(pooled.shape) == (N, got.shape[1] // 2, got.shape[2] // 2, K)
