@@ -84,6 +84,9 @@ MEASURED_TRAFFIC = {
         (134.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv3_N32_counters.txt"),
     ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "bf16", "direct"):
         (534.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # the same kernel from NHWC tensors: 86.3 + 51.4 MB
+    ("vgg16_conv3_N32_C256_K256_H56", "NHWC", "bf16", "direct"):
+        (137.7e6, "profiles/direct16_rows_bf16_nhwc_vgg16_conv3_N32_counters.txt"),
     # gemm_rows_kernel in bf16: 271.5 MB fetched + 56.9 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "epilogue"):
         (328.4e6, "profiles/epilogue_bf16_nchw_vgg16_conv3_N32_counters.txt"),
