@@ -204,8 +204,12 @@ __global__ __launch_bounds__(256, 2) void direct16_kernel(const T* __restrict__ 
         fptr += fstep;
     };
     uint32_t raw[NTASK][8];
-    // a stage's second channel vector may lie past C: the first one is loaded instead, and masked
+    // A stage's second channel vector may lie past C: the first one is loaded instead, and masked.  So may the whole
+    // stage (the bank is padded to 32 channels, C is a multiple of 8: C = 8, 40, 72, ...): the first stage's channels
+    // are loaded then -- xs has moved on by cs stages -- so that no address leaves the tensor.
+    auto stage_base = [&](int cs) { return cs * 16 < g.C ? xs : xs - (size_t)cs * xstep; };
     auto x_load = [&](int cs) {
+        const char* const xb = stage_base(cs);
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
             const int v = tpk[q] >> 20;
@@ -213,7 +217,7 @@ __global__ __launch_bounds__(256, 2) void direct16_kernel(const T* __restrict__ 
             unsigned off = (xoff[q] & ~3u) - (vok ? 0u : (unsigned)v * 8u * hw2);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {     // a scalar base and a 32-bit offset per load
-                raw[q][e] = *reinterpret_cast<const uint32_t*>(xs + off);
+                raw[q][e] = *reinterpret_cast<const uint32_t*>(xb + off);
                 off += hw2;
             }
         }
@@ -235,7 +239,7 @@ __global__ __launch_bounds__(256, 2) void direct16_kernel(const T* __restrict__ 
                 const bool vok = cs * 16 + v * 8 < g.C;
                 poff[q] = (xoff[q] & ~3u) - (vok ? 0u : (unsigned)v * 8u * hw2);
             }
-            raw[q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
+            raw[q][e] = *reinterpret_cast<const uint32_t*>(stage_base(cs) + poff[q]);
             poff[q] += hw2;
         }
     };

@@ -14,7 +14,10 @@ pytestmark = pytest.mark.gpu
 # (N, C, K, H, W): blocks that span several images (14x14, 6x8), widths that do and do not fill a block's columns,
 # channel counts with half a stage left over (8, 24, 40), filter counts off the 64-filter tile, a single row
 SHAPES = [(2, 16, 64, 14, 14), (5, 8, 40, 6, 8), (1, 24, 130, 37, 20), (3, 40, 70, 9, 66), (2, 64, 64, 40, 34),
-          (1, 16, 8, 1, 2), (4, 32, 96, 28, 28), (2, 16, 64, 224, 224)]
+          (1, 16, 8, 1, 2), (4, 32, 96, 28, 28), (2, 16, 64, 224, 224),
+          # the bank is padded to 32 channels: with C = 8, 40, 72 the last stage of 16 channels lies wholly past C
+          # (its loads must stay inside the tensor: the first stage's channels again, masked)
+          (3, 72, 64, 30, 34), (2, 8, 128, 100, 130), (1, 40, 64, 64, 62)]
 
 
 @pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
