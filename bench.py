@@ -32,6 +32,8 @@ Prints ONE JSON line:
   configs      (default workload only, after its timed region) the other benchmark configurations, a few steps
                each: ms (median), effective TFLOP/s, the dominant kernel with its fraction of the MFMA peak and of
                min(MFMA peak, flop/byte x 8 TB/s); for the 13-layer f16 / bf16 passes also per layer
+               configs.reference_published_sweep: the reference's only committed latencies (NHWC, H=22, C=K=128,
+               N = 1 .. 128, layoutTest/NHWC/result.num) beside this library's, timed as the reference timed them
 """
 import argparse
 import json
@@ -275,6 +277,42 @@ def main():
         torch.cuda.empty_cache()
         return res
 
+    def published_sweep():
+        """The one measurement the reference commits (layoutTest/NHWC/result.num:1, made by layoutTest/NHWC/test.sh:3-8
+        with convModule_NHWC_padding.cu:84-99): wrapedConv_NHWC at H = W = 22, C = K = 128, pad 1, fp32, N = 1 .. 128, the
+        mean of 10 calls that each transform the filters and end in a device synchronisation -- on a GPU it does not name.
+        Timed here the same way (`us_sync_each_call`), and back to back on the stream (`us_back_to_back`, median)."""
+        ref_us = [51.939201, 53.334396, 83.395195, 107.584000, 180.300797, 320.105621, 645.052795, 1236.102295]
+        Ns, sync_us, b2b_us, algos = [1, 2, 4, 8, 16, 32, 64, 128], [], [], []
+        for N in Ns:
+            (x, w, y), = device_tensors([(N, 128, 128, 22)], LAYOUT["NHWC"], "f32", 0x22)
+
+            def call():
+                ops.conv(x, w, 1, LAYOUT["NHWC"], out=y)
+            r0 = time.perf_counter()
+            while time.perf_counter() - r0 < 0.05:
+                call()
+                torch.cuda.synchronize()
+            best = []
+            for _ in range(5):                     # five times the reference's 10-call loop; the median loop counts
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(10):
+                    call()
+                    torch.cuda.synchronize()
+                e1.record()
+                torch.cuda.synchronize()
+                best.append(e0.elapsed_time(e1) * 100.0)
+            sync_us.append(round(statistics.median(best), 2))
+            ms, _ = timed(call, 100, 10, group=10)
+            b2b_us.append(round(ms * 1e3, 2))
+            algos.append(ops.ALGO_NAMES[ops.pick_algo(LAYOUT["NHWC"], DT["f32"], N, 128, 128, 22, 22)])
+        return {"what": "wrapedConv_NHWC fp32, H=W=22, C=K=128, pad 1, filter transform in every call", "N": Ns,
+                "unit": "us per call", "us_sync_each_call": sync_us, "us_back_to_back": b2b_us, "algo": algos,
+                "reference_us": [round(v, 2) for v in ref_us], "reference_hardware": "an NVIDIA GPU the reference does not name",
+                "reference_source": "layoutTest/NHWC/result.num:1",
+                "reference_over_this": [round(r / v, 2) for r, v in zip(ref_us, sync_us)]}
+
     layers = layers_of(args.workload)
     multi = len(layers) > 1
     layout, tdt, dt, algo = LAYOUT[args.layout], TDT[args.dtype], DT[args.dtype], ALGO[args.algo]
@@ -434,6 +472,7 @@ def main():
         del tensors
         torch.cuda.empty_cache()
         out["configs"] = {name: other_config(wl, dty, lay) for (name, wl, dty, lay) in OTHER_CONFIGS}
+        out["configs"]["reference_published_sweep"] = published_sweep()
 
     if not args.no_cpu_baseline:
         import oracle
