@@ -1,5 +1,8 @@
-// mfma_rate: what the 16-bit matrix pipe of this machine sustains, measured -- the practical roof the direct
-// convolution kernels are read against.  Three loops on one workgroup per CU, all operands resident in LDS:
+// mfma_rate: what the matrix pipe of this machine sustains, measured -- the practical roof the direct convolution
+// kernels (16-bit) and the batched GEMMs (fp32) are read against.  Four loops on one workgroup per CU:
+//   0. v_mfma_f32_32x32x2_f32 back to back, 8 accumulators per wave, operands in registers (against 157.3 TFLOP/s:
+//      one multiply per 64 clocks and SIMD at 2.4 GHz);
+// and, all operands resident in LDS,
 //   1. v_mfma_f32_32x32x16_bf16 back to back, 8 accumulators per wave, no memory traffic;
 //   2. the same with R ds_read_b128 per 8 multiplies (operand fetch from LDS, one step ahead);
 //   3. the 18-step stage of the 8-wave direct kernel (direct16_rows.hpp): 36 fragment reads and 72 multiplies per
@@ -71,6 +74,36 @@ __global__ __launch_bounds__(512, 1) void plain_kernel(float* out, int iters, in
     if (s == 12345.678f) out[tid] = s;                       // never true: keeps the multiplies
 }
 
+// loop 0: v_mfma_f32_32x32x2_f32 back to back (64 clocks each), 8 accumulators per wave, operands in registers
+__global__ __launch_bounds__(512, 1) void plain32_kernel(float* out, int iters, int real) {
+    const int tid = threadIdx.x;
+    floatx16 acc[8];
+    for (int j = 0; j < 8; ++j)
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+    float f[8];
+    for (int q = 0; q < 8; ++q) {
+        unsigned h = (tid * 8 + q) * 2654435761u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        // real: random sign and mantissa, exponents of 0.125 .. 2; trivial: tiny integers read as floats (denormals)
+        f[q] = real ? __uint_as_float((h & 0x807FFFFFu) | ((124u + ((h >> 8) & 3u)) << 23)) : __uint_as_float(h >> 28);
+    }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[(t + m) & 7], f[(t + 3 * m + 1) & 7], acc[m], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if ((it & 15) == 15)
+            for (int j = 0; j < 8; ++j)
+                for (int r = 0; r < 16; ++r) acc[j][r] *= 1e-3f;
+    }
+    float s = 0;
+    for (int j = 0; j < 8; ++j)
+        for (int r = 0; r < 16; ++r) s += acc[j][r];
+    if (s == 12345.678f) out[tid] = s;
+}
+
 // loop 3: the stage schedule of direct16_rows_kernel (filter rows r, input rows rho, columns s; see there)
 __global__ __launch_bounds__(512, 1) void stage_kernel(float* out, int iters, int real, int PW) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -129,7 +162,8 @@ __global__ __launch_bounds__(512, 1) void stage_kernel(float* out, int iters, in
 }
 
 static int g_cus = 0;
-template <typename F> static void report(const char* name, int waves, int real, double mfma_per_simd, F launch) {
+template <typename F> static void report(const char* name, int waves, int real, double mfma_per_simd, F launch, int clocks = 32,
+                                          double peak = 2500.0) {
     hipEvent_t a, b;
     CHECK(hipEventCreate(&a));
     CHECK(hipEventCreate(&b));
@@ -142,9 +176,9 @@ template <typename F> static void report(const char* name, int waves, int real, 
         CHECK(hipEventSynchronize(b));
         CHECK(hipEventElapsedTime(&ms, a, b));
     }
-    const double frac = mfma_per_simd * 32 / 2.4e9 / (ms * 1e-3);
+    const double frac = mfma_per_simd * clocks / 2.4e9 / (ms * 1e-3);
     printf("%-34s %-8s data, %d waves/SIMD: %7.3f ms  %5.1f ns per multiply and SIMD  %.2f of nominal peak (%.0f TFLOP/s over %d CUs)\n", name,
-           real ? "real" : "trivial", waves / 4, ms, ms * 1e6 / mfma_per_simd, frac, frac * 2500.0 * g_cus / 256, g_cus);
+           real ? "real" : "trivial", waves / 4, ms, ms * 1e6 / mfma_per_simd, frac, frac * peak * g_cus / 256, g_cus);
 }
 
 int main() {
@@ -161,6 +195,8 @@ int main() {
     for (int real = 0; real < 2; ++real)
         for (int waves = 4; waves <= 8; waves += 4) {
             const double per_simd = (double)iters * 64 * waves / 4;
+            report("fp32 multiplies only (32x32x2)", waves, real, (double)(iters / 2) * 64 * waves / 4,
+                   [&] { hipLaunchKernelGGL(plain32_kernel, dim3(g_cus), dim3(64 * waves), 0, 0, out, iters / 2, real); }, 64, 157.3);
             report("multiplies only", waves, real, per_simd,
                    [&] { hipLaunchKernelGGL(plain_kernel<0>, dim3(g_cus), dim3(64 * waves), LDS_BYTES, 0, out, iters, real); });
             report("4 LDS reads per 8 multiplies", waves, real, per_simd,
