@@ -171,3 +171,20 @@ def test_vgg16_relu_chain_n32(oracle, dtype, layout):
     chain = rel(x16, x32)
     print(f"dtype={dtype} layout={layout} 13-layer chain at N=32 against the fp32 chain: {chain:.3e}")
     assert chain <= TOL[dtype], chain
+
+
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("N", [1, 2, 4, 8, 16, 32, 64, 128])
+def test_the_references_published_sweep(oracle, N, layout):
+    """The one shape the reference commits latencies for (layoutTest/NHWC/test.sh:3-8: `a.out <N> 22 128 128` for
+    N = 1 .. 128, the shape of its notebooks' accuracy checks at N = 64): the automatic choice -- F(2x2) up to
+    N = 8, F(4x4) beyond -- against the oracle's convolution of the whole batch, and against the F(2x2) pipeline."""
+    C = K = 128
+    H = 22
+    x, w = seeded(N, C, K, H, 0x2200 + N)
+    want = oracle.direct_conv_f32(host(x), host(w), 1)
+    xl, wl = to_layout(x, layout), to_layout(w, layout)
+    y = from_layout(ops.conv(xl, wl, 1, layout), layout)
+    assert oracle.rel_l2(host(y), want) <= TOL[ops.F32]
+    y2 = from_layout(ops.conv(xl, wl, 1, layout, algo=ops.ALGO_STAGED), layout)
+    assert rel(y, y2) <= 2e-5
