@@ -675,4 +675,189 @@ __global__ __launch_bounds__(256, 2) void gemm_128x128_walk_kernel(const T* __re
     __builtin_amdgcn_s_waitcnt(0x0F70);                  // the surplus requests of the last stages
 }
 
+// =============================================================================
+// The walking GEMM with the product stores of a pair spread over the first stages of the NEXT pair.
+//
+// In gemm_128x128_walk_kernel a wave stores its 64 x 64 block of a finished pair in one burst of 64 instructions,
+// 19 % of its time, during which it multiplies nothing; the matrix pipe of a SIMD idles whenever both of its waves are
+// out of their multiplies.  Here the finished accumulators move to a second register set and are stored two
+// instructions at a time behind the multiplies of the next pair's first RING stages (a quarter of the block per
+// stage: the ring slot names the quarter, so the reduction must be a multiple of RING stages long); only a
+// workgroup's last pair is stored in a burst.  224 registers instead of 160: still two workgroups per CU.
+// =============================================================================
+template <typename T, int NV, bool PK, int RING>
+__global__ __launch_bounds__(256, 2) void gemm_128x128_walk_spread_kernel(const T* __restrict__ U, const T* __restrict__ V,
+                                                                          float* __restrict__ Mo, int Cp, int Kp, long Pp,
+                                                                          int kTiles, int pTiles, int nxi, int groups) {
+    typedef typename Mma<T>::vec vec;
+    constexpr int CV = ChanVec<T>::n;
+    static_assert(RING == 4 && NV == 4, "a quarter of the block per ring slot, eight (group, i, j) steps per stage");
+    __shared__ vec As0[NV][GEMM_BM], As1[NV][GEMM_BM], As2[NV][GEMM_BM], As3[NV][GEMM_BM];
+    __shared__ vec Bs0[NV][GEMM_BN], Bs1[NV][GEMM_BN], Bs2[NV][GEMM_BN], Bs3[NV][GEMM_BN];
+    auto aslot = [&](auto sl) -> vec(*)[GEMM_BM] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return As0; else if constexpr (S == 1) return As1; else if constexpr (S == 2) return As2; else return As3;
+    };
+    auto bslot = [&](auto sl) -> vec(*)[GEMM_BN] {
+        constexpr int S = decltype(sl)::value;
+        if constexpr (S == 0) return Bs0; else if constexpr (S == 1) return Bs1; else if constexpr (S == 2) return Bs2; else return Bs3;
+    };
+    const int b = blockIdx.x;
+    const int xcd = b & 7, v = b >> 3;                   // ids go round-robin to the XCDs
+    const int gl = v / kTiles, ktile = v - gl * kTiles;
+    const int grp = gl * 8 + xcd;
+    const int units = pTiles * nxi;                      // pairs, q = xi * pTiles + tile column
+    if (grp >= groups || grp >= units) return;
+    const int mine = (units - grp + groups - 1) / groups;    // pairs grp, grp + groups, ...
+    const int k0 = ktile * GEMM_BM;
+    const int CQ = Cp / CV, nch = CQ / NV;               // a multiple of RING (the host checks)
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const unsigned lane_off = lane * 16;
+    const uint64_t stepU = (uint64_t)NV * Kp * 16, stepV = (uint64_t)NV * Pp * 16;
+    constexpr int WV = (RING - 2) * NV;
+
+    floatx16 acc[2][2], prv[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = prv[i][j][r] = 0.f;
+
+    // ---- load side: the pair whose rows are being requested (as in gemm_128x128_walk_kernel)
+    uint64_t sptr[NV];
+    int lq = grp, lst = 0;
+    auto point_at = [&](int q) {
+        const int xi = q / pTiles, ptile = q - xi * pTiles;
+        const vec* Ub = reinterpret_cast<const vec*>(U) + (size_t)xi * CQ * Kp + k0;
+        const vec* Vb = reinterpret_cast<const vec*>(V) + (size_t)xi * CQ * Pp + (size_t)ptile * GEMM_BN;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int piece = wave + 4 * i;
+            const int opnd = i / (NV / 2);
+            const int row = (piece >> 1) % NV, half = piece & 1;
+            sptr[i] = opnd ? reinterpret_cast<uint64_t>(Vb + (size_t)row * Pp + half * 64)
+                           : reinterpret_cast<uint64_t>(Ub + (size_t)row * Kp + half * 64);
+        }
+    };
+    point_at(lq);
+    auto stage_load = [&](auto sl) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int piece = wave + 4 * i;
+            const int opnd = i / (NV / 2);
+            const int row = (piece >> 1) % NV, half = piece & 1;
+            dma_row(sptr[i], lane_off, opnd ? &bslot(sl)[row][half * 64] : &aslot(sl)[row][half * 64]);
+        }
+        if (++lst == nch) {
+            lst = 0;
+            if (lq + groups < units) {
+                lq += groups;
+                point_at(lq);
+            } else {
+                lst = nch - 1;                           // past the last pair: the last stage again (never read)
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) sptr[i] += (i / (NV / 2)) ? stepV : stepU;
+        }
+    };
+    // ---- compute side
+    long pitch = PK ? (long)Kp : Pp;                     // (opaque: the store addresses are not to be computed ahead
+    asm volatile("" : "+s"(pitch));                      //  of the loop and kept in registers across it)
+    auto block_of = [&](int q) {                         // this lane's corner of pair q's 64 x 64 block
+        const int xi = q / pTiles, ptile = q - xi * pTiles;
+        const long p0 = (long)ptile * GEMM_BN;
+        return Mo + (size_t)xi * Kp * Pp + (PK ? (size_t)(p0 + wm * 64 + 4 * lh) * pitch + k0 + wn * 64 + l32
+                                               : (size_t)(k0 + wm * 64 + 4 * lh) * pitch + p0 + wn * 64 + l32);
+    };
+    float* Mprev = nullptr;
+    // store n = 0..63 of the previous pair's block: rows i = n / 32, register (n / 2) % 16, half n % 2
+    // (n is a constant once the loops around the call are unrolled)
+    auto store_one = [&](int n) {
+        const int i = n >> 5, r = (n >> 1) & 15, j = n & 1;
+        Mprev[(size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * pitch + j * 32] = prv[i][j][r];
+        prv[i][j][r] = 0.f;
+    };
+    // The wait before the barrier is for the rows this wave requested three stages ago: "all but my newest WV
+    // operations" -- interleaved stores only make it wait for more than it must.
+    auto stage = [&](auto sl, auto with_stores) {
+        constexpr int S = decltype(sl)::value;
+        constexpr bool ST = decltype(with_stores)::value;
+        __builtin_amdgcn_s_waitcnt((WV & 0xF) | (0x7 << 4) | (0xF << 8) | ((WV >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        stage_load(std::integral_constant<int, (decltype(sl)::value + RING - 1) % RING>{});
+        __builtin_amdgcn_sched_barrier(0);
+        vec a[2][2], bq[2][2];
+        auto frag_load = [&](int g) {
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
+                const vec fa = aslot(sl)[2 * g + lh][(PK ? wn : wm) * 64 + qq * 32 + l32];
+                const vec fb = bslot(sl)[2 * g + lh][(PK ? wm : wn) * 64 + qq * 32 + l32];
+                a[g & 1][qq] = PK ? fb : fa;
+                bq[g & 1][qq] = PK ? fa : fb;
+            }
+        };
+        frag_load(0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            if (g == 0) frag_load(1);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    Mma<T>::run(a[g & 1][i], bq[g & 1][j], acc[i][j]);
+                    if constexpr (ST) {              // two of the quarter's sixteen stores behind every step
+                        const int n = 16 * S + 2 * (4 * g + 2 * i + j);
+                        __builtin_amdgcn_sched_barrier(0);
+                        store_one(n);
+                        store_one(n + 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for_each_const(std::make_integer_sequence<int, RING - 1>{}, stage_load);
+    int cq = grp;
+#pragma unroll 1
+    for (int pair = 0; pair < mine; ++pair) {
+        // the first RING stages carry the previous pair's stores (spread over two or four times as many stages,
+        // 8 or 4 stores to a stage, measured 1-3 % slower)
+        if (pair > 0) for_each_const(std::make_integer_sequence<int, RING>{}, [&](auto sl) { stage(sl, std::true_type{}); });
+        else for_each_const(std::make_integer_sequence<int, RING>{}, [&](auto sl) { stage(sl, std::false_type{}); });
+#pragma unroll 1
+        for (int st = RING; st < nch; st += RING)
+            for_each_const(std::make_integer_sequence<int, RING>{}, [&](auto sl) { stage(sl, std::false_type{}); });
+        // the pair's reduction is complete: its sums move to the second register set
+        Mprev = block_of(cq);
+        cq += groups;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    prv[i][j][r] = acc[i][j][r];
+                    acc[i][j][r] = 0.f;
+                }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  // the surplus requests of the last stages
+    // the last pair's block, in one go
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float* row = Mprev + (size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * pitch;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) row[j * 32] = prv[i][j][r];
+        }
+}
+
 }  // namespace wino
