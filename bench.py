@@ -69,9 +69,9 @@ WORKLOADS = {
 # script (the summary file holds the counters and the copy-kernel scale factor), keyed by
 # (workload, layout, dtype, resolved algo): (bytes, summary under profiles/).
 MEASURED_TRAFFIC = {
-    # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_kernel): 320.7 MB fetched + 231.2 MB written
+    # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_spread_kernel): 320.9 MB fetched + 231.2 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged_f4"):
-        (551.9e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+        (552.1e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
     # 636.1 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"):
         (747.2e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_counters.txt"),
@@ -105,8 +105,8 @@ OTHER_CONFIGS = [
     ("cfg5_vgg16_all13_N32_bf16", "vgg16_all13", "bf16", "NCHW"),
     ("cfg5_vgg16_all13_N32_bf16_NHWC", "vgg16_all13", "bf16", "NHWC"),
 ]
-KERNEL_OF = {"staged": "gemm_128x128_kernel / gemm_128x128_walk_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
-             "staged_f4": "gemm_128x128_kernel / gemm_128x128_walk_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel"}
+KERNEL_OF = {"staged": "gemm_128x128_kernel / gemm_128x128_walk_kernel / gemm_128x128_walk_spread_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
+             "staged_f4": "gemm_128x128_walk_spread_kernel / gemm_128x128_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel"}
 
 
 def main():
