@@ -153,6 +153,8 @@ def wino_gemm(U, V, m=2):
     """Mo[t*t][K][P] = sum_c U[xi][c][k] V[xi][c][p]."""
     nxi, C, K = U.shape
     P = V.shape[2]
+    assert nxi == (m + 2) ** 2 and V.shape[:2] == (nxi, C), "all coordinate planes of both operands"
+    assert U.flags.c_contiguous and V.flags.c_contiguous and U.dtype == np.float32 and V.dtype == np.float32
     Mo = np.empty((nxi, K, P), np.float32)
     _ck(lib().oracle_wino_gemm(m, C, K, P, _p(U), _p(V), _p(Mo)), "gemm")
     return Mo

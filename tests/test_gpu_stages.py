@@ -128,6 +128,34 @@ def test_batched_gemm(oracle, C, K, P, porder):
     assert np.array_equal(Mo[:, :K, :P], want)
 
 
+@pytest.mark.parametrize("porder", [ops.PRODUCT_KP, ops.PRODUCT_PK])
+@pytest.mark.parametrize("C,K,P", [(64, 256, 6272), (128, 256, 6272), (256, 128, 12544), (256, 256, 6300), (512, 256, 6272),
+                                   (48, 256, 6272), (80, 256, 6272)])
+def test_batched_gemm_over_the_resident_set(oracle, C, K, P, porder):
+    """Shapes with several rounds of work for a resident set of workgroups: the GEMM then walks its (coordinate, tile
+    column) pairs, with a finished pair's product stored during the next pair's first stages when the reduction is
+    a multiple of four stages long (4, 8, 16, 32 here; 3 and 5: stored in one go).  Small integers: the product is
+    exact, compared over all of it with a device-side fp32 matrix product (itself exact on these values) and, for the
+    first and the last 70 tiles, with the oracle."""
+    g = ops.geometry(ops.F32, 1, C, K, 4, 4, 1)
+    Cp, Kp = g["Cp"], g["Kp"]
+    Pp = (P + 127) // 128 * 128
+    gen = torch.Generator(device="cuda").manual_seed(C * 7 + K)
+    Ud = torch.zeros((16, Cp, Kp), device="cuda")
+    Vd = torch.zeros((16, Cp, Pp), device="cuda")
+    Ud[:, :C, :K] = torch.randint(-3, 4, (16, C, K), device="cuda", generator=gen).float()
+    Vd[:, :C, :P] = torch.randint(-5, 6, (16, C, P), device="cuda", generator=gen).float()
+    pack = lambda t: t.reshape(16, Cp // 4, 4, -1).permute(0, 1, 3, 2).contiguous()
+    Mo = ops.batched_gemm(pack(Ud), pack(Vd), C, K, P, porder)
+    if porder == ops.PRODUCT_PK:
+        Mo = Mo.transpose(1, 2)
+    want = torch.matmul(Ud.transpose(1, 2), Vd)               # [16][Kp][Pp]
+    assert torch.equal(Mo[:, :K, :P], want[:, :K, :P])
+    for p0 in (0, P - 70):
+        ref = oracle.wino_gemm(np.ascontiguousarray(host(Ud[:, :C, :K])), np.ascontiguousarray(host(Vd[:, :C, p0:p0 + 70])))
+        assert np.array_equal(host(Mo[:, :K, p0:p0 + 70]), ref)
+
+
 def test_batched_gemm_floats(oracle):
     C, K, P = 64, 128, 256
     U = synth.normal(16 * C * K, 8, 0.2).reshape(16, C, K)
