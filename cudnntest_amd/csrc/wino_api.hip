@@ -391,12 +391,14 @@ int launch_gemm_t(int nxi, int Cp, int Kp, long Pp, const void* U, const void* V
     constexpr int RING = sizeof(T) == 4 ? 4 : 3;     // from measurements, see gemm.hpp
     // the walking kernel: an uncut reduction of at most 24 stages (beyond, the starts and ends it saves weigh less
     // than its 3 % slower loop: C = 512 in fp32 measured 488 against 470 us, C = 256 242 against 256 us), and
-    // work for several rounds of the resident set
+    // work for three rounds of the resident set
     const int slots = 2 * device_cus(), per_xcd = slots / 8 / std::max(kTiles, 1);
     // (fp32 reductions of a multiple of four stages run the variant that spreads a pair's stores over the next
     // pair's first stages: C = 512 measured 456 against 466 us, C = 256 226 against 242 us)
     const int walk_max = sizeof(T) == 4 && NV == 4 && chunks % RING == 0 ? 32 : 24;
-    if (splits == 1 && chunks <= walk_max && per_xcd >= 1 && (long)pTiles * nxi >= 3L * per_xcd * 8) {
+    // (and from two pairs to a group: N = 64, C = K = 512 at 14 x 14, 2.25 pairs to a group, 157 against 163 us)
+    const long walk_min = sizeof(T) == 4 && NV == 4 && chunks % RING == 0 ? 2 : 3;
+    if (splits == 1 && chunks <= walk_max && per_xcd >= 1 && (long)pTiles * nxi >= walk_min * per_xcd * 8) {
         const int groups = per_xcd * 8;
         if constexpr (sizeof(T) == 4 && NV == 4) {
             if (chunks % RING == 0) {
