@@ -434,7 +434,7 @@ __global__ __launch_bounds__(256) void input_transform_nchw_small_kernel(const T
                                                                          int in_blocks, int stepC, int stepH,
                                                                          int stepW, FilterJob fj) {
     constexpr int CV = ChanVec<T>::n;
-    constexpr int NB = 8;                              // loads in flight per thread
+    constexpr int NB = M == 4 ? 16 : 8;                // loads in flight per thread (fp32 28 x 28 planes: 16 measured 72 against 75 us)
     extern __shared__ __attribute__((aligned(16))) unsigned char in_smem_raw[];
     int bid = blockIdx.x;
     if constexpr (M == 4) {
