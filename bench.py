@@ -320,8 +320,9 @@ def main():
 
     stack = None
     if args.workload == "vgg16_stack":
-        if args.algo == "staged_f4":
-            print("bench.py: the stack driver has no F(4x4,3x3) mode", file=sys.stderr)
+        if args.algo in ("staged_f4", "direct"):
+            print("bench.py: the stack driver takes auto (which prepares F(4x4) and direct-path filters per layer where "
+                  "it will run them), staged, epilogue or fused as a layer's algorithm", file=sys.stderr)
             sys.exit(2)
         pools = {1, 3, 6, 9, 12}
         descs = [dict(K=K, layout_in=layout, layout_out=layout, relu=True, pool=i in pools, algo=algo)
@@ -408,7 +409,8 @@ def main():
     traffic, traffic_source = MEASURED_TRAFFIC.get((args.workload, args.layout, args.dtype, algo_label), (None, None))
     roofline = {"bound": "mfma", "kernel": KERNEL_OF.get(algo_label, "per-layer choice"),
                 "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
+                "frac": round(achieved / peak, 4), "time_source": "HIP events the library records around the kernel on its launch stream",
+                "traffic": traffic, "traffic_source": traffic_source,
                 "flops_per_launch": gemm_flops if not multi else None}
 
     N0, C0, K0, H0 = layers[0]
@@ -428,6 +430,7 @@ def main():
         "metric": "effective TFLOP/s (direct-conv FLOPs), VGG-16 3x3 layer, N=32",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "ms_per_step_wall_mean": round(ms_wall, 4),
+        "value_wall_mean": round(direct_flops / (ms_wall * 1e-3) / 1e12, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": args.workload, "layers": len(layers), "N": N0, "C": C0, "K": K0, "H": H0, "W": H0,
@@ -491,6 +494,12 @@ def main():
                                           "the first of the 13 layers once (all N images, convolution and ReLU)") +
                                          ", fp32 direct convolution, OpenMP",
                                "ms": round((c1 - c0) * 1e3, 1)}
+    # the last key of the line (a record that keeps only the line's tail still holds every configuration):
+    # name -> [ms, effective TFLOP/s, AUTO's pipeline, dominant kernel's fraction of min(MFMA peak, flop/byte x 8 TB/s)]
+    if "configs" in out:
+        out["configs_summary"] = {name: [c["ms"], c["effective_tflops"], c.get("algo", "per layer"),
+                                         c.get("frac_of_attainable", c.get("frac"))]
+                                  for name, c in out["configs"].items() if "ms" in c}
     print(json.dumps(out), flush=True)
 
 

@@ -55,6 +55,7 @@ SYMBOLS = {
     "wino_f4_input_transform": (_i, [_i] * 8 + [_vp, _vp, _vp]),
     "wino_f4_batched_gemm": (_i, [_i, _i, _i, _i, _l, _vp, _vp, _vp, _vp]),
     "wino_f4_output_transform": (_i, [_i, _i, _i, _i, _u, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "wino_f4_gemm_output": (_i, [_i, _i, _i, _u, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "wino_layout_transform": (_i, [_i] * 7 + [_vp, _vp, _vp]),
     "wino_stage_timing": (_i, [_i]),
     "wino_stage_times": (_i, [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(_l)]),

@@ -59,6 +59,9 @@ template <> struct Mma<bf16_t> {
 // issued one instruction earlier included, which leaves a wave's matrix pipe idle for an LDS round trip at
 // every step.  Written out, the load is invisible to that bookkeeping: every kernel that uses it waits for its
 // rows itself (s_waitcnt vmcnt before the workgroup's barrier), which they did already.
+// M0 is written here and not named as a clobber: it is a reserved register for this compiler (which refuses it on a
+// clobber list as undefined behaviour), never holds a value across instructions, and is set by the compiler itself
+// right before each of its own uses.
 __device__ __forceinline__ void dma_row(uint64_t sbase, unsigned lane_off, void* lds_dst) {
     const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_dst);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(sbase) : "memory");

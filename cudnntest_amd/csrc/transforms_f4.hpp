@@ -295,36 +295,12 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
     }
 }
 
-// ---- output transform ------------------------------------------------------------------------------
-// PK = false: Mo[36][Kp][Pp], thread per (tile p, filter k), p fastest
-// PK = true : Mo[36][Pp][Kp], thread per (filter k, tile p), k fastest
-// Bias, ReLU and 2x2 max pooling as in the F(2x2) output stage: with pooling, s describes the pooled tensor
-// (Ho/2 x Wo/2) and a tile gives 2x2 pooled values; a window cut by the border is dropped.
-template <typename T, bool PK>
-__global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* __restrict__ Mo, T* __restrict__ y,
-                                                                   ActStrides s, int N, int K, int Ho, int Wo, int th,
-                                                                   int tw, long P, long Pp, int Kp, int order,
-                                                                   Epilogue ep) {
-    long p;
-    int k;
-    if (PK) {
-        k = blockIdx.x * blockDim.x + threadIdx.x;
-        p = (long)blockIdx.y * blockDim.y + threadIdx.y;
-    } else {
-        p = (long)blockIdx.x * blockDim.x + threadIdx.x;
-        k = blockIdx.y;
-    }
-    if (p >= P || k >= K) return;
-    const size_t plane = (size_t)Kp * Pp;
-    const float* mp = PK ? Mo + (size_t)p * Kp + k : Mo + (size_t)k * Pp + p;
-    float m[36];
-#pragma unroll
-    for (int xi = 0; xi < 36; ++xi) m[xi] = mp[xi * plane];
-    float o[4][4];
-    output_tile_transform_f4(m, o);
-    int n, ty, tx;
-    decode_tile(p, order, N, th, tw, n, ty, tx);
-    const float bv = bias_of<T>(ep, k);
+// The 4x4 outputs o of tile (n, ty, tx) and filter k on their way out: bias, ReLU, 2x2 max pooling (s then describes
+// the pooled tensor, Ho/2 x Wo/2, a tile gives 2x2 pooled values and a window cut by the border is dropped), stores --
+// one 4-element store per output row where the destination is W-contiguous with rows a multiple of 4 wide.
+template <typename T>
+__device__ __forceinline__ void store_tile_f4(T* __restrict__ y, const ActStrides& s, int n, int k, int ty, int tx, int Ho,
+                                              int Wo, float (&o)[4][4], const Epilogue& ep, float bv) {
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
@@ -368,6 +344,38 @@ __global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* _
             const int oh = 4 * ty + a, ow = 4 * tx + b;
             if (oh < Ho && ow < Wo) yp[oh * s.h + ow * s.w] = from_f32<T>(o[a][b]);
         }
+}
+
+// ---- output transform ------------------------------------------------------------------------------
+// PK = false: Mo[36][Kp][Pp], thread per (tile p, filter k), p fastest
+// PK = true : Mo[36][Pp][Kp], thread per (filter k, tile p), k fastest
+// Bias, ReLU and 2x2 max pooling as in the F(2x2) output stage: with pooling, s describes the pooled tensor
+// (Ho/2 x Wo/2) and a tile gives 2x2 pooled values; a window cut by the border is dropped.
+template <typename T, bool PK>
+__global__ __launch_bounds__(256) void output_transform_f4_kernel(const float* __restrict__ Mo, T* __restrict__ y,
+                                                                   ActStrides s, int N, int K, int Ho, int Wo, int th,
+                                                                   int tw, long P, long Pp, int Kp, int order,
+                                                                   Epilogue ep) {
+    long p;
+    int k;
+    if (PK) {
+        k = blockIdx.x * blockDim.x + threadIdx.x;
+        p = (long)blockIdx.y * blockDim.y + threadIdx.y;
+    } else {
+        p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+        k = blockIdx.y;
+    }
+    if (p >= P || k >= K) return;
+    const size_t plane = (size_t)Kp * Pp;
+    const float* mp = PK ? Mo + (size_t)p * Kp + k : Mo + (size_t)k * Pp + p;
+    float m[36];
+#pragma unroll
+    for (int xi = 0; xi < 36; ++xi) m[xi] = mp[xi * plane];
+    float o[4][4];
+    output_tile_transform_f4(m, o);
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    store_tile_f4<T>(y, s, n, k, ty, tx, Ho, Wo, o, ep, bias_of<T>(ep, k));
 }
 
 }  // namespace wino

@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -15,6 +16,7 @@
 #include "direct16.hpp"
 #include "direct16_rows.hpp"
 #include "gemm.hpp"
+#include "gemm_rows_f4.hpp"
 #include "transforms.hpp"
 #include "transforms_f4.hpp"
 
@@ -216,8 +218,29 @@ inline size_t tail_part_bytes(int dtype, const Geometry& g) {
     return (size_t)rows_tail_groups(dtype, g) * 8 * ((g.K + GO_T - 1) / GO_T) * 4 * 64 * 256 * sizeof(float);
 }
 
+// The F(4x4) GEMM with the output transform in its epilogue (gemm_rows_f4.hpp): 64 x 64 patches dealt to the 8 XCDs
+// (to as many as there are patches), one persistent workgroup per CU (fewer when that would leave a workgroup less
+// than 4 stages), each with room for one patch's partial outputs and an arrival counter.  fp32 only.
+struct F4RowsPlan {
+    int kTiles, pTiles, nparts, grid;
+    size_t part_bytes;
+};
+bool f4_rows_plan(int dtype, const Geometry& g, F4RowsPlan* p) {
+    if (dtype != WINO_F32 || g.m != 4) return false;
+    p->kTiles = (g.K + GF4_T - 1) / GF4_T;
+    p->pTiles = (int)((g.P + GF4_T - 1) / GF4_T);
+    const long patches = (long)p->kTiles * p->pTiles;
+    p->nparts = (int)std::min<long>(8, patches);
+    const long per_part = patches / p->nparts * 6 * (g.Cp / 16);                 // stages of the XCD with the fewest patches
+    const long sx = std::max<long>(1, std::min<long>(std::min<long>(device_cus() / 8, (long)(kCounterBytes / sizeof(int)) / 8), per_part / 4));
+    p->grid = (int)sx * 8;
+    p->part_bytes = (size_t)p->grid * GF4_PART * sizeof(float);
+    return true;
+}
+
 // What a pipeline keeps in scratch: STAGED (and the F(4x4) mode) U, V and the product; EPILOGUE U, V and the
-// partial sums of its cut-up workgroups; FUSED U only.  The default is the largest of them.
+// partial sums of its cut-up workgroups (EPILOGUE_F4: of the workgroups that share a patch); FUSED U only.
+// The default is the largest of them.
 Scratch scratch_layout(const Geometry& g, int dtype, int algo = WINO_ALGO_STAGED) {
     const size_t es = dtype_size(dtype);
     const size_t nxi = (size_t)(g.m + 2) * (g.m + 2);
@@ -232,7 +255,9 @@ Scratch scratch_layout(const Geometry& g, int dtype, int algo = WINO_ALGO_STAGED
     s.m_off = s.v_off + al(nxi * (size_t)g.Cp * g.Pp * es);
     const size_t copies = g.m == 2 ? (size_t)gemm_splits(dtype, g.Cp, g.Kp, g.Pp) : 1;
     const size_t product = copies * nxi * (size_t)g.Kp * g.Pp * sizeof(float);
-    s.total = s.m_off + al(algo == WINO_ALGO_EPILOGUE ? tail_part_bytes(dtype, g) : product);
+    F4RowsPlan fp;
+    if (algo == WINO_ALGO_EPILOGUE_F4 && f4_rows_plan(dtype, g, &fp)) s.total = s.m_off + al(fp.part_bytes);
+    else s.total = s.m_off + al(algo == WINO_ALGO_EPILOGUE ? tail_part_bytes(dtype, g) : product);
     return s;
 }
 
@@ -650,6 +675,30 @@ int launch_f4_output(int layout, int order, int porder, unsigned flags, const vo
     return WINO_OK;
 }
 
+// part: room for plan.part_bytes; cnt: the arena's arrival counters (zero between launches)
+int launch_f4_gemm_rows(int dst, int order, unsigned flags, const void* bias, const Geometry& g, const F4RowsPlan& plan,
+                        const void* U, const void* V, void* y, float* part, int* cnt, hipStream_t st) {
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set.load(std::memory_order_acquire)) {
+        HIP_TRY(hipFuncSetAttribute((const void*)gemm_rows_f4_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GF4_LDS));
+        HIP_TRY(hipFuncSetAttribute((const void*)gemm_rows_f4_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GF4_LDS));
+        attr_set.store(true, std::memory_order_release);
+    }
+    const ActStrides ys = out_strides(dst, flags, g.N, g.K, g.Ho, g.Wo);
+    const Epilogue ep = make_epilogue(flags, bias);
+    const int spin_limit = 1 << 22;                       // x ~1 us: seconds, against a wait that is normally over before it starts
+    if (dst == WINO_NHWC)
+        hipLaunchKernelGGL((gemm_rows_f4_kernel<true>), dim3((unsigned)plan.grid), dim3(512), GF4_LDS, st, (const float*)U,
+                           (const float*)V, (float*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, g.Pp, order, ep,
+                           plan.kTiles, plan.pTiles, plan.nparts, part, cnt, spin_limit);
+    else
+        hipLaunchKernelGGL((gemm_rows_f4_kernel<false>), dim3((unsigned)plan.grid), dim3(512), GF4_LDS, st, (const float*)U,
+                           (const float*)V, (float*)y, ys, g.N, g.K, g.Ho, g.Wo, g.th, g.tw, g.P, g.Cp, g.Kp, g.Pp, order, ep,
+                           plan.kTiles, plan.pTiles, plan.nparts, part, cnt, spin_limit);
+    LAUNCH_CHECK("f4_gemm_rows");
+    return WINO_OK;
+}
+
 #define DISPATCH_DTYPE(dtype, CALL)                          \
     switch (dtype) {                                         \
     case WINO_F32: { typedef float T; return CALL; }         \
@@ -806,11 +855,11 @@ inline int direct16_rows_wf(const Geometry& g) { return (g.K % 128 == 0 || g.K >
 
 template <typename T, int WF, bool XN = false, bool YN = XN>
 int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};    // (per instantiation; setting it twice from two threads is harmless)
+    if (!attr_set.load(std::memory_order_acquire)) {
         HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, XN, YN>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     D16R<WF>::LDS));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs
     const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
@@ -846,11 +895,11 @@ bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g)
 
 template <typename T, int NPG, bool ROWS>
 int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
-    static bool attr_set = false;                // (per instantiation; the attribute is a property of the kernel)
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};    // (per instantiation; the attribute is a property of the kernel)
+    if (!attr_set.load(std::memory_order_acquire)) {
         HIP_TRY(hipFuncSetAttribute((const void*)direct16_kernel<T, NPG, ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     2 * D16_BUF));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     // persistent grid: two workgroups per CU (or as many as there are tiles), a multiple of the 8 XCDs
     const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
@@ -963,9 +1012,11 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
 // at C = K = 128, H = 112; 130 against 164 us at C = K = 256, H = 56; 75 against 79 and 127 against 135 us for the
 // two 28 x 28 shapes, which only the 8-wave kernel wins; at 14 x 14 the Winograd pipelines are faster, 55 against
 // 98 us; NHWC tensors, 8-wave kernel only: 236 against 462, 92 against 150, 143 against 257, 73 against 96, 122
-// against 170, 68 against 79, 117 against 133 us).  x: the input tensor if known (its alignment decides).
-bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x) {
+// against 170, 68 against 79, 117 against 133 us).  x, y: the tensors if known (their alignment decides: with an NHWC
+// side only the 8-wave kernel runs, and it stores 4-byte pairs unless it pools).
+bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y) {
     if (!direct16_ok(src, dst, dtype, flags, g) || misaligned(x, src == WINO_NHWC ? 16 : 4)) return false;
+    if ((src == WINO_NHWC || dst == WINO_NHWC) && !(flags & WINO_FLAG_POOL2) && misaligned(y, 4)) return false;
     D16Geom d;
     const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d);
     if (plan8 && g.Ho >= 28 && g.Wo >= 28 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus()) return true;
@@ -986,21 +1037,36 @@ bool auto_f4(int dtype, const Geometry& g) {
     const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
     return tiles4 >= 512;
 }
-int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, bool have_w) {
+// which of the two F(4x4) pipelines then runs (g4: the layer's F(4x4) geometry)
+int auto_f4_algo(int dtype, const Geometry& g4) {
+    F4RowsPlan plan;
+    (void)plan;
+    (void)dtype;
+    (void)g4;
+    return WINO_ALGO_STAGED_F4;
+}
+int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y, bool have_w) {
     if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
-    if (have_w && auto_direct16(src, dst, dtype, flags, g, x)) return WINO_ALGO_DIRECT;
-    if (have_w && auto_f4(dtype, g)) return WINO_ALGO_STAGED_F4;
+    if (have_w && auto_direct16(src, dst, dtype, flags, g, x, y)) return WINO_ALGO_DIRECT;
+    if (have_w && auto_f4(dtype, g)) {
+        Geometry g4;
+        make_geometry(dtype, g.N, g.C, g.K, g.H, g.W, g.pad, &g4, 4);
+        return auto_f4_algo(dtype, g4);
+    }
     const int algo = pick_algo(src, dtype, g);
     return algo == WINO_ALGO_FUSED && g.pad > 1 ? WINO_ALGO_EPILOGUE : algo;   // the single kernel masks one ring of padding
 }
 
-int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned flags, const void* bias, int N, int C, int K,
-                 int H, int W, int pad, const void* x, const void* w, const void* Upre, void* y, void* stream) {
+int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo, unsigned flags, const void* bias, int N, int C,
+                 int K, int H, int W, int pad, const void* x, const void* w, const void* Upre, void* y, void* stream) {
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g, 4))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
     hipStream_t st = (hipStream_t)stream;
-    const Scratch sc = scratch_layout(g, dtype);
+    F4RowsPlan plan;
+    if (algo == WINO_ALGO_EPILOGUE_F4 && !f4_rows_plan(dtype, g, &plan))
+        return fail(WINO_ERR_UNSUPPORTED, "the F(4x4) pipeline with the output transform in the GEMM is built for fp32 tensors");
+    const Scratch sc = scratch_layout(g, dtype, algo);
     void* base = nullptr;
     int rc = ss.get(sc.total, &base);
     if (rc) return rc;
@@ -1025,6 +1091,10 @@ int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, unsigned 
         DISPATCH_DTYPE_RC(rc, dtype, launch_f4_input<T>(src, order, g, x, V, st, fj));
         if (rc) return rc;
     }
+    if (algo == WINO_ALGO_EPILOGUE_F4) {
+        StageScope t(WINO_STAGE_GEMM, st);
+        return launch_f4_gemm_rows(dst, order, flags, bias, g, plan, U, V, y, Mo, (int*)base, st);   // (the product region holds the partial outputs)
+    }
     {
         StageScope t(WINO_STAGE_GEMM, st);
         rc = launch_gemm(36, dtype, porder, g.Cp, g.Kp, g.Pp, U, V, Mo, st);
@@ -1038,7 +1108,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
               int W, int pad, const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
     if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
-    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_DIRECT) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
+    if (algo < WINO_ALGO_AUTO || algo > WINO_ALGO_EPILOGUE_F4) return fail(WINO_ERR_INVALID, "unknown algo %d", algo);
     if (!x || (!w && !Upre) || !y) return fail(WINO_ERR_INVALID, "null tensor pointer");
     if (misaligned(x, elem_bytes(dtype)) || misaligned(w, elem_bytes(dtype)) || misaligned(y, elem_bytes(dtype)) ||
         misaligned(bias, elem_bytes(dtype)))
@@ -1051,8 +1121,8 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     if ((flags & WINO_FLAG_POOL2) && (g.Ho < 2 || g.Wo < 2))
         return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", g.Ho, g.Wo);
     if (algo == WINO_ALGO_AUTO) {
-        algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
-        if (algo == WINO_ALGO_STAGED_F4) Upre = nullptr;      // transformed filters handed in alongside w are F(2x2) ones
+        algo = resolve_auto(src, dst, dtype, flags, g, x, y, w != nullptr);
+        if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4) Upre = nullptr;      // transformed filters handed in alongside w are F(2x2) ones
     }
     if (algo == WINO_ALGO_DIRECT) {
         if (!w) return fail(WINO_ERR_INVALID, "the direct path needs the filter bank, not its Winograd transform");
@@ -1069,7 +1139,8 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
         return launch_direct16(src, dst, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
     }
-    if (algo == WINO_ALGO_STAGED_F4) return conv_f4_impl(ss, src, dst, dtype, flags, bias, N, C, K, H, W, pad, x, w, Upre, y, stream);
+    if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4)
+        return conv_f4_impl(ss, src, dst, dtype, algo, flags, bias, N, C, K, H, W, pad, x, w, Upre, y, stream);
 
     hipStream_t st = (hipStream_t)stream;
     const Scratch sc = scratch_layout(g, dtype, algo);
@@ -1132,15 +1203,10 @@ constexpr size_t kNoAllocBytes = WINO_NOALLOC_SCRATCH_BYTES;
 void* g_noalloc_ptr[kMaxDevices] = {};
 std::mutex g_noalloc_mu;
 
-__global__ void fill_zero_kernel(unsigned* p, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
-}
-
-// The current device's copy of `scratch`; on the first call for a device its arrival counters are cleared by a
-// kernel on `st` (a fill kernel, not a memset: the caller may be recording a graph).  Later launches leave the
-// counters at zero themselves.
-int noalloc_scratch(hipStream_t st, void** out) {
+// The current device's copy of `scratch`.  Nothing is cleared here: the array is a zero-initialised object of the
+// device image, the only part of it that must be zero when a kernel starts is the arrival counters at its head,
+// and every kernel that counts arrivals returns its counters to zero before it ends.
+int noalloc_scratch(void** out) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return fail(WINO_ERR_UNSUPPORTED, "device index %d out of range", dev);
@@ -1149,9 +1215,6 @@ int noalloc_scratch(hipStream_t st, void** out) {
         void* ptr = nullptr;
         HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         if (!ptr || misaligned(ptr, 256)) return fail(WINO_ERR_HIP, "built-in scratch buffer not found on device %d", dev);
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(kCounterBytes / 4 / 256)), dim3(256), 0, st, (unsigned*)ptr,
-                           (int)(kCounterBytes / 4));
-        LAUNCH_CHECK("fill_zero");
         g_noalloc_ptr[dev] = ptr;
     }
     *out = g_noalloc_ptr[dev];
@@ -1179,10 +1242,10 @@ int conv_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     Geometry g;
     int passes = 1;
     if (valid_layout(src) && valid_layout(dst) && valid_dtype(dtype) && x && y && (w || Upre) &&
-        make_geometry(dtype, N, C, K, H, W, pad, &g) && algo >= WINO_ALGO_AUTO && algo <= WINO_ALGO_DIRECT) {
+        make_geometry(dtype, N, C, K, H, W, pad, &g) && algo >= WINO_ALGO_AUTO && algo <= WINO_ALGO_EPILOGUE_F4) {
         if (algo == WINO_ALGO_AUTO) {
-            algo = resolve_auto(src, dst, dtype, flags, g, x, w != nullptr);
-            if (algo == WINO_ALGO_STAGED_F4) Upre = nullptr;  // transformed filters handed in alongside w are F(2x2) ones
+            algo = resolve_auto(src, dst, dtype, flags, g, x, y, w != nullptr);
+            if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4) Upre = nullptr;  // transformed filters handed in alongside w are F(2x2) ones
         }
         passes = batch_passes(src, dst, dtype, algo, g);
     }
@@ -1243,7 +1306,7 @@ int wino_conv_noalloc(int src, int dst, int dtype, int algo, unsigned flags, int
         ~NoTiming() { t_no_timing = false; }
     } guard;
     ScratchSource ss;
-    const int rc = noalloc_scratch((hipStream_t)stream, &ss.fixed);
+    const int rc = noalloc_scratch(&ss.fixed);
     if (rc) return rc;
     ss.fixed_bytes = kNoAllocBytes;
     return conv_impl(ss, src, dst, dtype, algo, flags, N, C, K, H, W, pad, x, w, nullptr, bias, y, stream);
@@ -1255,7 +1318,7 @@ int wino_pick_algo(int layout, int dtype, int N, int C, int K, int H, int W, int
     Geometry g;
     if (!make_geometry(dtype, N, C, K, H, W, pad, &g))
         return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d H=%d W=%d pad=%d", N, C, K, H, W, pad);
-    return resolve_auto(layout, layout, dtype, 0, g, nullptr, true);
+    return resolve_auto(layout, layout, dtype, 0, g, nullptr, nullptr, true);
 }
 
 int wino_geometry(int dtype, int N, int C, int K, int H, int W, int pad, int* th, int* tw, long* P, int* Cp, int* Kp,
@@ -1281,7 +1344,8 @@ size_t wino_workspace_bytes(int dtype, int N, int C, int K, int H, int W, int pa
     }
     Geometry g4;
     size_t need = scratch_layout(g, dtype).total;
-    if (make_geometry(dtype, N, C, K, H, W, pad, &g4, 4)) need = std::max(need, scratch_layout(g4, dtype).total);
+    if (make_geometry(dtype, N, C, K, H, W, pad, &g4, 4))
+        need = std::max(need, std::max(scratch_layout(g4, dtype).total, scratch_layout(g4, dtype, WINO_ALGO_EPILOGUE_F4).total));
     return need;
 }
 
@@ -1497,6 +1561,29 @@ int wino_f4_output_transform(int layout, int dtype, int tile_order, int product_
                                               y, (hipStream_t)stream));
 }
 
+int wino_f4_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int N, int C, int K, int Ho, int Wo,
+                        const void* U, const void* V, void* y, void* stream) {
+    if (!valid_layout(layout)) return fail(WINO_ERR_INVALID, "unknown layout %d", layout);
+    if (!valid_dtype(dtype)) return fail(WINO_ERR_INVALID, "unknown dtype %d", dtype);
+    if (!valid_order(tile_order)) return fail(WINO_ERR_INVALID, "unknown tile order %d", tile_order);
+    if (!U || !V || !y) return fail(WINO_ERR_INVALID, "null pointer");
+    if (misaligned(U, 16) || misaligned(V, 16)) return fail(WINO_ERR_INVALID, "GEMM operands must be 16-byte aligned");
+    if (flags & ~(unsigned)(WINO_FLAG_RELU | WINO_FLAG_POOL2)) return fail(WINO_ERR_INVALID, "unknown flags 0x%x", flags);
+    Geometry g;
+    // geometry from the output size: pad 1 keeps H == Ho
+    if (!make_geometry(dtype, N, C, K, Ho, Wo, 1, &g, 4))
+        return fail(WINO_ERR_INVALID, "bad shape N=%d C=%d K=%d Ho=%d Wo=%d", N, C, K, Ho, Wo);
+    if ((flags & WINO_FLAG_POOL2) && (Ho < 2 || Wo < 2)) return fail(WINO_ERR_INVALID, "2x2 pooling of a %dx%d output", Ho, Wo);
+    F4RowsPlan plan;
+    if (!f4_rows_plan(dtype, g, &plan))
+        return fail(WINO_ERR_UNSUPPORTED, "the F(4x4) GEMM with the output transform in its epilogue is built for fp32 operands");
+    void* base = nullptr;                      // partial outputs and arrival counters: the arena (shared like a whole-layer call's)
+    const int rc = arena_get(kCounterBytes + plan.part_bytes, &base);
+    if (rc) return rc;
+    return launch_f4_gemm_rows(layout, tile_order, flags, nullptr, g, plan, U, V, y, (float*)((char*)base + kCounterBytes),
+                               (int*)base, (hipStream_t)stream);
+}
+
 int wino_stage_timing(int enable) {
     std::lock_guard<std::mutex> lk(g_spans_mu);
     g_timing = enable != 0;
@@ -1572,13 +1659,14 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
         void* out = l + 1 == n ? y : s->act[l & 1];
         const void* bias = L.has_bias ? L.bias : nullptr;
         int rc;
-        Geometry g;
+        Geometry g, g4;
         make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g);
+        make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4);
         if (L.U4) {
-            rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, WINO_ALGO_STAGED_F4, L.flags, s->N, L.C, L.K, L.H,
-                           L.W, 1, in, nullptr, L.U4, bias, out, stream);
+            rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, auto_f4_algo(s->dtype, g4), L.flags, s->N, L.C, L.K,
+                           L.H, L.W, 1, in, nullptr, L.U4, bias, out, stream);
         } else if (L.W9 && !misaligned(in, 4) && (!misaligned(out, 4) || (L.flags & WINO_FLAG_POOL2)) &&
-                   auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in)) {
+                   auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in, out)) {
             // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
             rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
@@ -1655,7 +1743,7 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
             e = hipMalloc(&L.U4, (size_t)36 * g4.Cp * g4.Kp * es);
         }
         if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && direct16_layer &&
-            auto_direct16(L.layout_in, L.layout_out, dtype, L.flags, g, nullptr))
+            auto_direct16(L.layout_in, L.layout_out, dtype, L.flags, g, nullptr, nullptr))
             e = hipMalloc(&L.W9, direct16_bank_bytes(g));
         if (e != hipSuccess) return bail(e);
     }
@@ -1723,7 +1811,8 @@ int wino_stack_forward_graph(wino_stack_t* s, const void* x, void* y, void* stre
         if (!make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g)) return fail(WINO_ERR_INVALID, "bad layer shape");
         need = std::max(need, scratch_layout(g, s->dtype).total);
         Geometry g4;
-        if (L.U4 && make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4)) need = std::max(need, scratch_layout(g4, s->dtype).total);
+        if (L.U4 && make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4))
+            need = std::max(need, scratch_layout(g4, s->dtype, auto_f4_algo(s->dtype, g4)).total);
     }
     void* base = nullptr;
     int rc = arena_get(need, &base);
@@ -1773,7 +1862,7 @@ int wino_warmup(void) {
     hipLaunchKernelGGL(warmup_kernel, dim3(1), dim3(1), 0, 0);
     LAUNCH_CHECK("warmup");
     void* unused = nullptr;                    // also the set-up of wino_conv_noalloc's buffer on this device
-    return noalloc_scratch(nullptr, &unused);
+    return noalloc_scratch(&unused);
 }
 
 int wino_sync(void* stream) {
@@ -1783,6 +1872,6 @@ int wino_sync(void* stream) {
 
 const char* wino_last_error(void) { return g_err; }
 
-const char* wino_version(void) { return "wino_amd 0.1 (gfx950, F(2x2,3x3))"; }
+const char* wino_version(void) { return "wino_amd 0.3 (gfx950; F(2x2,3x3), F(4x4,3x3), direct)"; }
 
 }  // extern "C"

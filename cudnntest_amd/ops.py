@@ -23,7 +23,7 @@ from . import _lib
 
 NCHW, NHWC, CHWN = 0, 1, 2
 F32, F16, BF16 = 0, 1, 2
-ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED, ALGO_STAGED_F4, ALGO_DIRECT = 0, 1, 2, 3, 4, 5
+ALGO_AUTO, ALGO_STAGED, ALGO_EPILOGUE, ALGO_FUSED, ALGO_STAGED_F4, ALGO_DIRECT, ALGO_EPILOGUE_F4 = 0, 1, 2, 3, 4, 5, 6
 TILES_BATCH_MAJOR, TILES_BATCH_MINOR = 0, 1
 PRODUCT_KP, PRODUCT_PK = 0, 1
 FLAG_RELU = 1
@@ -83,7 +83,7 @@ def geometry(dtype, N, C, K, H, W, pad):
 
 
 ALGO_NAMES = {ALGO_AUTO: "auto", ALGO_STAGED: "staged", ALGO_EPILOGUE: "epilogue", ALGO_FUSED: "fused",
-              ALGO_STAGED_F4: "staged_f4", ALGO_DIRECT: "direct"}
+              ALGO_STAGED_F4: "staged_f4", ALGO_DIRECT: "direct", ALGO_EPILOGUE_F4: "epilogue_f4"}
 
 
 def pick_algo(layout, dtype, N, C, K, H, W, pad=1):
@@ -369,6 +369,15 @@ def f4_output_transform(Mo, N, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MA
     _lib.check(_lib.load().wino_f4_output_transform(int(layout), _DTYPES[dtype], tile_order, product_order,
                                                     (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0), N, K, Ho, Wo,
                                                     _ptr(Mo), _ptr(y), _stream()), "wino_f4_output_transform")
+    return y
+
+
+def f4_gemm_output(U, V, N, C, K, Ho, Wo, layout=NCHW, tile_order=TILES_BATCH_MAJOR, relu=False, pool=False):
+    """y straight from the F(4x4) operands: the 36-way GEMM with the output transform in its epilogue (fp32)."""
+    y = torch.empty(act_shape(layout, N, K, Ho // 2 if pool else Ho, Wo // 2 if pool else Wo), dtype=U.dtype, device=U.device)
+    _lib.check(_lib.load().wino_f4_gemm_output(int(layout), _dt(U), tile_order,
+                                               (FLAG_RELU if relu else 0) | (FLAG_POOL2 if pool else 0), N, C, K, Ho, Wo,
+                                               _ptr(U), _ptr(V), _ptr(y), _stream()), "wino_f4_gemm_output")
     return y
 
 

@@ -1,5 +1,9 @@
 /*
- * wino_amd.h -- C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) convolution library.
+ * wino_amd.h -- C ABI of the MI355X (gfx950) Winograd 3x3 convolution library: F(2x2,3x3) and F(4x4,3x3)
+ * pipelines in fp32, F(2x2,3x3) with f16 / bf16 storage, and direct MFMA convolutions where those are faster.
+ * What a caller of the whole-layer entry points gets under WINO_ALGO_AUTO: fp32 layers with C, K >= 128 run in
+ * F(4x4,3x3), the reference's own tile size (relative L2 error against a direct convolution 3e-6 to 5e-6), other
+ * fp32 layers in F(2x2,3x3) (about 1e-6), 2-byte layers in F(2x2,3x3) or directly (about 2e-3 bf16, 3e-4 f16).
  *
  * Every entry point takes plain device pointers and sizes; `stream` is a
  * hipStream_t passed as void* (NULL = the null stream).  Calls are asynchronous
@@ -65,7 +69,7 @@ typedef enum {
                                for fp32 layers with C, K >= 128 and at least 512 tiles when it is
                                given the filter bank itself; transformed filters handed to this algorithm by
                                name must come from wino_f4_filter_transform. */
-    WINO_ALGO_DIRECT = 5     /* no Winograd at all, the convolution itself on the matrix cores.  Two kernels:
+    WINO_ALGO_DIRECT = 5,    /* no Winograd at all, the convolution itself on the matrix cores.  Two kernels:
                                layers with C <= 4 (the network's first layer, which the reference runs through
                                the same wrappers: comparison/layoutCompare.cu:38-46): the 9*C <= 36 products of an
                                output as one short MFMA reduction, any layout, fp32 or 2-byte;
@@ -83,6 +87,12 @@ typedef enum {
                                shape just named), not for C <= 4; needs the filter bank itself (not
                                wino_conv_prepared).
                                What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW and NHWC layers. */
+    WINO_ALGO_EPILOGUE_F4 = 6 /* F(4x4,3x3) with the output transform A^T (.) A in the epilogue of the 36-way GEMM: no
+                               product tensor in HBM.  The arrangement of the reference's fused F(4x4) kernels
+                               (fusedTest/winotrans.cuh:1530-1574: 36 running products, A^T acc A in registers, 16
+                               stores) for the matrix cores, one Winograd row resident at a time.  fp32, any layout
+                               pair, bias / ReLU / pooling; transformed filters as for WINO_ALGO_STAGED_F4; 2-byte
+                               tensors are refused (WINO_ERR_UNSUPPORTED). */
 } wino_algo_t;
 
 /* order of the tile index p inside the transformed operands */
@@ -155,8 +165,8 @@ int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags,
  * does not see it).  A problem whose pipeline needs more scratch than the buffer holds is refused with
  * WINO_ERR_WORKSPACE and a message giving both sizes: ask for WINO_ALGO_FUSED (keeps only the transformed
  * filters, 16*Cp*Kp elements) or WINO_ALGO_DIRECT, or use a smaller batch.  The first call on a device looks the
- * buffer up and clears its counters with a small kernel on `stream`; wino_warmup() does the same ahead of time
- * (do one of the two before recording a graph).  Every call on a GPU shares that GPU's buffer: calls that overlap
+ * buffer's address up (wino_warmup() does the same ahead of time); nothing is cleared: the buffer is a
+ * zero-initialised object of the device image, and the kernels that count arrivals in it leave their counters at zero.  Every call on a GPU shares that GPU's buffer: calls that overlap
  * on one GPU (two streams, two threads) race, exactly as whole-layer calls sharing the arena do.
  */
 #define WINO_NOALLOC_SCRATCH_BYTES (64u << 20)
@@ -223,6 +233,11 @@ int wino_f4_batched_gemm(int dtype, int product_order, int C, int K, long P, con
                          float *Mo, void *stream);
 int wino_f4_output_transform(int layout, int dtype, int tile_order, int product_order, unsigned flags, int N,
                              int K, int Ho, int Wo, const float *Mo, void *y, void *stream);
+/* The 36-way GEMM with the output transform in its epilogue: y directly from U and V (fp32; pad 1 geometry, as
+ * wino_gemm_output).  The GEMM + inverse transform of the reference's fused kernel, fusedTest/winotrans.cuh:1530-1574.
+ * Takes its partial-sum scratch from the device's arena, like a whole-layer call. */
+int wino_f4_gemm_output(int layout, int dtype, int tile_order, unsigned flags, int N, int C, int K, int Ho, int Wo,
+                        const void *U, const void *V, void *y, void *stream);
 
 /* ---- plain layout permutation (bench harness; the reference has no such kernel) */
 int wino_layout_transform(int src, int dst, int dtype, int N, int C, int H, int W, const void *in,

@@ -16,9 +16,11 @@
 // reference would let pass silently, is reported on stderr.
 //
 // Difference: inputTran_gpu / filterTran_gpu / gemmOutput_gpu are accepted and
-// ignored.  The library works in F(2x2,3x3), whose intermediates are larger
-// than the F(4x4,3x3) buffers a reference caller sizes (36*MSize*KSize ...), so
-// it draws scratch from its own per-device arena (or from wino_set_workspace).
+// ignored.  The library picks its pipeline per layer -- F(4x4,3x3) like the
+// reference for fp32 layers with C, K >= 128, F(2x2,3x3) or a direct kernel
+// otherwise -- and pads its operands to its own tile sizes, so its scratch is
+// not what a reference caller sizes (36*MSize*KSize ...): it draws scratch from
+// its own per-device arena (or from wino_set_workspace).
 #pragma once
 #include <cstdio>
 

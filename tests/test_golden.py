@@ -49,12 +49,13 @@ def test_oracle_winograd_stages_reproduce_the_fixtures(oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("algo", [ops.ALGO_AUTO, ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_STAGED_F4])
+@pytest.mark.parametrize("algo", [ops.ALGO_AUTO, ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_STAGED_F4,
+                                  ops.ALGO_EPILOGUE_F4])
 @pytest.mark.parametrize("problem", PROBLEMS)
 def test_hip_path_matches_the_fixtures(oracle, problem, algo):
     from gpu_util import TOL, dev, host
     x, w = FIX[problem + "_x"], FIX[problem + "_w"]
-    exact = problem.endswith("_int") and algo != ops.ALGO_STAGED_F4     # F(4x4)'s 1/6, 1/24 are not dyadic
+    exact = problem.endswith("_int") and algo not in (ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4)     # F(4x4)'s 1/6, 1/24 are not dyadic
     for pad in (0, 1):
         want = FIX[f"{problem}_y_pad{pad}"]
         for src, dst in itertools.product(LAYOUTS, LAYOUTS):

@@ -69,7 +69,7 @@ def test_n64_c512_every_pipeline(oracle, H, layout):
     ks, want = oracle_planes(oracle, x, w)
     xl, wl = to_layout(x, layout), to_layout(w, layout)
     base = None
-    for algo in (ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_STAGED_F4, ops.ALGO_AUTO):
+    for algo in (ops.ALGO_STAGED, ops.ALGO_EPILOGUE, ops.ALGO_FUSED, ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4, ops.ALGO_AUTO):
         y = from_layout(ops.conv(xl, wl, 1, layout, algo=algo), layout)
         assert tuple(y.shape) == (N, K, H, H)
         err = oracle.rel_l2(host(y[-1:][:, ks]), want)

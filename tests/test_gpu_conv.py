@@ -234,3 +234,19 @@ def test_element_aligned_views_of_images_larger_than_a_workgroup(dtype, algo):
         got = ops.conv(_view_at(x, shift), _view_at(w, shift), 1, ops.NCHW, algo=algo, relu=True, out=out)
         assert got.data_ptr() % 8 != 0
         assert torch.equal(got, want), (shift, (got.float() - want.float()).abs().max().item())
+
+
+@pytest.mark.parametrize("layouts", [(ops.NHWC, ops.NHWC), (ops.NCHW, ops.NHWC), (ops.NHWC, ops.NCHW)])
+def test_auto_with_an_nhwc_side_and_an_output_that_is_only_element_aligned(layouts):
+    """A 2-byte layer large enough for the direct path, x aligned, y at an odd element offset: with an NHWC side only
+    the 8-wave direct kernel could run, and it stores 4-byte pairs -- the automatic choice has to see y's alignment
+    and take the Winograd pipelines instead of refusing.  Small integers: every pipeline gives the same bits."""
+    src, dst = layouts
+    N, C, K, H = 32, 64, 64, 56
+    x, w = synth.conv_inputs(N, C, K, H, H, seed=31, layout=src, integer=True)
+    xd, wd = dev(x, ops.BF16), dev(w, ops.BF16)
+    want = ops.conv(xd, wd, 1, src, dst, algo=ops.ALGO_AUTO, relu=True)
+    out = _view_at(torch.zeros_like(want), 1)
+    assert out.data_ptr() % 4 != 0
+    got = ops.conv(xd, wd, 1, src, dst, algo=ops.ALGO_AUTO, relu=True, out=out)
+    assert torch.equal(got, want)

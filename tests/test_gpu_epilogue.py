@@ -72,8 +72,9 @@ def test_floats_within_tolerance(oracle, algo, layout, dtype):
     assert oracle.rel_l2(got, want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("f4_algo", [ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4])
 @pytest.mark.parametrize("shape", [(2, 5, 7, 8, 8), (1, 16, 70, 9, 7), (3, 32, 20, 6, 10), (2, 24, 40, 13, 18)])
-def test_f4_bias_relu_pool_every_layout_pair(oracle, shape):
+def test_f4_bias_relu_pool_every_layout_pair(oracle, shape, f4_algo):
     """The F(4x4,3x3) pipeline's output stage: the same three steps, 2x2 pooled values per 4x4 tile.  Its transforms
     hold sixths and twenty-fourths, so integers do not come out bit for bit: the layer tolerance (relative L2 1e-4 in
     fp32) applies, and the pooled and unpooled shapes are checked."""
@@ -85,18 +86,19 @@ def test_f4_bias_relu_pool_every_layout_pair(oracle, shape):
         for relu, pool, with_bias in [(True, True, True), (False, True, False), (True, False, True), (False, False, True)]:
             b = bias if with_bias else None
             want = expected(oracle, xs, ws, b, 1, src, dst, relu, pool)
-            got = host(ops.conv(dev(xs), dev(ws), 1, src, dst, ops.ALGO_STAGED_F4, relu=relu, pool=pool,
+            got = host(ops.conv(dev(xs), dev(ws), 1, src, dst, f4_algo, relu=relu, pool=pool,
                                 bias=dev(b) if with_bias else None))
             assert got.shape == want.shape, (src, dst, relu, pool)
             assert oracle.rel_l2(got, want) <= TOL[ops.F32], (src, dst, relu, pool, with_bias)
 
 
-def test_f4_pad0_odd_output_drops_the_cut_windows(oracle):
+@pytest.mark.parametrize("f4_algo", [ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4])
+def test_f4_pad0_odd_output_drops_the_cut_windows(oracle, f4_algo):
     N, C, K, H, W = 2, 6, 5, 9, 8          # pad 0: 7 x 6 outputs -> 3 x 3 pooled; the last tile row holds one pooled row
     x, w = synth.conv_inputs(N, C, K, H, W, seed=3)
     bias = synth.normal(K, seed=9, std=0.5).astype(np.float32)
     want = expected(oracle, x, w, bias, 0, ops.NCHW, ops.NCHW, True, True)
-    got = host(ops.conv(dev(x), dev(w), 0, algo=ops.ALGO_STAGED_F4, relu=True, pool=True, bias=dev(bias)))
+    got = host(ops.conv(dev(x), dev(w), 0, algo=f4_algo, relu=True, pool=True, bias=dev(bias)))
     assert got.shape == (N, K, 3, 3)
     assert oracle.rel_l2(got, want) <= TOL[ops.F32]
     # the stage function takes the pooling flag (no bias)

@@ -116,25 +116,73 @@ def test_f4_output_transform(oracle, layout, order, porder, N, K, Ho, Wo):
         assert np.array_equal(y, np.maximum(want, 0) if relu else want)
 
 
+F4_ALGOS = [ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4]
+
+
+@pytest.mark.parametrize("layout,order", [(ops.NCHW, ops.TILES_BATCH_MAJOR), (ops.NHWC, ops.TILES_BATCH_MAJOR),
+                                          (ops.CHWN, ops.TILES_BATCH_MINOR), (ops.NCHW, ops.TILES_BATCH_MINOR)])
+@pytest.mark.parametrize("C,K,N,Ho,Wo", [(16, 64, 1, 8, 8),        # one patch: a single workgroup or a few sharing it
+                                         (40, 130, 3, 40, 40),      # 15 patches, filters and tiles ragged
+                                         (80, 200, 2, 56, 60),      # 28 patches on 8 XCDs: uneven shares
+                                         (256, 64, 8, 28, 28),      # one filter tile, 7 tile patches, 16 stages to a row
+                                         (48, 256, 16, 30, 30)])    # 64 patches: most workgroups hold parts of two
+def test_f4_gemm_with_the_output_transform_in_its_epilogue(oracle, layout, order, C, K, N, Ho, Wo):
+    """y straight from U and V (gemm_rows_f4_kernel): the persistent workgroups cut the stage sequence of their XCD's
+    patches into equal runs, so most patches are summed from the partial outputs of two or more workgroups.  Small
+    integers: every product and partial sum is exact, so the result equals the oracle's GEMM followed by its output
+    transform bit for bit -- twice in a row (the arrival counters return to zero), with ReLU the second time."""
+    g = ops.f4_geometry(ops.F32, N, C, K, Ho, Wo, 1)
+    Cp, Kp, Pp, P, th, tw = g["Cp"], g["Kp"], g["Pp"], g["P"], g["th"], g["tw"]
+    U = np.zeros((36, Cp, Kp), np.float32)
+    V = np.full((36, Cp, Pp), 3.0e38, np.float32)        # tile columns past P hold anything: they may not leak
+    U[:, :C, :K] = synth.small_ints(36 * C * K, 13 + C, -2, 2).reshape(36, C, K)
+    Vm = synth.small_ints(36 * C * P, 14 + K, -3, 3).reshape(36, C, P)
+    V[:, :, :P] = 0
+    V[:, :C, :P] = Vm[:, :, batch_minor_perm(N, th, tw)] if order == ops.TILES_BATCH_MINOR else Vm
+    M = oracle.wino_gemm(np.ascontiguousarray(U[:, :C, :K]), np.ascontiguousarray(Vm), m=4)
+    want = oracle.wino_output_transform(M, N, Ho, Wo, layout, m=4)
+    Ud, Vd = pack_operand(U), pack_operand(V)
+    for relu in (False, True):
+        y = host(ops.f4_gemm_output(Ud, Vd, N, C, K, Ho, Wo, layout, order, relu))
+        assert np.array_equal(y, np.maximum(want, 0) if relu else want), relu
+
+
+@pytest.mark.parametrize("algo", F4_ALGOS)
 @pytest.mark.parametrize("shape", [(2, 3, 4, 5, 5), (1, 8, 8, 6, 6), (3, 5, 7, 9, 9), (2, 16, 130, 7, 10), (1, 1, 1, 3, 3)])
-def test_f4_layers_all_layout_pairs(oracle, shape):
+def test_f4_layers_all_layout_pairs(oracle, shape, algo):
     N, C, K, H, W = shape
     x, w = synth.conv_inputs(N, C, K, H, W, seed=sum(shape))
     for src, dst in itertools.product(LAYOUTS, LAYOUTS):
         xs, ws = synth.act_to_layout(x, src), synth.flt_to_layout(w, src)
         want = oracle.direct_conv(xs, ws, 1, src, dst)
-        got = host(ops.conv(dev(xs), dev(ws), 1, src, dst, ops.ALGO_STAGED_F4))
+        got = host(ops.conv(dev(xs), dev(ws), 1, src, dst, algo))
         assert oracle.rel_l2(got, want) <= TOL[ops.F32], (src, dst)
 
 
+@pytest.mark.parametrize("algo", F4_ALGOS)
 @pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("shape", [(1, 64, 64, 56, 56), (64, 128, 128, 22, 22), (4, 128, 96, 14, 14), (2, 3, 64, 32, 32)])
-def test_f4_floats_within_tolerance(oracle, layout, shape):
+def test_f4_floats_within_tolerance(oracle, layout, shape, algo):
     # second shape is the one the reference's notebooks use: N=64, C=K=128, H=22
     N, C, K, H, W = shape
     x, w = synth.conv_inputs(N, C, K, H, W, seed=2000 + sum(shape), layout=layout)
     want = oracle.direct_conv(x, w, 1, layout)
-    got = host(ops.conv(dev(x), dev(w), 1, layout, algo=ops.ALGO_STAGED_F4))
+    got = host(ops.conv(dev(x), dev(w), 1, layout, algo=algo))
     err = oracle.rel_l2(got, want)
-    print(f"F(4x4) layout {layout} shape {shape}: rel L2 {err:.2e}, sum|err| {np.abs(got - want).sum():.2f}")
+    print(f"F(4x4) algo {algo} layout {layout} shape {shape}: rel L2 {err:.2e}, sum|err| {np.abs(got - want).sum():.2f}")
     assert err <= TOL[ops.F32], err
+
+
+def test_the_two_f4_pipelines_agree_on_the_headline_layer_bit_for_bit_from_call_to_call():
+    """N=32, C=K=256, 56x56: 392 patches on 256 workgroups -- every workgroup holds parts of two or three patches.
+    Against the staged F(4x4) pipeline (same products, another order of the sums: 1e-5), and twice the same bits."""
+    N, C, K, H = 32, 256, 256, 56
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.rand((N, C, H, H), device="cuda", generator=g) * 2 - 1
+    w = torch.randn((K, C, 3, 3), device="cuda", generator=g) * (2.0 / (9 * C)) ** 0.5
+    for dst in LAYOUTS:
+        a = ops.conv(x, w, 1, ops.NCHW, dst, algo=ops.ALGO_STAGED_F4)
+        b = ops.conv(x, w, 1, ops.NCHW, dst, algo=ops.ALGO_EPILOGUE_F4)
+        c = ops.conv(x, w, 1, ops.NCHW, dst, algo=ops.ALGO_EPILOGUE_F4)
+        assert torch.equal(b, c)
+        assert ((a - b).double().norm() / a.double().norm()).item() <= 1e-5

@@ -51,7 +51,7 @@ def test_fp32_floats_f4_and_auto(oracle, shape):
         xs, ws = synth.act_to_layout(x, src), synth.flt_to_layout(w, src)
         want = synth.act_from_layout(oracle.direct_conv(xs, ws, pad, src), src) + bias[None, :, None, None]
         want = synth.act_to_layout(np.maximum(want, 0).astype(np.float32), src)
-        for algo in (ops.ALGO_STAGED_F4, ops.ALGO_AUTO):
+        for algo in (ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4, ops.ALGO_AUTO):
             got = host(ops.conv(dev(xs), dev(ws), pad, src, algo=algo, relu=True, bias=dev(bias)))
             assert oracle.rel_l2(got, want) <= 2e-5, (src, algo)
 
