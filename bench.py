@@ -25,6 +25,8 @@ Prints ONE JSON line:
                measured with rocprofv3 --pmc (traffic_source names the summary under profiles/), null where
                no such run is committed
   cpu_baseline the oracle's fp32 OpenMP direct convolution on this host's cores (reported, not a target)
+  configs_summary   the LAST key of the line: every entry of `configs` as [ms, effective TFLOP/s, pipeline, fraction of
+               what the two roofs allow], so that a record which keeps only the line's tail still holds them all
   stages       per-stage ms and achieved GB/s (algorithmic bytes) or TFLOP/s
   ms_per_step_filters_prepared   the same K steps with the filter bank transformed beforehand (single-layer runs)
   layout_transforms   the stand-alone permutations of the layer's input between its layout and the other two
@@ -104,8 +106,9 @@ OTHER_CONFIGS = [
     ("cfg5_vgg16_all13_N32_f16", "vgg16_all13", "f16", "NCHW"),
     ("cfg5_vgg16_all13_N32_bf16", "vgg16_all13", "bf16", "NCHW"),
     ("cfg5_vgg16_all13_N32_bf16_NHWC", "vgg16_all13", "bf16", "NHWC"),
+    ("cfg5_vgg16_all13_N32_bf16_CHWN", "vgg16_all13", "bf16", "CHWN"),
 ]
-KERNEL_OF = {"staged": "gemm_128x128_kernel / gemm_128x128_walk_kernel / gemm_128x128_walk_spread_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
+KERNEL_OF = {"epilogue_f4": "gemm_rows_f4_kernel", "staged": "gemm_128x128_kernel / gemm_128x128_walk_kernel / gemm_128x128_walk_spread_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
              "staged_f4": "gemm_128x128_walk_spread_kernel / gemm_128x128_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel"}
 
 
@@ -117,7 +120,7 @@ def main():
     ap.add_argument("--workload", default="vgg16_conv3_N32_C256_K256_H56", choices=sorted(WORKLOADS))
     ap.add_argument("--layout", default="NCHW", choices=["NCHW", "NHWC", "CHWN"])
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"])
-    ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4", "direct"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "staged", "epilogue", "fused", "staged_f4", "direct", "epilogue_f4"])
     ap.add_argument("--shape", default=None, metavar="N,C,K,H",
                     help="a single layer of this shape instead of a named workload (kernel experiments)")
     ap.add_argument("--batch", type=int, default=32, help="N of the vgg16_all13 / vgg16_stack workloads")
@@ -155,7 +158,8 @@ def main():
     TDT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
     DT = {"f32": ops.F32, "f16": ops.F16, "bf16": ops.BF16}
     ALGO = {"auto": ops.ALGO_AUTO, "staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE,
-            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4, "direct": ops.ALGO_DIRECT}
+            "fused": ops.ALGO_FUSED, "staged_f4": ops.ALGO_STAGED_F4, "direct": ops.ALGO_DIRECT,
+            "epilogue_f4": ops.ALGO_EPILOGUE_F4}
 
     if args.shape:
         WORKLOADS["custom"] = [tuple(int(v) for v in args.shape.split(","))]
@@ -200,7 +204,7 @@ def main():
         """the dominant kernel of one layer against both roofs"""
         dt, es, peak = DT[dtype], (4 if dtype == "f32" else 2), MFMA_PEAK_TFLOPS[dtype]
         name = ops.ALGO_NAMES[a]
-        f4 = a == ops.ALGO_STAGED_F4
+        f4 = a in (ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4)
         g = ops.f4_geometry(dt, N, C, K, H, H, 1) if f4 else ops.geometry(dt, N, C, K, H, H, 1)
         P, nxi = g["P"], (36 if f4 else 16)
         xb, yb = N * C * H * H * es, N * K * H * H * es
@@ -208,6 +212,7 @@ def main():
         kb = {"staged": nxi * P * C * es + nxi * K * C * es + nxi * P * K * 4,
               "staged_f4": nxi * P * C * es + nxi * K * C * es + nxi * P * K * 4,
               "epilogue": 16 * P * C * es + 16 * K * C * es + yb,
+              "epilogue_f4": 36 * P * C * es + 36 * K * C * es + yb,
               "fused": xb + 16 * K * C * es + yb,
               "direct": xb + 9 * K * C * es + yb}[name]
         ai = flops / kb
@@ -376,7 +381,7 @@ def main():
     resolved = []
     for (N, C, K, H) in layers:
         a = ops.pick_algo(layout, dt, N, C, K, H, H) if algo == ops.ALGO_AUTO else algo
-        f4 = a == ops.ALGO_STAGED_F4
+        f4 = a in (ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4)
         g = ops.f4_geometry(dt, N, C, K, H, H, 1) if f4 else ops.geometry(dt, N, C, K, H, H, 1)
         P, nxi = g["P"], (36 if f4 else 16)
         resolved.append(ops.ALGO_NAMES[a])
@@ -435,7 +440,7 @@ def main():
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": args.workload, "layers": len(layers), "N": N0, "C": C0, "K": K0, "H": H0, "W": H0,
                    "pad": 1, "layout": args.layout, "algo": args.algo, "resolved_algo": resolved,
-                   "winograd": "F(4x4,3x3)" if algo_label == "staged_f4" else "F(2x2,3x3)",
+                   "winograd": "F(4x4,3x3)" if algo_label in ("staged_f4", "epilogue_f4") else "F(2x2,3x3)",
                    "filter_transform_in_step": stack is None, "relu": multi,
                    "bias_and_pooling_in_step": stack is not None, "hip_graph": args.graph},
         "roofline": roofline,
@@ -443,11 +448,11 @@ def main():
     }
 
     # ---- the same K steps with the filter bank transformed beforehand (filter transform excluded) ----
-    if not multi and stack is None and resolved[0] in ("staged", "epilogue", "fused", "staged_f4"):
+    if not multi and stack is None and resolved[0] in ("staged", "epilogue", "fused", "staged_f4", "epilogue_f4"):
         x0, w0, y0 = tensors[0]
-        U0 = ops.f4_filter_transform(w0, layout) if resolved[0] == "staged_f4" else ops.filter_transform(w0, layout)
+        U0 = ops.f4_filter_transform(w0, layout) if resolved[0] in ("staged_f4", "epilogue_f4") else ops.filter_transform(w0, layout)
         a0 = {"staged": ops.ALGO_STAGED, "epilogue": ops.ALGO_EPILOGUE, "fused": ops.ALGO_FUSED,
-              "staged_f4": ops.ALGO_STAGED_F4}[resolved[0]]
+              "staged_f4": ops.ALGO_STAGED_F4, "epilogue_f4": ops.ALGO_EPILOGUE_F4}[resolved[0]]
         out["ms_per_step_filters_prepared"] = round(
             timed(lambda: ops.conv_prepared(x0, U0, K0, 1, layout, algo=a0, out=y0), args.steps, args.warmup)[0], 4)
 

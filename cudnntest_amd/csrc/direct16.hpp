@@ -42,6 +42,7 @@ struct D16Geom {
     int N, C, K, H, W, pad, Ho, Wo;
     int BR, BC;            // output rows x columns of a block
     int WC;                // (8-wave kernel) waves side by side in a block
+    int ds;                // (8-wave kernel) pixel slots between the tap columns: 1, or N for CHWN tensors taken as one image of width W * N
     int PW, LR;            // LDS: pixel slots per row (BC + 2), rows (BR + 2 + 2 per image boundary a block can span)
     int PP;                // column pairs loaded per row
     int colBlocks, rowBlocks, kTiles;

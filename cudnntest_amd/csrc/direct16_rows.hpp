@@ -27,32 +27,41 @@
 
 namespace wino {
 
-template <int WF> struct D16R {
+// DIL: the tensors are [C][H][W][N] (CHWN).  A channel plane row of such a tensor is W * N contiguous elements in
+// which the horizontal neighbours of a pixel lie N elements away: the layer is a convolution of ONE image of width
+// W * N with the tap columns N elements apart and N * pad zeros on either side of a row, and that is how the kernel
+// runs it -- the same loads (neighbouring elements of a row in pairs: two images), the same stores, the tap columns
+// of a fragment g.ds pixel slots apart instead of one.  The halo of a block's rows is 2 N slots wide, so an input
+// stage is larger (6 rows x (128 + 2 N) slots with 128-filter tiles) and the filter ring is two deep instead of three.
+template <int WF, bool DIL = false> struct D16R {
     static constexpr int KT = 64 * WF;                       // filters per tile
     static constexpr int WP = 8 / WF;                        // waves along the rows of a block
     static constexpr int FB = 9 * 2 * KT * 16;               // bytes of a filter stage: [tap][channel vector][KT] vectors
-    static constexpr int XPLANE = WF == 2 ? 704 : 1360;      // pixel slots per channel-vector plane (LR * PW must fit)
+    static constexpr int XPLANE = DIL ? (WF == 2 ? 1152 : 1920) : (WF == 2 ? 704 : 1360);   // pixel slots per channel-vector plane (LR * PW must fit)
     static constexpr int XB = 2 * XPLANE * 16;               // bytes of an input stage
-    static constexpr int LDS = 3 * FB + 2 * XB;
+    static constexpr int NFR = DIL ? 2 : 3;                  // filter stages in the ring
+    static constexpr int LDS = NFR * FB + 2 * XB;
     static constexpr int FROWS = 18 * WF;                    // 1 KB rows of a filter stage
     static constexpr int NF = (FROWS + 7) / 8;               // filter requests per wave and stage (some rows twice)
-    static constexpr int NTASK = WF == 2 ? 2 : 3;            // input tasks per thread and stage
+    static constexpr int NTASK = DIL ? (WF == 2 ? 3 : 4) : (WF == 2 ? 2 : 3);   // input tasks per thread and stage
 };
+static_assert(D16R<1, true>::LDS <= 160 * 1024 && D16R<2, true>::LDS <= 160 * 1024, "LDS of the CHWN instantiations");
 
 // XN: x is [N][H][W][C].  The 8 channels of a pixel's vector are 16 contiguous bytes of x: an input task is one pixel
 // slot of one channel vector (a 16-byte load, a 16-byte LDS write, zeros where the slot lies outside the image), the
 // two vectors of a pixel on neighbouring lanes.  YN: y is [N][Ho][Wo][K].  The multiplies take the pixel fragment as
 // the first operand, so a lane holds one FILTER and its registers the pixels: the 32 filters of a wave's half are 64
 // contiguous bytes of a pixel of y.  The two are independent: a layer may read one layout and write the other.
-template <typename T, int WF, bool XN = false, bool YN = XN>
+template <typename T, int WF, bool XN = false, bool YN = XN, bool DIL = false>
 __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restrict__ x, const T* __restrict__ W9,
                                                                T* __restrict__ y, D16Geom g, Epilogue ep) {
     typedef typename Mma<T>::vec vec;
-    typedef D16R<WF> P;
+    typedef D16R<WF, DIL> P;
+    static_assert(!DIL || (!XN && !YN), "CHWN tensors on both sides");
     constexpr int NTASK = XN ? (2 * P::XPLANE + 511) / 512 : P::NTASK;   // input tasks per thread and stage
     constexpr int NX = XN ? NTASK : 8 * NTASK;                           // and the requests they make
-    extern __shared__ __attribute__((aligned(16))) unsigned char d16r_smem[];     // [3][FB] filters, [2][XB] input
-    unsigned char* const xsm = d16r_smem + 3 * P::FB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char d16r_smem[];     // [NFR][FB] filters, [2][XB] input
+    unsigned char* const xsm = d16r_smem + P::NFR * P::FB;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -99,8 +108,11 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         }
         const int m = t % g.PP, rr = t / g.PP;
         const int lr = rr % g.LR, v = min(rr / g.LR, 1);
-        const int slot0 = 2 * m - g.pad;                     // the pair (c0 + 2m - 2 pad, + 1) sits in slots (2m - pad, + 1)
-        tpk[q] = lr | (2 * m - 2 * g.pad + 8) << 8 | v << 20;
+        // padw zero columns left of a row (pad, or N * pad for CHWN); pairs start at even columns of the image:
+        // the pair (c0 + 2m - 2 ceil(padw / 2), + 1) sits in slots (2m - padw % 2, + 1)
+        const int padw = g.pad * g.ds, hp = (padw + 1) >> 1;
+        const int slot0 = 2 * m - (padw & 1);
+        tpk[q] = lr | (2 * m - 2 * hp + 64) << 8 | v << 20;
         const int wbits = (slot0 >= 0 && slot0 < g.PW ? 1 : 0) | (slot0 + 1 >= 0 && slot0 + 1 < g.PW ? 2 : 0);
         ldsw[q] = t < ntask ? (((v * P::XPLANE + lr * g.PW + slot0) * 16) | wbits) : 0;
     }
@@ -139,7 +151,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                 xoff[q] = ((unsigned)(((dnc * g.H + ihc) * g.W + iwc) * g.C + v * 8) * 2u) | (in ? 1u : 0u);   // a multiple of 16
                 continue;
             }
-            const int iw = t.c0 + ((tpk[q] >> 8) & 0xFFF) - 8;
+            const int iw = t.c0 + ((tpk[q] >> 8) & 0xFFF) - 64;
             const bool in = (ldsw[q] & 3) != 0 && t.n0 + dn < g.N && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
             const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 2);
             const int dnc = min(dn, g.N - 1 - t.n0);
@@ -272,7 +284,8 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 #pragma unroll
             for (int i = 0; i < 2; ++i) a[r][i] = *reinterpret_cast<const vec*>(fs + (3 * r + s) * (2 * P::KT * 16) + i * 512);
         };
-        auto ldb = [&](int t) { b[t % 3] = *reinterpret_cast<const vec*>(xrow[t % 6] + (t / 6) * 16); };
+        const int dsb = g.ds * 16;                           // bytes between the tap columns of a fragment
+        auto ldb = [&](int t) { b[t % 3] = *reinterpret_cast<const vec*>(xrow[t % 6] + (DIL ? (t / 6) * dsb : (t / 6) * 16)); };
         lda(0, 0);
         ldb(0);
         lda(1, 0);
@@ -440,10 +453,11 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             }
     };
 
-    // the filters of the stage after the next, into the ring slot that was read last in the previous stage
+    // the filters of the stage after the next, into the ring slot that was read last in the previous stage (a ring of
+    // two: the next stage's, into the other slot)
     auto f_next = [&](int fslot) {
         if (!cf.valid) return false;
-        f_request(cf, fslot == 0 ? 2 : fslot - 1);
+        f_request(cf, P::NFR == 2 ? fslot ^ 1 : (fslot == 0 ? 2 : fslot - 1));
         advance(cf);
         return true;
     };
@@ -483,7 +497,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     const int site = (wave >> 2) == 0 ? 2 + (wave & 1) : (wave & 1);
     f_request(cf, 0);
     advance(cf);
-    if (cf.valid) {
+    if (P::NFR > 2 && cf.valid) {
         f_request(cf, 1);
         advance(cf);
     }
@@ -523,11 +537,14 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                 x_commit(xslot ^ 1);
                 pending = false;
             }
+            // (a filter ring of two: the filters requested now are read in the next stage, so they go first and
+            // only the input requests may still be on their way at the stage's end)
+            if (P::NFR == 2) f_next(fslot);
             if (cx.valid) {
                 x_request();
                 xreq = true;
             }
-            freq = f_next(fslot);
+            if (P::NFR > 2) freq = f_next(fslot);
         });
         const int newest = (xreq ? NX : 0) + (freq ? P::NF : 0);
         if (cs == nst - 1) {
@@ -538,7 +555,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         } else {
             wait_barrier(newest);
         }
-        fslot = fslot == 2 ? 0 : fslot + 1;
+        fslot = fslot == P::NFR - 1 ? 0 : fslot + 1;
         xslot ^= 1;
         if (++cs == nst) {
             cs = 0;

@@ -813,7 +813,7 @@ bool direct16_plan(const Geometry& g, int npg, bool rows, D16Geom* d) {
         while (BR > 1 && (lr_of(BR) * PW > D16_PLANE || 2 * lr_of(BR) * PP > 768)) --BR;
     if (lr_of(BR) * PW > D16_PLANE || 2 * lr_of(BR) * PP > 768) return false;
     d->N = g.N; d->C = g.C; d->K = g.K; d->H = g.H; d->W = g.W; d->pad = g.pad; d->Ho = g.Ho; d->Wo = g.Wo;
-    d->BR = BR; d->BC = BC; d->PW = PW; d->LR = lr_of(BR); d->PP = PP;
+    d->BR = BR; d->BC = BC; d->PW = PW; d->LR = lr_of(BR); d->PP = PP; d->WC = 1; d->ds = 1;
     d->colBlocks = (g.Wo + BC - 1) / BC;
     d->rowBlocks = (int)((G + BR - 1) / BR);
     d->maxcross = (g.Ho + BR - 2) / g.Ho;
@@ -826,9 +826,20 @@ bool direct16_plan(const Geometry& g, int npg, bool rows, D16Geom* d) {
 
 // The 8-wave kernel of direct16_rows.hpp: blocks of 32/WF rows x 32 columns whose waves own 4 consecutive rows of one
 // image.  WF = 2 (128 filters per tile) when that wastes no filters, else 1.
-template <int WF>
-bool direct16_rows_plan(const Geometry& g, D16Geom* d) {
-    typedef D16R<WF> P;
+// DIL: a CHWN layer taken as ONE image of width W * N whose tap columns lie N elements apart (direct16_rows.hpp).
+template <int WF, bool DIL = false>
+bool direct16_rows_plan(const Geometry& gl, D16Geom* d) {
+    typedef D16R<WF, DIL> P;
+    Geometry g = gl;
+    int ds = 1;
+    if (DIL) {
+        // (pairs of neighbouring elements are two images; the zero columns of a row must fit the task encoding)
+        if (gl.N % 2 != 0 || (long)gl.pad * gl.N > 64 || (long)gl.W * gl.N >= (1L << 24)) return false;
+        ds = gl.N;
+        g.N = 1;
+        g.W = gl.W * gl.N;
+        g.Wo = gl.Wo * gl.N;
+    }
     const long G = (long)g.N * g.Ho;
     if (g.Ho % 4 != 0 || g.K % 64 != 0 || g.Wo % 2 != 0) return false;
     // the block's waves (4 rows x 32 columns each) side by side until they span the image, the rest stacked
@@ -837,11 +848,12 @@ bool direct16_rows_plan(const Geometry& g, D16Geom* d) {
     const int BR = 4 * (P::WP / WC), BC = 32 * WC;
     if (G < BR) return false;
     const int maxcross = g.Ho % BR == 0 ? 0 : (g.Ho + BR - 2) / g.Ho;     // images a block's rows can span beyond the first
-    const int PW = std::min(BC, (g.Wo + 1) / 2 * 2) + 2;      // slots of an LDS row: the block's columns (or the image's) + 2
-    const int LR = BR + 2 + 2 * maxcross, PP = (PW - 2) / 2 + 1 + g.pad;
+    const int PW = std::min(BC, (g.Wo + 1) / 2 * 2) + 2 * ds; // slots of an LDS row: the block's columns (or the image's) + the two tap columns
+    const int padw = g.pad * ds;                              // zero columns left of a row; pairs start at even columns
+    const int LR = BR + 2 + 2 * maxcross, PP = (PW + (padw & 1) + 1) / 2;
     if (LR * PW > P::XPLANE || 2 * LR * PP > P::NTASK * 512 || LR > 255 || PW > 2048) return false;
     d->N = g.N; d->C = g.C; d->K = g.K; d->H = g.H; d->W = g.W; d->pad = g.pad; d->Ho = g.Ho; d->Wo = g.Wo;
-    d->BR = BR; d->BC = BC; d->WC = WC; d->PW = PW; d->LR = LR; d->PP = PP;
+    d->BR = BR; d->BC = BC; d->WC = WC; d->PW = PW; d->LR = LR; d->PP = PP; d->ds = ds;
     d->colBlocks = (g.Wo + BC - 1) / BC;
     d->rowBlocks = (int)((G + BR - 1) / BR);
     d->maxcross = maxcross;
@@ -853,18 +865,19 @@ bool direct16_rows_plan(const Geometry& g, D16Geom* d) {
 }
 inline int direct16_rows_wf(const Geometry& g) { return (g.K % 128 == 0 || g.K > 256) ? 2 : 1; }
 
-template <typename T, int WF, bool XN = false, bool YN = XN>
+template <typename T, int WF, bool XN = false, bool YN = XN, bool DIL = false>
 int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
     static std::atomic<bool> attr_set{false};    // (per instantiation; setting it twice from two threads is harmless)
     if (!attr_set.load(std::memory_order_acquire)) {
-        HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, XN, YN>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    D16R<WF>::LDS));
+        HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, XN, YN, DIL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    D16R<WF, DIL>::LDS));
         attr_set.store(true, std::memory_order_release);
     }
     // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs
     const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
     const long blocks = std::max<long>(8, std::min<long>(device_cus(), (tiles + 7) / 8 * 8) / 8 * 8);
-    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN>), dim3((unsigned)blocks), dim3(512), D16R<WF>::LDS, st, (const T*)x,
+    constexpr int kLds = D16R<WF, DIL>::LDS;
+    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN, DIL>), dim3((unsigned)blocks), dim3(512), kLds, st, (const T*)x,
                        (const T*)W9, (T*)y, d, ep);
     LAUNCH_CHECK("direct16_rows");
     return WINO_OK;
@@ -872,16 +885,20 @@ int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, 
 
 size_t direct16_bank_bytes(const Geometry& g) { return (size_t)9 * round_up(g.C, 32) * round_up(g.K, 128) * 2; }
 
-// whether a layer runs on the 8-wave kernel (given 4-byte aligned tensors)
-bool direct16_big(const Geometry& g, D16Geom* d) {
-    const bool plan = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, d) : direct16_rows_plan<1>(g, d);
+// whether a layer runs on the 8-wave kernel (given 4-byte aligned tensors); chwn: as one image of width W * N
+bool direct16_big(const Geometry& g, D16Geom* d, bool chwn = false) {
+    const bool plan = chwn ? (direct16_rows_wf(g) == 2 ? direct16_rows_plan<2, true>(g, d) : direct16_rows_plan<1, true>(g, d))
+                           : (direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, d) : direct16_rows_plan<1>(g, d));
     return plan && (long)d->rowBlocks * d->colBlocks * d->kTiles >= device_cus() / 2;
 }
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
     D16Geom d;
-    if (dtype == WINO_F32 || src == WINO_CHWN || dst == WINO_CHWN || g.C % 8 != 0 || g.pad > 1 ||
-        (long)g.N * g.K * g.Ho * g.Wo >= (1L << 31))
-        return false;
+    if (dtype == WINO_F32 || g.C % 8 != 0 || g.pad > 1 || (long)g.N * g.K * g.Ho * g.Wo >= (1L << 31)) return false;
+    if (src == WINO_CHWN || dst == WINO_CHWN) {
+        // CHWN on both sides: the 8-wave kernel only, no pooling (a pooling window's columns are N elements apart);
+        // 32-bit byte offsets inside a stage's 16 channel planes
+        return src == dst && !(flags & WINO_FLAG_POOL2) && (long)g.H * g.W * g.N * 2 * 16 < (1L << 32) && direct16_big(g, &d, true);
+    }
     if (src == WINO_NHWC || dst == WINO_NHWC) {
         // an NHWC side: the 8-wave kernel only; offsets inside a block's images are 32-bit
         if (!direct16_big(g, &d)) return false;
@@ -918,7 +935,8 @@ int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const
 enum { D16_PACK_RUN = 0, D16_PACK = 1, D16_RUN = 2 };
 int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x,
                     const void* w, void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN) {
-    const bool nhwc = layout == WINO_NHWC, ynhwc = dst == WINO_NHWC;
+    const bool nhwc = layout == WINO_NHWC, ynhwc = dst == WINO_NHWC, chwn = layout == WINO_CHWN;
+    if (chwn != (dst == WINO_CHWN)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: CHWN tensors on both sides or on neither");
     if (misaligned(x, nhwc ? 16 : 4))
         return fail(WINO_ERR_UNSUPPORTED, "the 16-bit direct path loads column pairs (NHWC: channel vectors): x must be 4-byte (16-byte) aligned");
     D16Geom d;
@@ -926,7 +944,8 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
     // the chip short of tiles
     int npg = 4, wf = direct16_rows_wf(g);
     const bool pool = (flags & WINO_FLAG_POOL2) != 0;        // (pooled values are stored one by one: no alignment asked of y)
-    const bool big = (pool || !misaligned(y, 4)) && direct16_big(g, &d);
+    const bool big = (pool || !misaligned(y, 4)) && !(chwn && pool) && direct16_big(g, &d, chwn);
+    if (chwn && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of CHWN tensors: the 8-wave kernel's layer shapes, an even batch, no pooling, y 4-byte aligned");
     if ((nhwc || ynhwc) && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of NHWC tensors: the 8-wave kernel's layer shapes, y 4-byte aligned");
     if (pool && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: pooling needs the 8-wave kernel's layer shapes");
     const bool rows = !big && direct16_plan(g, 4, true, &d) && (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
@@ -940,7 +959,7 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
     const Epilogue ep = make_epilogue(flags, bias);
     const FltStrides fs = flt_strides(layout, g.K, g.C);
     dim3 pgrid((d.Kp + 63) / 64, d.CQ);
-    const bool pvec = g.C % 8 == 0 && !misaligned(w, 16);
+    const bool pvec = g.C % 8 == 0 && !misaligned(w, 16) && !chwn;          // ([C][3][3][K] banks: element by element)
 #define D16_GO(T)                                                                                                  \
     if (mode != D16_RUN) {                                                                                         \
         if (pvec && nhwc) hipLaunchKernelGGL((direct16_pack_kernel<T, 2>), pgrid, dim3(64), 0, st, (const T*)w, (T*)W9, fs, g.K, g.C, d.Kp, d.CQ); \
@@ -949,6 +968,8 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
         LAUNCH_CHECK("direct16_pack");                                                                             \
     }                                                                                                              \
     if (mode == D16_PACK) return WINO_OK;                                                                          \
+    if (chwn) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, false, true>(d, ep, x, W9, y, st);         \
+                return launch_direct16_rows_t<T, 1, false, false, true>(d, ep, x, W9, y, st); }                    \
     if (nhwc && ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, true>(d, ep, x, W9, y, st);        \
                          return launch_direct16_rows_t<T, 1, true, true>(d, ep, x, W9, y, st); }                   \
     if (nhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, false>(d, ep, x, W9, y, st);                \
@@ -1018,6 +1039,14 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     if (!direct16_ok(src, dst, dtype, flags, g) || misaligned(x, src == WINO_NHWC ? 16 : 4)) return false;
     if ((src == WINO_NHWC || dst == WINO_NHWC) && !(flags & WINO_FLAG_POOL2) && misaligned(y, 4)) return false;
     D16Geom d;
+    if (src == WINO_CHWN) {                    // (both sides, direct16_ok has checked; the 8-wave kernel only)
+        if (misaligned(y, 4)) return false;
+        const bool planc = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2, true>(g, &d) : direct16_rows_plan<1, true>(g, &d);
+        // (measured at N = 32 in bf16, direct against the fastest Winograd pipeline: 177 against 532 us at C = K = 64,
+        // H = 224; 140 against 307 at C = K = 128, H = 112; 73 against 91 and 130 against 183 at 56 x 56; at 28 x 28 the
+        // 7 x 7 blocks of a filter tile leave a quarter of the chip idle: 121 against 72, 225 against 128 us)
+        return planc && g.Ho >= 48 && g.Wo >= 48 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus();
+    }
     const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d);
     if (plan8 && g.Ho >= 28 && g.Wo >= 28 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus()) return true;
     if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 48 || g.Wo < 48) return false;
@@ -1734,7 +1763,7 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
         // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte NCHW and NHWC layers)
-        const bool direct16_layer = dtype != WINO_F32 && L.layout_in != WINO_CHWN && L.layout_out != WINO_CHWN && L.C % 8 == 0;
+        const bool direct16_layer = dtype != WINO_F32 && (L.layout_in == WINO_CHWN) == (L.layout_out == WINO_CHWN) && L.C % 8 == 0;
         if (e == hipSuccess && (L.C <= 4 || direct16_layer)) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         // what AUTO runs outside the F(2x2) kernels gets its filters prepared once as well
         if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && auto_f4(dtype, g)) {

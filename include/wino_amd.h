@@ -83,10 +83,14 @@ typedef enum {
                                the source's layout), C a multiple of 8 and, from NHWC, a 16-byte aligned x run on the
                                larger of its two kernels (the 8-wave one) when the layer has its shape: output height a multiple of 4, even output width, K a multiple of 64, at least a
                                tile for every other CU; other NHWC layers are refused (WINO_ERR_UNSUPPORTED).
+                               2-byte CHWN -> CHWN layers (comparison/wrapedConv_CHWN.cuh:16-82) run on the same kernel, taken as one
+                               image of width W * N whose tap columns lie N elements apart: the same shape conditions, an
+                               even batch of at most 32 images (more where the rows are short), x and y 4-byte aligned, no
+                               pooling; other CHWN layers, and layers with CHWN on one side only, are refused.
                                Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (the
                                shape just named), not for C <= 4; needs the filter bank itself (not
                                wino_conv_prepared).
-                               What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW and NHWC layers. */
+                               What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW, NHWC and CHWN layers. */
     WINO_ALGO_EPILOGUE_F4 = 6 /* F(4x4,3x3) with the output transform A^T (.) A in the epilogue of the 36-way GEMM: no
                                product tensor in HBM.  The arrangement of the reference's fused F(4x4) kernels
                                (fusedTest/winotrans.cuh:1530-1574: 36 running products, A^T acc A in registers, 16

@@ -129,6 +129,75 @@ def test_nhwc_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
         assert err <= (1e-3 if dtype == ops.F16 else 5e-3), err
 
 
+# (N, C, K, H, W, pad) for [C][H][W][N] tensors, which the 8-wave kernel takes as ONE image of width W * N with its tap
+# columns N elements apart:
+#   * N = 32, 128-filter tiles: a block is 4 rows x 4 columns x 32 images, 14 x 14 blocks per filter tile;
+#   * N = 32, K = 64 (64-filter tiles, 8 waves side by side: 8 columns x 32 images), a last stage half past C;
+#   * N = 8: four columns to a wave, a row of 60 x 8 elements that ends inside a block; K = 192, no padding;
+#   * N = 6: pairs of images, a block's 128 elements are 21 1/3 columns;
+#   * 28 x 28 images, 512 filters: 7 x 7 blocks per filter tile, 16 stages.
+CHWN_SHAPES = [(32, 64, 128, 56, 56, 1), (32, 24, 64, 64, 80, 1), (8, 16, 192, 130, 62, 0), (6, 32, 256, 96, 100, 1),
+               (32, 256, 512, 28, 28, 1)]
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", CHWN_SHAPES)
+def test_chwn_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
+    """[C][H][W][N] tensors and [C][3][3][K] filters.  Whole tensors against the staged Winograd pipeline from the same
+    layout and against the NCHW direct kernel (same products, same order of summation: the same bits), planes of
+    the first and last image against the oracle; twice; floats within the direct path's rounding."""
+    N, C, K, H, W, pad = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -1, 1).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    xl, wl = synth.act_to_layout(x, ops.CHWN), synth.flt_to_layout(w, ops.CHWN)
+    xd, wd, bd = dev(xl, dtype), dev(wl, dtype), dev(bias, dtype)
+    if shape[:5] == (32, 64, 128, 56, 56):                  # what AUTO takes for such layers (at 28 x 28: Winograd)
+        assert ops.pick_algo(ops.CHWN, dtype, N, C, K, H, W, pad) == ops.ALGO_DIRECT
+    if shape[:5] == (32, 256, 512, 28, 28):
+        assert ops.pick_algo(ops.CHWN, dtype, N, C, K, H, W, pad) != ops.ALGO_DIRECT
+    ref = ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_STAGED, relu=True, bias=bd)
+    nchw = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+    ks = sorted({0, K // 2, K - 1})
+    for rep in range(2):
+        got = ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+        assert torch.equal(got, ref), rep
+        assert torch.equal(got.permute(3, 0, 1, 2), nchw), rep
+        for n in (0, N - 1):
+            want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], pad) + bias[ks][None, :, None, None], 0)
+            assert np.array_equal(host(got.permute(3, 0, 1, 2)[n:n + 1][:, ks]), rounded(want.astype(np.float32), dtype, oracle)), (rep, n)
+    # pooling windows span columns N elements apart: not in this kernel's stores; other layouts on one side neither
+    with pytest.raises(_lib.WinoError) as e:
+        ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+    assert e.value.code == -2
+    with pytest.raises(_lib.WinoError) as e:
+        ops.conv(xd, wd, pad, ops.CHWN, ops.NCHW, algo=ops.ALGO_DIRECT)
+    assert e.value.code == -2
+    assert torch.equal(ops.conv(xd, wd, pad, ops.CHWN, relu=True, bias=bd, pool=True),
+                       ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True))
+    # floats: only the final rounding separates it from the oracle
+    xf, wf = synth.conv_inputs(N, C, K, H, W, seed=5 + sum(shape))
+    xr, wr = rounded(xf, dtype, oracle), rounded(wf, dtype, oracle)
+    gotf = ops.conv(dev(synth.act_to_layout(xr, ops.CHWN), dtype), dev(synth.flt_to_layout(wr, ops.CHWN), dtype), pad, ops.CHWN,
+                    algo=ops.ALGO_DIRECT)
+    for n in (0, N - 1):
+        err = oracle.rel_l2(host(gotf.permute(3, 0, 1, 2)[n:n + 1]), oracle.direct_conv(xr[n:n + 1], wr, pad))
+        assert err <= (1e-3 if dtype == ops.F16 else 5e-3), err
+
+
+def test_chwn_layers_the_8_wave_kernel_does_not_take():
+    """An odd batch, a batch whose halo does not fit the LDS plane (N = 64), an output height off the 4-row strips: refused
+    by name, and the automatic choice runs them through the Winograd pipelines."""
+    for (N, C, K, H) in [(5, 16, 64, 32), (64, 16, 128, 32), (16, 16, 64, 30)]:
+        x = torch.zeros((C, H, H, N), device="cuda", dtype=torch.bfloat16)
+        w = torch.zeros((C, 3, 3, K), device="cuda", dtype=torch.bfloat16)
+        with pytest.raises(_lib.WinoError) as e:
+            ops.conv(x, w, 1, ops.CHWN, algo=ops.ALGO_DIRECT)
+        assert e.value.code == -2
+        assert ops.pick_algo(ops.CHWN, ops.BF16, N, C, K, H, H, 1) != ops.ALGO_DIRECT
+        ops.conv(x, w, 1, ops.CHWN)
+
+
 @pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
 @pytest.mark.parametrize("shape", [(2, 64, 64, 56, 56), (1, 128, 256, 28, 28), (3, 256, 64, 14, 14)])
 def test_floats_within_tolerance(oracle, shape, dtype):
