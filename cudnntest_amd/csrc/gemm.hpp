@@ -67,6 +67,14 @@ __device__ __forceinline__ void dma_row(uint64_t sbase, unsigned lane_off, void*
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(sbase) : "memory");
 }
 
+// a wave-uniform 64-bit value, for the compiler too (scalar registers): values that are uniform by construction
+// (derived from the workgroup id and kernel arguments through a cursor the compiler keeps in memory) still have to
+// reach the scalar operands of dma_row
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
 constexpr int GEMM_BM = 128, GEMM_BN = 128;
 
 constexpr int GO_T = 64;   // patch edge (filters and tiles)

@@ -40,13 +40,6 @@ constexpr int GF4_OPND = 6 * GF4_PLANE;                // one operand's stage: 2
 constexpr int GF4_LDS = GF4_RING * 2 * GF4_OPND;       // 144 KB
 constexpr int GF4_PART = 128 * 512;                    // floats of a patch's partial outputs: [128 registers][512 threads]
 
-// a wave-uniform 64-bit value, for the compiler too (scalar registers): the cursor below is uniform by construction,
-// which the compiler cannot always see
-__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return ((uint64_t)hi << 32) | lo;
-}
-
 // dma_row with the LDS destination as a byte address in a scalar register (no pointer conversion per request)
 __device__ __forceinline__ void dma_row_to(uint64_t sbase, unsigned lane_off, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(sbase) : "memory");

@@ -865,20 +865,41 @@ bool direct16_rows_plan(const Geometry& gl, D16Geom* d) {
 }
 inline int direct16_rows_wf(const Geometry& g) { return (g.K % 128 == 0 || g.K > 256) ? 2 : 1; }
 
+// Scratch of the 8-wave direct kernel for the workgroups that share a tile: one block of partial sums per workgroup
+// (128 registers x 512 threads) and an arrival counter each (the arena's first 4 KB).
+struct D16Share {
+    float* part = nullptr;
+    int* cnt = nullptr;
+};
+constexpr size_t kD16PartPerWg = (size_t)128 * 512 * sizeof(float);
+size_t direct16_part_bytes() { return (size_t)(device_cus() / 8 * 8) * kD16PartPerWg; }
+
 template <typename T, int WF, bool XN = false, bool YN = XN, bool DIL = false>
-int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
+int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, const D16Share& sh,
+                           hipStream_t st) {
     static std::atomic<bool> attr_set{false};    // (per instantiation; setting it twice from two threads is harmless)
     if (!attr_set.load(std::memory_order_acquire)) {
         HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, XN, YN, DIL>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     D16R<WF, DIL>::LDS));
         attr_set.store(true, std::memory_order_release);
     }
-    // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs
+    // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs.  The
+    // tiles left over after the full rounds are shared out by stages (partial sums through scratch) when they would
+    // occupy at most half of the workgroups: sharing costs a workgroup about six stage times (its accumulators out and
+    // in, two or three partial tiles to set up instead of one), so a last round that is three quarters full is better
+    // left alone (measured at N = 32 in bf16, shared against whole: C = K = 256 at 56 x 56, 24 tiles over 32 workgroups
+    // of an XCD, 136 against 129 us; C = K = 512 at 28 x 28, 28 over 32, 131 against 125 us).
     const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
-    const long blocks = std::max<long>(8, std::min<long>(device_cus(), (tiles + 7) / 8 * 8) / 8 * 8);
+    const long per_xcd = ((long)d.rowBlocks * d.colBlocks + 7) / 8 * d.kTiles;      // tiles of the XCD with the most
+    const long sx_all = std::max<long>(1, device_cus() / 8);
+    const long left_over = per_xcd % sx_all;
+    // (a run of at least four stages to every workgroup, or the kernel deals the left-over tiles out whole anyway)
+    const bool share = sh.part && left_over > 0 && 2 * left_over <= sx_all && left_over * (d.CQ / 2) >= 4 * sx_all &&
+                       sx_all * 8 <= (long)(kCounterBytes / sizeof(int));
+    const long sx = share ? sx_all : std::max<long>(1, std::min<long>(sx_all, (tiles + 7) / 8));
     constexpr int kLds = D16R<WF, DIL>::LDS;
-    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN, DIL>), dim3((unsigned)blocks), dim3(512), kLds, st, (const T*)x,
-                       (const T*)W9, (T*)y, d, ep);
+    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN, DIL>), dim3((unsigned)(sx * 8)), dim3(512), kLds, st, (const T*)x,
+                       (const T*)W9, (T*)y, d, ep, share ? sh.part : nullptr, share ? sh.cnt : nullptr, 1 << 22);
     LAUNCH_CHECK("direct16_rows");
     return WINO_OK;
 }
@@ -934,7 +955,7 @@ int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const
 // for tensors of the same alignment.
 enum { D16_PACK_RUN = 0, D16_PACK = 1, D16_RUN = 2 };
 int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x,
-                    const void* w, void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN) {
+                    const void* w, void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN, const D16Share& sh = D16Share{}) {
     const bool nhwc = layout == WINO_NHWC, ynhwc = dst == WINO_NHWC, chwn = layout == WINO_CHWN;
     if (chwn != (dst == WINO_CHWN)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: CHWN tensors on both sides or on neither");
     if (misaligned(x, nhwc ? 16 : 4))
@@ -968,16 +989,16 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
         LAUNCH_CHECK("direct16_pack");                                                                             \
     }                                                                                                              \
     if (mode == D16_PACK) return WINO_OK;                                                                          \
-    if (chwn) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, false, true>(d, ep, x, W9, y, st);         \
-                return launch_direct16_rows_t<T, 1, false, false, true>(d, ep, x, W9, y, st); }                    \
-    if (nhwc && ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, true>(d, ep, x, W9, y, st);        \
-                         return launch_direct16_rows_t<T, 1, true, true>(d, ep, x, W9, y, st); }                   \
-    if (nhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, false>(d, ep, x, W9, y, st);                \
-                return launch_direct16_rows_t<T, 1, true, false>(d, ep, x, W9, y, st); }                           \
-    if (ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, true>(d, ep, x, W9, y, st);               \
-                 return launch_direct16_rows_t<T, 1, false, true>(d, ep, x, W9, y, st); }                          \
-    if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, st);                                  \
-    if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, st);                                             \
+    if (chwn) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, false, true>(d, ep, x, W9, y, sh, st);         \
+                return launch_direct16_rows_t<T, 1, false, false, true>(d, ep, x, W9, y, sh, st); }                    \
+    if (nhwc && ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, true>(d, ep, x, W9, y, sh, st);        \
+                         return launch_direct16_rows_t<T, 1, true, true>(d, ep, x, W9, y, sh, st); }                   \
+    if (nhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, false>(d, ep, x, W9, y, sh, st);                \
+                return launch_direct16_rows_t<T, 1, true, false>(d, ep, x, W9, y, sh, st); }                           \
+    if (ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, true>(d, ep, x, W9, y, sh, st);               \
+                 return launch_direct16_rows_t<T, 1, false, true>(d, ep, x, W9, y, sh, st); }                          \
+    if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, sh, st);                                  \
+    if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, sh, st);                                             \
     if (rows) return launch_direct16_t<T, 4, true>(d, ep, x, W9, y, st);                                           \
     if (npg == 4) return launch_direct16_t<T, 4, false>(d, ep, x, W9, y, st);                                      \
     if (npg == 2) return launch_direct16_t<T, 2, false>(d, ep, x, W9, y, st);                                      \
@@ -1162,11 +1183,20 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (!direct16_ok(src, dst, dtype, flags, g))
             return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for pad 0 and 1: for C <= 4, and for 2-byte NCHW tensors with "
                                               "C a multiple of 8 and an even width (pooling: output height a multiple of 4, K a multiple of 64, a large layer)");
+        // counters, the re-ordered bank, and the partial sums of workgroups that share a tile (left out, and the
+        // tiles run whole, where a fixed scratch buffer has no room for them)
         void* base = nullptr;
-        const int rcb = ss.get(kCounterBytes + direct16_bank_bytes(g), &base);
+        const size_t bank = (direct16_bank_bytes(g) + 255) / 256 * 256;
+        const bool share = !ss.fixed || kCounterBytes + bank + direct16_part_bytes() <= ss.fixed_bytes;
+        const int rcb = ss.get(kCounterBytes + bank + (share ? direct16_part_bytes() : 0), &base);
         if (rcb) return rcb;
+        D16Share sh;
+        if (share) {
+            sh.part = (float*)((char*)base + kCounterBytes + bank);
+            sh.cnt = (int*)base;
+        }
         StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-        return launch_direct16(src, dst, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
+        return launch_direct16(src, dst, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream, D16_PACK_RUN, sh);
     }
     if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4)
         return conv_f4_impl(ss, src, dst, dtype, algo, flags, bias, N, C, K, H, W, pad, x, w, Upre, y, stream);
@@ -1697,8 +1727,14 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
         } else if (L.W9 && !misaligned(in, 4) && (!misaligned(out, 4) || (L.flags & WINO_FLAG_POOL2)) &&
                    auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in, out)) {
             // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
+            void* base = nullptr;                           // the partial sums of workgroups that share a tile: the arena
+            rc = arena_get(kCounterBytes + direct16_part_bytes(), &base);
+            if (rc) return rc;
+            D16Share sh;
+            sh.part = (float*)((char*)base + kCounterBytes);
+            sh.cnt = (int*)base;
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-            rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
+            rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN, sh);
         } else {
             rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
                            L.wraw, L.U, bias, out, stream);
@@ -1839,6 +1875,7 @@ int wino_stack_forward_graph(wino_stack_t* s, const void* x, void* y, void* stre
         Geometry g;
         if (!make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g)) return fail(WINO_ERR_INVALID, "bad layer shape");
         need = std::max(need, scratch_layout(g, s->dtype).total);
+        if (L.W9) need = std::max(need, kCounterBytes + direct16_part_bytes());
         Geometry g4;
         if (L.U4 && make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4))
             need = std::max(need, scratch_layout(g4, s->dtype, auto_f4_algo(s->dtype, g4)).total);

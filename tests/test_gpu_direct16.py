@@ -185,6 +185,33 @@ def test_chwn_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
         assert err <= (1e-3 if dtype == ops.F16 else 5e-3), err
 
 
+@pytest.mark.parametrize("shape,layout", [((46, 256, 128, 56, 56), ops.NCHW), ((46, 256, 128, 56, 56), ops.NHWC),
+                                          ((10, 512, 128, 56, 56), ops.NCHW), ((44, 256, 256, 56, 56), ops.NHWC),
+                                          ((24, 256, 256, 56, 56), ops.CHWN)])
+def test_left_over_tiles_shared_out_by_stages(oracle, shape, layout):
+    """Layers whose last round of tiles would occupy at most half of the workgroups: the 8-wave kernel cuts the stage
+    sequence of those tiles into equal runs, workgroups leave partial sums of the tiles they share in scratch and the
+    tile's owner adds them in a fixed order.  One full round and nine tiles more per XCD; a fraction of a round only
+    (every workgroup holds parts of tiles); two filter tiles, two rounds and fourteen tiles; a CHWN layer.  Small integers: exact whatever the order of the sums --
+    the staged Winograd pipeline's bits, the oracle's planes, three times in a row (the arrival counters return to
+    zero)."""
+    N, C, K, H, W = shape
+    dtype = ops.BF16
+    x = synth.small_ints(N * C * H * W, sum(shape), -1, 1).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    xd, wd, bd = dev(synth.act_to_layout(x, layout), dtype), dev(synth.flt_to_layout(w, layout), dtype), dev(bias, dtype)
+    ref = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=bd)
+    ks = sorted({0, K // 2, K - 1})
+    for rep in range(3):
+        got = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+        assert torch.equal(got, ref), rep
+    g = synth.act_from_layout(host(got), layout)
+    for n in (0, N - 1):
+        want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], 1) + bias[ks][None, :, None, None], 0)
+        assert np.array_equal(g[n:n + 1][:, ks], rounded(want.astype(np.float32), dtype, oracle)), n
+
+
 def test_chwn_layers_the_8_wave_kernel_does_not_take():
     """An odd batch, a batch whose halo does not fit the LDS plane (N = 64), an output height off the 4-row strips: refused
     by name, and the automatic choice runs them through the Winograd pipelines."""
