@@ -170,6 +170,193 @@ __global__ __launch_bounds__(256) void direct_small_c_kernel(const T* __restrict
     }
 }
 
+// Direct 3x3 convolution for layers with FEW OUTPUT PIXELS and a reduction of any length (a batch of one image: the
+// reference's sweep starts at layer 1-2 with batch 1, comparison/layoutCompare.cu:38-46).  Such a layer is a few
+// microseconds of arithmetic; through the Winograd pipelines it is three dependent launches, each of which starts,
+// fills and drains a pipeline, and whose 64- and 128-wide patches occupy a fraction of the chip.  Here it is ONE
+// launch with the smallest unit the matrix instruction has: a workgroup computes a tile of 4 x 8 pixels for 32
+// filters, and its eight waves share the REDUCTION -- wave v takes channels 4v .. 4v+3, then 32 further on, 18
+// v_mfma_f32_32x32x2_f32 per group of 4 channels, the next group's operands on their way meanwhile -- so that a
+// layer with C = 64 is one chain of 36 multiplies per wave.  What binds such a kernel is the number of memory
+// instructions a CU can take (about one per 16 clocks, whatever its width), so a wave fetches a group with as few
+// as the layout allows and hands the elements to the lanes that multiply them through LDS of its own:
+//   * the input patch of a group, 4 channels x 6 x 10 elements (zeros where the padding is), is 4 loads per lane;
+//   * the filter block, 32 filters x 36 elements, is contiguous per filter in a [K][C][3][3] bank: 5 loads of 16
+//     bytes per lane (any other order, or C not a multiple of 4: 18 loads of one element);
+//   * the waves' partial sums meet in LDS and each wave stores two of the 16 filter rows of the sum (bias, ReLU).
+// Any layout on either side (element strides), any padding; the partial sums are added in wave order, so results do
+// not depend on the launch.
+constexpr int DFP_NE = 18;                  // multiplies per group of 4 channels
+constexpr int DFP_ROW = 37;                 // floats per filter in the wave's strip of LDS (36 + 1: the 32 lanes of a read hit 32 banks)
+constexpr int DFP_PATCH = 4 * 6 * 10;       // a group's input patch: 4 channels x (4 + 2) rows x (8 + 2) columns
+
+template <typename T>
+__global__ __launch_bounds__(512) void direct_few_pixels_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                T* __restrict__ y, ActStrides xs, FltStrides ws,
+                                                                ActStrides ys, int N, int C, int K, int H, int W, int pad,
+                                                                int Ho, int Wo, int tiles_y, int tiles_x, int PT,
+                                                                Epilogue ep) {
+    constexpr int NE = DFP_NE;
+    __shared__ float red[8][16][64];                          // the partial sums
+    __shared__ float strip[8][32 * DFP_ROW];                  // per wave, a group's filter block: [filter][channel * 9 + tap]
+    __shared__ float patch[8][DFP_PATCH];                     // per wave, a group's input patch: [channel][row][column]
+    __shared__ int tabw[36];                                  // byte offset of (channel, tap) 0 .. 35 of a group in w
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int pt = (int)(blockIdx.x % (unsigned)PT), kt = (int)(blockIdx.x / (unsigned)PT);
+    if (tid < 36) tabw[tid] = (int)((tid / 9) * ws.c + ((tid % 9) / 3) * ws.r + (tid % 3) * ws.s) * (int)sizeof(T);
+
+    // the workgroup's pixels: tile (n, ty, tx) of 4 rows x 8 columns; lane l32: row l32 / 8, column l32 % 8
+    const int n = pt / (tiles_y * tiles_x), trem = pt - n * tiles_y * tiles_x;
+    const int oh0 = (trem / tiles_x) * 4, ow0 = (trem % tiles_x) * 8;
+    const int py = l32 >> 3, px = l32 & 7;
+    // byte offsets fit 32 bits (the host checks the tensor sizes)
+
+    // Input patch as loaded: element 64 j + lane of [4][6][10], j < 4: byte offset in x relative to the group's
+    // first channel (0 and a zero mask where the element lies in the padding or past the patch).
+    unsigned offx[4], mx[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int p = 64 * j + lane;
+        const int c = (p * 1093) >> 16, rem = p - 60 * c;                    // p / 60, p % 60 (p < 256)
+        const int rr = (rem * 205) >> 11, cc = rem - 10 * rr;                 // rem / 10, rem % 10 (rem < 64)
+        const int ih = oh0 - pad + rr, iw = ow0 - pad + cc;
+        const bool in = p < DFP_PATCH && ih >= 0 && ih < H && iw >= 0 && iw < W;
+        offx[j] = in ? (unsigned)((int)(n * xs.n + c * xs.c + ih * xs.h + iw * xs.w) * (int)sizeof(T)) : 0u;
+        mx[j] = in ? 0xFFFFFFFFu : 0u;
+    }
+    __syncthreads();
+    // Filter block as loaded: a bank in [K][C][3][3] order holds a filter's 36 elements of a group contiguously:
+    // 16-byte piece 64 j + lane of the [32][9] pieces, j < 5.  Any other order: element 64 j + lane of [32][36],
+    // j < 18.  Byte offset in w relative to the group's first channel, mask (filters past K), place in the strip.
+    const bool wide = ws.s == 1 && ws.r == 3 && ws.c == 9 && (C & 3) == 0;
+    unsigned offw[NE], mw[NE];
+    int sidx[NE];
+#pragma unroll
+    for (int j = 0; j < NE; ++j) {
+        const int idx = 64 * j + lane;
+        if (wide) {
+            const int fk = (idx * 7282) >> 16, part = idx - 9 * fk;           // idx / 9, idx % 9 (idx < 320)
+            const bool fok = j < 5 && fk < 32 && kt * 32 + fk < K;
+            offw[j] = fok ? (unsigned)(((kt * 32 + fk) * (int)ws.k + 4 * part) * (int)sizeof(T)) : 0u;
+            mw[j] = fok ? 0xFFFFFFFFu : 0u;
+            sidx[j] = fk < 32 ? fk * DFP_ROW + 4 * part : 0;
+        } else {
+            const int fk = (idx * 1821) >> 16, fkk = idx - 36 * fk;           // idx / 36, idx % 36 (idx < 1152)
+            const bool fok = kt * 32 + fk < K;
+            offw[j] = fok ? (unsigned)(((kt * 32 + fk) * (int)ws.k) * (int)sizeof(T) + tabw[fkk]) : 0u;
+            mw[j] = fok ? 0xFFFFFFFFu : 0u;
+            sidx[j] = idx + fk;                                               // [fk][fkk] in rows of 37
+        }
+    }
+    const char* xg = reinterpret_cast<const char*>(x) + (size_t)(wave * 4) * xs.c * sizeof(T);   // this wave's group: first channel
+    const char* wg = reinterpret_cast<const char*>(w) + (size_t)(wave * 4) * ws.c * sizeof(T);
+    const size_t xstep = (size_t)32 * xs.c * sizeof(T), wstep = (size_t)32 * ws.c * sizeof(T);
+
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    // the group on its way: 4 patch elements; 5 filter pieces of 4 elements (wide) or 18 elements
+    T rb[4];
+    struct alignas(4) T4 { T v[4]; };
+    T4 rw4[5];
+    T rw[NE];
+    int cleft = 0;                                            // channels of that group that exist, counted from the wave's first
+    int crem = C - wave * 4;
+    auto load = [&]() __attribute__((always_inline)) {        // the group at xg, wg; the pointers move on
+        cleft = crem;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // (a channel past C: the first element of the group's first channel is read instead, and masked)
+            const int c = ((64 * j + lane) * 1093) >> 16;
+            rb[j] = *reinterpret_cast<const T*>(xg + (c < crem ? offx[j] : 0u));
+        }
+        if (wide) {
+#pragma unroll
+            for (int j = 0; j < 5; ++j) rw4[j] = *reinterpret_cast<const T4*>(wg + offw[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NE; ++j) {
+                const int idx = 64 * j + lane, fkk = idx - 36 * ((idx * 1821) >> 16);
+                rw[j] = *reinterpret_cast<const T*>(wg + (fkk < 9 * crem ? offw[j] : 0u));
+            }
+        }
+        xg += xstep;
+        wg += wstep;
+        crem -= 32;
+    };
+    float* const mine = strip[wave];
+    float* const mypatch = patch[wave];
+    float a[NE], b[NE];
+    // the group that has arrived -> the wave's strip and patch -> a, b: multiply e of a lane takes reduction index
+    // 18 lh + e of the group, (channel 2 lh + e / 9, tap e % 9)
+    auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int p = 64 * j + lane, c = (p * 1093) >> 16;
+            if (p < DFP_PATCH) mypatch[p] = __uint_as_float(__float_as_uint(to_f32(rb[j])) & (c < cleft ? mx[j] : 0u));
+        }
+        if (wide) {
+#pragma unroll
+            for (int j = 0; j < 5; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (j < 4 || lane < 32) mine[sidx[j] + i] = __uint_as_float(__float_as_uint(to_f32(rw4[j].v[i])) & mw[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NE; ++j) {
+                const int idx = 64 * j + lane, fkk = idx - 36 * ((idx * 1821) >> 16);
+                mine[sidx[j]] = __uint_as_float(__float_as_uint(to_f32(rw[j])) & (fkk < 9 * cleft ? mw[j] : 0u));
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const float* ar = mine + l32 * DFP_ROW + 18 * lh;
+        const float* br = mypatch + 120 * lh + py * 10 + px;
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            a[e] = ar[e];
+            b[e] = br[(e / 9) * 60 + ((e % 9) / 3) * 10 + e % 3];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+    // groups of this wave: channels 4 wave + 32 i
+    const int ng = C > wave * 4 ? (C - wave * 4 + 31) / 32 : 0;
+    if (ng > 0) load();
+#pragma unroll 1
+    for (int i = 0; i < ng; ++i) {
+        stage();
+        if (i + 1 < ng) load();
+#pragma unroll
+        for (int e = 0; e < NE; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+    }
+
+    // the eight partial sums meet in LDS; wave v adds and stores registers 2v and 2v + 1 of the sum: register r of a
+    // lane is filter 8 * (r / 4) + 4 * lh + r % 4 of the tile, the lane's pixel
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    const int oh = oh0 + py, ow = ow0 + px;
+    const long yq = n * ys.n + oh * ys.h + ow * ys.w;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int r = 2 * wave + j;
+        float v = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += red[u][r][lane];
+        const int kk = kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        if (oh < Ho && ow < Wo && kk < K) {
+            v += bias_of<T>(ep, kk);
+            if (ep.relu) v = fmaxf(v, 0.f);
+            y[yq + kk * ys.c] = from_f32<T>(v);
+        }
+    }
+}
+
 // The same for 2-byte tensors on the 16-bit matrix instruction: the 9*C <= 36 taps of an output are NE =
 // ceil(9*C/16) v_mfma_f32_32x32x16 (2 for C = 3) instead of 14 fp32 ones -- a fourteenth of the matrix time.
 // The products are the same (two 2-byte values multiply exactly in fp32 either way), only the order in which

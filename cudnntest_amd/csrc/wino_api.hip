@@ -788,6 +788,26 @@ int launch_direct(int src, int dst, int dtype, unsigned flags, const void* bias,
     DISPATCH_DTYPE(dtype, launch_direct_t<T>(src, dst, flags, bias, g, x, w, y, st));
 }
 
+// The one-launch kernel for fp32 layers with few output pixels (direct_few_pixels_kernel): offered while its units of
+// 4 x 8 pixels x 32 filters fit four rounds of the chip; pooled outputs stay on the Winograd path.
+long direct_few_units(const Geometry& g) { return (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 7) / 8) * ((g.K + 31) / 32); }
+bool direct_few_ok(int dtype, unsigned flags, const Geometry& g) {
+    return dtype == WINO_F32 && !(flags & WINO_FLAG_POOL2) && direct_few_units(g) <= 4L * device_cus() &&
+           (long)g.N * g.C * g.H * g.W < (1L << 29) && (long)g.N * g.K * g.Ho * g.Wo < (1L << 29) &&
+           (long)g.K * g.C * 9 < (1L << 29);                                                 // 32-bit byte offsets
+}
+int launch_direct_few(int src, int dst, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
+                      void* y, hipStream_t st) {
+    const int tiles_y = (g.Ho + 3) / 4, tiles_x = (g.Wo + 7) / 8, PT = g.N * tiles_y * tiles_x;
+    const ActStrides xs = act_strides(src, g.N, g.C, g.H, g.W), ys = act_strides(dst, g.N, g.K, g.Ho, g.Wo);
+    const FltStrides fs = flt_strides(src, g.K, g.C);
+    hipLaunchKernelGGL(direct_few_pixels_kernel<float>, dim3((unsigned)direct_few_units(g)), dim3(512), 0, st, (const float*)x,
+                       (const float*)w, (float*)y, xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, tiles_y, tiles_x, PT,
+                       make_epilogue(flags, bias));
+    LAUNCH_CHECK("direct_few_pixels");
+    return WINO_OK;
+}
+
 // ---- direct convolution of 2-byte NCHW tensors on the 16-bit matrix instruction (direct16.hpp) ----------------
 // Block shape for a layer: BC columns (even, at most 32: the one that wastes the fewest lanes on the image's width,
 // the widest among equals), BR = pixels per workgroup / BC rows, shrunk until the block's input rows fit a buffer
@@ -1074,6 +1094,16 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
     return tiles >= 2L * device_cus();
 }
+// Small fp32 layers go to the one-launch direct kernel while its cost -- rounds of the chip times groups of 32
+// channels -- stays small (measured against the fastest Winograd pipeline, NCHW: N = 1, C = K = 64, H = 56: 8.6
+// against 17.2 us; N = 2: 13.8 against 20.4; N = 1, C = K = 128, H = 28: 11.1 against 17.3; H = 56: 21.3 against
+// 23.4; N = 1, C = K = 256, H = 28: 19.8 against 23.5; N = 4, C = K = 64, H = 56: 26.2 against 27.1; beyond that the
+// Winograd pipelines win: N = 2, C = K = 256, H = 28: 37.6 against 27.0; N = 1, C = K = 512, H = 14: 36.5 against 25.9).
+bool auto_direct_few(int dtype, unsigned flags, const Geometry& g) {
+    if (!direct_few_ok(dtype, flags, g)) return false;
+    const long rounds = (direct_few_units(g) + device_cus() - 1) / device_cus();
+    return rounds * ((g.C + 31) / 32) <= 8;
+}
 // fp32 layers with a long reduction and enough 4x4 tiles run faster through the F(4x4,3x3) pipeline, product tensor
 // and all: 2.25 multiplies per output instead of 4, and a transformed input of 2.25x the tensor instead of 4x.
 // Measured at N = 32, NCHW, against the fastest F(2x2) pipeline: C = K = 256, H = 56: 0.37 against 0.54 ms;
@@ -1098,6 +1128,7 @@ int auto_f4_algo(int dtype, const Geometry& g4) {
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y, bool have_w) {
     if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x, y)) return WINO_ALGO_DIRECT;
+    if (have_w && auto_direct_few(dtype, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_f4(dtype, g)) {
         Geometry g4;
         make_geometry(dtype, g.N, g.C, g.K, g.H, g.W, g.pad, &g4, 4);
@@ -1179,6 +1210,10 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (direct_ok(dst, flags, g)) {
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
             return launch_direct(src, dst, dtype, flags, bias, g, x, w, y, (hipStream_t)stream);
+        }
+        if (direct_few_ok(dtype, flags, g)) {
+            StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
+            return launch_direct_few(src, dst, flags, bias, g, x, w, y, (hipStream_t)stream);
         }
         if (!direct16_ok(src, dst, dtype, flags, g))
             return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for pad 0 and 1: for C <= 4, and for 2-byte NCHW tensors with "
@@ -1798,9 +1833,10 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         make_geometry(dtype, N, L.C, L.K, L.H, L.W, 1, &g);
         hipError_t e = hipMalloc(&L.U, (size_t)16 * g.Cp * g.Kp * es);
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
-        // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte NCHW and NHWC layers)
+        // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte layers; small fp32 layers)
         const bool direct16_layer = dtype != WINO_F32 && (L.layout_in == WINO_CHWN) == (L.layout_out == WINO_CHWN) && L.C % 8 == 0;
-        if (e == hipSuccess && (L.C <= 4 || direct16_layer)) e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
+        if (e == hipSuccess && (L.C <= 4 || direct16_layer || auto_direct_few(dtype, L.flags, g)))
+            e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         // what AUTO runs outside the F(2x2) kernels gets its filters prepared once as well
         if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && auto_f4(dtype, g)) {
             Geometry g4;

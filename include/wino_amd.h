@@ -21,7 +21,8 @@
  * pad is 0 .. 1024 (the reference takes it arithmetically,
  * comparison/wrapedConv_NCHW.cuh:346-362, and its drivers pass 1).  The staged
  * and epilogue pipelines and WINO_ALGO_AUTO take any of these; WINO_ALGO_FUSED and
- * WINO_ALGO_DIRECT are built for 0 and 1 and answer WINO_ERR_UNSUPPORTED beyond.
+ * WINO_ALGO_DIRECT are built for 0 and 1 and answer WINO_ERR_UNSUPPORTED beyond
+ * (but for the small-layer fp32 kernel of WINO_ALGO_DIRECT, which takes any).
  *
  * Alignment: x, w, bias and y need only the alignment of their element type (any
  * view of a device allocation works).  The Winograd-domain operands U, V and the
@@ -69,7 +70,11 @@ typedef enum {
                                for fp32 layers with C, K >= 128 and at least 512 tiles when it is
                                given the filter bank itself; transformed filters handed to this algorithm by
                                name must come from wino_f4_filter_transform. */
-    WINO_ALGO_DIRECT = 5,    /* no Winograd at all, the convolution itself on the matrix cores.  Two kernels:
+    WINO_ALGO_DIRECT = 5,    /* no Winograd at all, the convolution itself on the matrix cores.  Three kinds of layer:
+                               small fp32 layers -- at most four rounds of the chip in units of 4 x 8 pixels x 32
+                               filters, e.g. the reference's sweep at batch 1 (comparison/layoutCompare.cu:38-46: N = 1,
+                               C = K = 64, 56 x 56) -- run as ONE launch whose waves share the channel reduction,
+                               any layout pair, any padding, bias and ReLU but no pooling;
                                layers with C <= 4 (the network's first layer, which the reference runs through
                                the same wrappers: comparison/layoutCompare.cu:38-46): the 9*C <= 36 products of an
                                output as one short MFMA reduction, any layout, fp32 or 2-byte;

@@ -62,7 +62,9 @@ def test_prepared_filters_match(oracle):
     x, w = synth.conv_inputs(N, C, K, H, W, seed=8)
     xd, wd = dev(x), dev(w)
     U = ops.filter_transform(wd)
-    assert torch.equal(ops.conv_prepared(xd, U, K), ops.conv(xd, wd))
+    # (with the filter bank itself AUTO may leave the Winograd kernels for so small a layer; with its transform it cannot)
+    assert torch.equal(ops.conv_prepared(xd, U, K), ops.conv(xd, wd, algo=ops.ALGO_STAGED))
+    assert oracle.rel_l2(host(ops.conv_prepared(xd, U, K)), host(ops.conv(xd, wd))) <= 1e-5
 
 
 def test_reference_call_surface(oracle):

@@ -1,7 +1,8 @@
-"""The direct path for layers with at most four input channels (WINO_ALGO_DIRECT; what AUTO picks for
-the network's first layer, comparison/layoutCompare.cu:38-46: 3 -> 64 channels).  Oracle: the CPU
-direct convolution.  Bit-exact on small integers for all nine layout pairs, with bias and ReLU; within the layer tolerance on floats; 2-byte tensors are
-multiplied in fp32 as well."""
+"""The direct path (WINO_ALGO_DIRECT) outside the 16-bit implicit GEMM: layers with at most four input channels
+(what AUTO picks for the network's first layer, comparison/layoutCompare.cu:38-46: 3 -> 64 channels; 2-byte tensors
+are multiplied in fp32 as well), and small fp32 layers of any channel count (the same sweep at batch 1).  Oracle: the
+CPU direct convolution.  Bit-exact on small integers for all nine layout pairs, with bias and ReLU; within the layer
+tolerance on floats."""
 import itertools
 
 import numpy as np
@@ -58,8 +59,8 @@ def test_what_the_path_is_not_built_for():
             ops.conv(x, w, algo=ops.ALGO_DIRECT, **kwargs)
         assert e.value.code == -2
         ops.conv(x, w, **kwargs)                     # AUTO falls back to the Winograd kernels
-    with pytest.raises(_lib.WinoError) as e:         # five channels
-        ops.conv(torch.zeros((1, 5, 8, 8), device="cuda"), torch.zeros((4, 5, 3, 3), device="cuda"), algo=ops.ALGO_DIRECT)
+    with pytest.raises(_lib.WinoError) as e:         # five channels and more output pixels than the small-layer kernel takes
+        ops.conv(torch.zeros((64, 5, 58, 58), device="cuda"), torch.zeros((64, 5, 3, 3), device="cuda"), algo=ops.ALGO_DIRECT)
     assert e.value.code == -2
     U = ops.filter_transform(w)
     with pytest.raises(_lib.WinoError) as e:         # transformed filters only
@@ -70,16 +71,57 @@ def test_what_the_path_is_not_built_for():
 
 @pytest.mark.parametrize("dtype", [ops.F32, ops.BF16])
 def test_direct_with_the_largest_filter_bank_that_fits_lds(oracle, dtype):
-    """K = 544 at C = 3: 17 filter tiles, 63 KB of LDS in fp32 (the path is offered up to 64 KB); K = 576 no
-    longer fits and AUTO goes back to the Winograd kernels.  Integers: bit-exact either way."""
+    """K = 544 at C = 3: 17 filter tiles, 63 KB of LDS in fp32 (the few-channel kernel is offered up to 64 KB); K = 576
+    no longer fits: a 2-byte layer goes back to the Winograd kernels, an fp32 one this small to the small-layer
+    kernel.  Integers: bit-exact either way."""
     from gpu_util import dev, host
     N, C, H, W = 1, 3, 9, 10
     for K, want_algo in ((544, ops.ALGO_DIRECT), (576, None)):
         x, w = synth.conv_inputs(N, C, K, H, W, seed=K, integer=True)
         got_algo = ops.pick_algo(ops.NCHW, dtype, N, C, K, H, W)
         if want_algo is None:
-            assert got_algo != ops.ALGO_DIRECT
+            assert (got_algo != ops.ALGO_DIRECT) == (dtype != ops.F32)
         else:
             assert got_algo == want_algo
         y = host(ops.conv(dev(x, dtype), dev(w, dtype), 1, ops.NCHW))
         assert np.array_equal(y, oracle.direct_conv(x, w, 1))
+
+
+FEW_SHAPES = [(1, 64, 64, 12, 16), (2, 7, 40, 6, 6), (1, 130, 70, 9, 11), (3, 36, 100, 13, 5), (1, 5, 33, 7, 20), (1, 8, 32, 3, 3)]
+
+
+@pytest.mark.parametrize("shape", FEW_SHAPES)
+def test_fp32_layers_with_few_pixels_bit_exact_on_integers(oracle, shape):
+    """direct_few_pixels_kernel: any number of channels in fp32 while the layer has few output pixels.  Channel counts
+    that are and are not multiples of 4 (16-byte and element-wise filter loads), of 32 (the waves' share of the
+    reduction), filter counts off the tile of 32, images off the 4 x 8 pixel tile, all nine layout pairs, pad 0 to 3."""
+    N, C, K, H, W = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    for pad in (1, 0, 2, 3):
+        if H + 2 * pad < 3 or W + 2 * pad < 3:
+            continue
+        for src, dst in itertools.product(SRC, DST):
+            xs, ws = synth.act_to_layout(x, src), synth.flt_to_layout(w, src)
+            want = synth.act_from_layout(oracle.direct_conv(xs, ws, pad, src, dst), dst) + bias[None, :, None, None]
+            want = synth.act_to_layout(np.ascontiguousarray(np.maximum(want, 0).astype(np.float32)), dst)
+            got = ops.conv(dev(xs), dev(ws), pad, src, dst, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias))
+            assert np.array_equal(host(got), want), (pad, src, dst)
+            plain = ops.conv(dev(xs), dev(ws), pad, src, dst, algo=ops.ALGO_DIRECT)
+            assert np.array_equal(host(plain), oracle.direct_conv(xs, ws, pad, src, dst)), (pad, src, dst)
+
+
+@pytest.mark.parametrize("layout", DST)
+def test_the_first_layer_of_the_references_sweep_at_batch_one(oracle, layout):
+    """N = 1, C = K = 64, 56 x 56 (comparison/layoutCompare.cu:38-46 at batch 1): AUTO runs it as one launch of the
+    small-layer kernel; floats within the fp32 tolerance of the oracle, and the Winograd pipeline agrees."""
+    N, C, K, H = 1, 64, 64, 56
+    x, w = synth.conv_inputs(N, C, K, H, H, seed=5, layout=layout)
+    want = oracle.direct_conv(x, w, 1, layout)
+    got = ops.conv(dev(x), dev(w), 1, layout, algo=ops.ALGO_DIRECT)
+    assert oracle.rel_l2(host(got), want) <= 1e-6
+    assert ops.pick_algo(layout, ops.F32, N, C, K, H, H) == ops.ALGO_DIRECT
+    assert torch.equal(ops.conv(dev(x), dev(w), 1, layout), got)
+    staged = ops.conv(dev(x), dev(w), 1, layout, algo=ops.ALGO_STAGED)
+    assert oracle.rel_l2(host(staged), host(got)) <= 1e-5

@@ -109,9 +109,11 @@ def test_paths_built_for_one_ring_of_padding_refuse(oracle):
         ops.conv(dev(x), dev(w), 2, algo=ops.ALGO_FUSED)
     got = host(ops.conv(dev(x), dev(w), 2))                                        # AUTO: a pipeline that can
     assert np.array_equal(got, oracle.direct_conv(x, w, 2))
-    x3, w3 = synth.conv_inputs(2, 3, 16, 20, 20, seed=6, integer=True)             # C <= 4: the direct kernel at pad 1
-    with pytest.raises(WinoError):
-        ops.conv(dev(x3), dev(w3), 2, algo=ops.ALGO_DIRECT)
+    x3, w3 = synth.conv_inputs(2, 3, 16, 20, 20, seed=6, integer=True)             # C <= 4: the direct kernel at pad 1;
+    with pytest.raises(WinoError):                                                 # 2-byte tensors: nothing direct at pad 2
+        ops.conv(dev(x3, ops.BF16), dev(w3, ops.BF16), 2, algo=ops.ALGO_DIRECT)
+    got = host(ops.conv(dev(x3), dev(w3), 2, algo=ops.ALGO_DIRECT))                # fp32: the small-layer kernel, any padding
+    assert np.array_equal(got, oracle.direct_conv(x3, w3, 2))
     assert np.array_equal(host(ops.conv(dev(x3), dev(w3), 2)), oracle.direct_conv(x3, w3, 2))
     with pytest.raises(WinoError):
         ops.conv(dev(x3), dev(w3), 1025)
