@@ -205,12 +205,71 @@ __global__ __launch_bounds__(256) void input_transform_f4_generic_kernel(const T
     for (int xi = 0; xi < 36; ++xi) vp[xi * plane] = from_f32<T>(v[xi]);
 }
 
+// ---- input transform, fp32, tiles in batch-minor order (CHWN sources) ------------------------------------------
+// Thread per (tile, channel vector): the four channels of the vector one after the other (36 loads in flight each
+// time), then 36 stores of 16 bytes.  With the batch fastest along the lanes a load instruction reads 256 contiguous
+// bytes of a pixel row of x and a store writes 1 KB of a coordinate plane -- a quarter of the memory instructions of
+// the thread-per-channel kernel above, which is what a CU runs out of first there (N = 32, C = 256, 56 x 56 from
+// CHWN: 72 against 85 us).  Byte offsets inside a channel plane of x and inside a coordinate plane of V are 32-bit
+// (the host checks).
+__global__ __launch_bounds__(256) void input_transform_f4_vec_kernel(const float* __restrict__ x, float* __restrict__ V,
+                                                                      ActStrides s, int N, int C, int H, int W, int pad,
+                                                                      int th, int tw, long P, long Pp, int Cp, int order,
+                                                                      FilterJob fj) {
+    if (gridDim.z == 2 && blockIdx.z == 0) {                 // dispatched first: the job runs under the input's workgroups
+        filter_job_f4<float>(fj);
+        return;
+    }
+    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int cq = blockIdx.y;
+    if (p >= P) return;
+    int n, ty, tx;
+    decode_tile(p, order, N, th, tw, n, ty, tx);
+    const int h0 = 4 * ty - pad, w0 = 4 * tx - pad;
+    unsigned roff[6], coff[6], rkeep[6], ckeep[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+        const int ih = h0 + i, iw = w0 + i;
+        rkeep[i] = (ih >= 0 && ih < H) ? 0xffffffffu : 0u;
+        ckeep[i] = (iw >= 0 && iw < W) ? 0xffffffffu : 0u;
+        roff[i] = (unsigned)((ih < 0 ? 0 : (ih >= H ? H - 1 : ih)) * s.h) * 4u;
+        coff[i] = (unsigned)((iw < 0 ? 0 : (iw >= W ? W - 1 : iw)) * s.w + n * s.n) * 4u;
+    }
+    float v[4][36];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int c = cq * 4 + e;
+        const unsigned chkeep = c < C ? 0xffffffffu : 0u;
+        const char* xp = reinterpret_cast<const char*>(x) + (size_t)(c < C ? c : C - 1) * s.c * sizeof(float);   // uniform
+        float raw[6][6], d[6][6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+#pragma unroll
+            for (int j = 0; j < 6; ++j) raw[i][j] = *reinterpret_cast<const float*>(xp + (roff[i] + coff[j]));
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+#pragma unroll
+            for (int j = 0; j < 6; ++j) d[i][j] = mask_keep(raw[i][j], rkeep[i] & ckeep[j] & chkeep);
+        input_tile_transform_f4(d, v[e]);
+    }
+    const size_t plane_bytes = (size_t)Cp * Pp * sizeof(float);
+    char* vb = reinterpret_cast<char*>(V) + (size_t)cq * Pp * 16;
+    const unsigned voff = (unsigned)p * 16u;
+#pragma unroll
+    for (int xi = 0; xi < 36; ++xi) {
+        *reinterpret_cast<float4*>(vb + voff) = make_float4(v[0][xi], v[1][xi], v[2][xi], v[3][xi]);
+        vb += plane_bytes;
+    }
+}
+
 // ---- input transform, fp32 NHWC source, batch-major tiles: a row of tiles staged in LDS ------------------------
 // In NHWC the channels of a pixel are contiguous and the pixels of a tile are not: a thread per (tile, channel)
 // gathers 4-byte pieces 4 pixels apart.  Here a workgroup takes one image, one tile row, a block of at most 14 tile
 // columns and 32 channels: the 6 x (4*tiles + 2) pixels it needs are loaded 16 bytes per lane, 8 lanes per pixel
-// (128 contiguous bytes; every load unconditional from a clamped address and masked afterwards, twelve of them in
-// flight per lane), and stored to LDS with a pixel pitch of 33 words.  Then one thread per (channel of a vector,
+// (128 contiguous bytes; every load unconditional from a clamped address and masked afterwards -- all twelve issued
+// before the first mask, under a branch that is uniform for the workgroup: with the loads inside a per-lane branch
+// the compiler waits for each one before it issues the next, 91 against 73 us on N = 32, C = 256, 56 x 56), and
+// stored to LDS with a pixel pitch of 33 words.  Then one thread per (channel of a vector,
 // tile, channel vector), channel fastest as in the layout-generic kernel: its 36 LDS reads hit distinct banks across
 // the wave (bank = 4*tile + channel + const), and the 4 lanes of a vector and the 16 tiles of a wave write 256
 // contiguous bytes of each coordinate plane of V.
@@ -247,23 +306,41 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
     // ---- pixels -> LDS
     const int npix = 6 * wlb;                                // <= 348: twelve passes of 32 pixels at most
     const int ch4 = tid & 7, pl = tid >> 3;                  // 16-byte piece of the 32 channels; pixel of a pass
+    const unsigned inv_wlb = (65536u + (unsigned)wlb - 1u) / (unsigned)wlb;      // pix / wlb = pix * inv_wlb >> 16 for pix < 348
+    const char* const xn = reinterpret_cast<const char*>(x) + (size_t)n * H * W * C * sizeof(float);   // the image (uniform)
+    const int c = c0 + 4 * ch4;
+    const bool vec = (C & 3) == 0 && c0 + F4N_CC <= C;         // uniform: every lane of the workgroup loads 16 bytes
     float4 raw[12];
+    unsigned keep[12];
+    if (vec) {
+        // (all loads first, unconditionally, from clamped addresses; the masks afterwards: the loads are in flight together)
 #pragma unroll
-    for (int q = 0; q < 12; ++q) {
-        const int pix = min(pl + 32 * q, npix - 1);
-        const int r = pix / wlb, col = pix - r * wlb;
-        const int ih = h0 + r, iw = w0 + col, c = c0 + 4 * ch4;
-        const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
-        const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - 1);
-        const unsigned keep = ok ? 0xFFFFFFFFu : 0u;
-        const float* src = x + (((size_t)n * H + ihc) * W + iwc) * C;
-        if ((C & 3) == 0 && c + 3 < C) {                     // wave-uniform unless C is not a multiple of 32
-            const float4 v = *reinterpret_cast<const float4*>(src + c);
-            raw[q] = make_float4(mask_keep(v.x, keep), mask_keep(v.y, keep), mask_keep(v.z, keep), mask_keep(v.w, keep));
-        } else {
+        for (int q = 0; q < 12; ++q) {
+            const int pix = min(pl + 32 * q, npix - 1);
+            const int r = (int)(((unsigned)pix * inv_wlb) >> 16), col = pix - r * wlb;
+            const int ih = h0 + r, iw = w0 + col;
+            const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
+            const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - 1);
+            keep[q] = ok ? 0xFFFFFFFFu : 0u;
+            const unsigned off = (unsigned)((ihc * W + iwc) * C + c) * 4u;       // byte offset in the image (< 2^32: the host checks)
+            raw[q] = *reinterpret_cast<const float4*>(xn + off);
+        }
+#pragma unroll
+        for (int q = 0; q < 12; ++q)
+            raw[q] = make_float4(mask_keep(raw[q].x, keep[q]), mask_keep(raw[q].y, keep[q]), mask_keep(raw[q].z, keep[q]), mask_keep(raw[q].w, keep[q]));
+    } else {
+#pragma unroll
+        for (int q = 0; q < 12; ++q) {
+            const int pix = min(pl + 32 * q, npix - 1);
+            const int r = (int)(((unsigned)pix * inv_wlb) >> 16), col = pix - r * wlb;
+            const int ih = h0 + r, iw = w0 + col;
+            const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
+            const int ihc = min(max(ih, 0), H - 1), iwc = min(max(iw, 0), W - 1);
+            const unsigned kp = ok ? 0xFFFFFFFFu : 0u;
+            const unsigned off = (unsigned)((ihc * W + iwc) * C) * 4u;
             float e[4];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) e[k] = mask_keep(src[min(c + k, C - 1)], c + k < C ? keep : 0u);
+            for (int k = 0; k < 4; ++k) e[k] = mask_keep(*reinterpret_cast<const float*>(xn + (off + (unsigned)min(c + k, C - 1) * 4u)), c + k < C ? kp : 0u);
             raw[q] = make_float4(e[0], e[1], e[2], e[3]);
         }
     }
@@ -277,21 +354,31 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
     }
     __syncthreads();
     // ---- tiles
-    const size_t vplane = (size_t)Cp * Pp;
+    const size_t vplane_bytes = (size_t)Cp * Pp * sizeof(float);
     const int nvec = min(F4N_CC, Cp - c0) / 4;               // channel vectors of this workgroup (Cp is a multiple of 16)
     const long p0 = ((long)n * th + ty) * tw + tx0;
+    const unsigned inv_ntx = (65536u + (unsigned)ntx - 1u) / (unsigned)ntx;
+    // a thread's 36 stores: a uniform plane base that moves on by a plane, and one 32-bit offset (a plane is < 2^32 bytes)
+    char* const vbase = reinterpret_cast<char*>(V) + ((size_t)(c0 / 4) * Pp + p0) * 16;
     for (int idx = tid; idx < nvec * ntx * 4; idx += 256) {
-        const int e = idx & 3, t = (idx >> 2) % ntx, ql = (idx >> 2) / ntx;
+        const int e = idx & 3, it = idx >> 2;
+        const int ql = (int)(((unsigned)it * inv_ntx) >> 16), t = it - ql * ntx;
         const float* src = sm + (4 * t) * F4N_PITCH + 4 * ql + e;
         float d[6][6], v[36];
 #pragma unroll
-        for (int i = 0; i < 6; ++i)
+        for (int i = 0; i < 6; ++i) {
+            const float* row = src + i * wlb * F4N_PITCH;
 #pragma unroll
-            for (int j = 0; j < 6; ++j) d[i][j] = src[(i * wlb + j) * F4N_PITCH];
+            for (int j = 0; j < 6; ++j) d[i][j] = row[j * F4N_PITCH];
+        }
         input_tile_transform_f4(d, v);
-        float* vp = V + ((size_t)(c0 / 4 + ql) * Pp + p0 + t) * 4 + e;
+        const unsigned voff = (unsigned)(((size_t)ql * Pp + t) * 16 + e * 4);
+        char* vb = vbase;
 #pragma unroll
-        for (int xi = 0; xi < 36; ++xi) vp[xi * vplane] = v[xi];
+        for (int xi = 0; xi < 36; ++xi) {
+            *reinterpret_cast<float*>(vb + voff) = v[xi];
+            vb += vplane_bytes;
+        }
     }
 }
 

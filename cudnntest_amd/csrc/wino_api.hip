@@ -588,7 +588,8 @@ int launch_f4_input(int layout, int order, const Geometry& g, const void* x, voi
                     const FilterJob& fj = FilterJob{}) {
     constexpr int CV = ChanVec<T>::n;
     const long job = fj.w ? (long)fj.Kp * (fj.Cp / CV) : 0;
-    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && sizeof(T) == 4 && g.N < 65535 && g.Cp / F4N_CC < 65535) {
+    if (layout == WINO_NHWC && order == WINO_TILES_BATCH_MAJOR && sizeof(T) == 4 && g.N < 65535 && g.Cp / F4N_CC < 65535 &&
+        (long)g.H * g.W * g.C * 4 < (1L << 32) && (long)g.Cp * g.Pp * 4 < (1L << 32)) {   // (32-bit byte offsets inside an image and a plane of V)
         const int colBlocks = (g.tw + F4N_TCB - 1) / F4N_TCB;
         dim3 grid((unsigned)(g.th * colBlocks), (g.Cp + F4N_CC - 1) / F4N_CC, g.N);
         const bool ride = job > 0 && (long)grid.x * grid.y * 256 >= job;
@@ -638,6 +639,24 @@ int launch_f4_input(int layout, int order, const Geometry& g, const void* x, voi
                 LAUNCH_CHECK("f4_input_transform_nchw_small");
                 return WINO_OK;
             }
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        // batch-minor tiles of a CHWN source: a thread per (tile, channel vector)
+        if (layout == WINO_CHWN && order == WINO_TILES_BATCH_MINOR && g.P < (1L << 28) && (long)g.N * g.H * g.W * 4 < (1L << 32) &&
+            (long)g.Cp * g.Pp * 4 < (1L << 32)) {
+            dim3 grid((unsigned)((g.P + 255) / 256), g.Cp / CV), block(256);
+            const bool ride = job > 0 && (long)grid.x * grid.y * 256 >= job;
+            if (job > 0 && !ride) {
+                const int rc = launch_f4_filter<T>(layout, fj.K, fj.C, fj.Kp, fj.Cp, fj.w, fj.U, st);
+                if (rc) return rc;
+            }
+            if (ride) grid.z = 2;
+            hipLaunchKernelGGL(input_transform_f4_vec_kernel, grid, block, 0, st, (const float*)x, (float*)V,
+                               act_strides(layout, g.N, g.C, g.H, g.W), g.N, g.C, g.H, g.W, g.pad, g.th, g.tw, g.P, g.Pp, g.Cp, order,
+                               ride ? fj : FilterJob{});
+            LAUNCH_CHECK("f4_input_transform_vec");
+            return WINO_OK;
         }
     }
     dim3 grid((unsigned)((g.P * CV + 255) / 256), g.Cp / CV), block(256);
