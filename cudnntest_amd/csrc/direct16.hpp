@@ -47,6 +47,7 @@ struct D16Geom {
     int PP;                // column pairs loaded per row
     int colBlocks, rowBlocks, kTiles;
     int maxcross;          // image boundaries a block can span
+    int a4, b3;            // (8-wave kernel) b3 > 0: every image is a4 blocks whose waves own 4 rows and b3 blocks whose waves own 3
     int CQ, Kp;            // channel vectors (a multiple of 4) and padded filters of the packed bank
     long G;                // N * Ho output rows
 };

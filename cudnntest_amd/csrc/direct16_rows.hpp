@@ -54,9 +54,7 @@ static_assert(D16R<1, true>::LDS <= 160 * 1024 && D16R<2, true>::LDS <= 160 * 10
 // contiguous bytes of a pixel of y.  The two are independent: a layer may read one layout and write the other.
 template <typename T, int WF, bool XN = false, bool YN = XN, bool DIL = false>
 __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restrict__ x, const T* __restrict__ W9,
-                                                               T* __restrict__ y, D16Geom g, Epilogue ep,
-                                                               float* __restrict__ part, int* __restrict__ cnt,
-                                                               int spin_limit) {
+                                                               T* __restrict__ y, D16Geom g, Epilogue ep) {
     typedef typename Mma<T>::vec vec;
     typedef D16R<WF, DIL> P;
     static_assert(!DIL || (!XN && !YN), "CHWN tensors on both sides");
@@ -73,58 +71,36 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     const int HW = g.H * g.W, Hp = g.Ho + 2;
     const int nst = g.CQ / 2;                                // stages of 16 channels per tile
 
-    // ---- this workgroup's tiles: sequence items s = s0, s0 + sstep, ... of its XCD, in ROUNDS ------------------------
-    // A layer has one to four tiles per CU, so a last round of whole tiles leaves a good part of the chip idle.  The
-    // items left over after the full rounds are therefore not dealt out whole: the sequence of their STAGES is cut into
-    // sstep equal runs, one per workgroup.  A run begins and ends in the middle of tiles; the sums over a part of a
-    // tile's channels are partial sums of its outputs.  The workgroup that holds a tile's LAST stage owns it: the
-    // others leave their accumulators in scratch (then an arrival counter) and the owner adds them to its own, in
-    // workgroup order, before it stores the tile.  Order inside a run: first the beginning of the
-    // tile that the next workgroup continues, then whole tiles, last the end of the tile that previous workgroups
-    // began: a workgroup only waits for lower workgroup ids of its own XCD, for something they do before they wait
-    // themselves; the wait is bounded all the same.  Without scratch (part == nullptr), or with less than four stages
-    // to a run, the left-over items are dealt out whole.
+    // ---- this workgroup's tiles: sequence items s = s0, s0 + sstep, ... < send of its XCD ------------------
     const int xcd = blockIdx.x & 7;
     const int sstep = gridDim.x >> 3;
     const int npb = g.colBlocks * g.rowBlocks;               // pixel blocks; block pbx*8 + xcd belongs to this XCD
     const int send = ((npb - xcd + 7) >> 3) * g.kTiles;
     const int s0 = (int)(blockIdx.x >> 3);
-    const int rounds = send / sstep, tail0 = rounds * sstep, ntail = send - tail0;
-    const int Tx = ntail * nst;                              // stages of the left-over items
-    const bool shared = part != nullptr && Tx >= 4 * sstep;
-    const int ra = shared ? (int)((long)s0 * Tx / sstep) : (s0 < ntail ? s0 * nst : 0);
-    const int rb = shared ? (int)((long)(s0 + 1) * Tx / sstep) : (s0 < ntail ? (s0 + 1) * nst : 0);
-    if (rounds == 0 && ra >= rb) return;
-    // the run [ra, rb) as up to three pieces (item, first stage, end stage), in the order they are computed:
-    // 0: the beginning of the tile that goes on past rb; 1: whole tiles (consecutive items); 2: the end of the tile
-    // begun before ra
-    const int hstart = rb / nst * nst;
-    const int at0 = rb == hstart ? rb : (hstart <= ra ? ra : hstart), len0 = rb - at0;
-    const int low_end = rb - len0;
-    const int at1 = min((ra + nst - 1) / nst * nst, low_end), len1 = low_end - at1;
-    const int len2 = at1 - ra;
-    // (item, first stage, stages, piece) of the pieces that are not empty, in order, in a small table in LDS: the
-    // cursors below fetch a piece with one read instead of carrying twelve more scalars through the stage loop
-    __shared__ int4 pc_tab[4];
-    if (tid == 0) {
-        int n = 0;
-        if (len0 > 0) pc_tab[n++] = make_int4(tail0 + at0 / nst, at0 % nst, len0, 0);
-        if (len1 > 0) pc_tab[n++] = make_int4(tail0 + at1 / nst, 0, len1, 1);
-        if (len2 > 0) pc_tab[n++] = make_int4(tail0 + ra / nst, ra % nst, len2, 2);
-        for (; n < 4; ++n) pc_tab[n] = make_int4(0, 0, 0, 3);
-    }
-    __syncthreads();
-    const int slot_me = xcd * sstep + s0;
+    if (s0 >= send) return;
     struct Tile {
-        int k0, c0, n0, oh0;
+        int k0, c0, n0, oh0, R;                              // R: output rows per wave, 4 or 3
     };
-    auto decode = [&](int s) __attribute__((always_inline)) {
+    // Row blocks: runs of BR = 4 S rows (S waves stacked) over the N * Ho rows of the batch; or, with g.b3 > 0, every
+    // image cut into g.a4 blocks whose waves own 4 rows and g.b3 blocks whose waves own 3 (Ho = S (4 a4 + 3 b3)), all
+    // the 4-row blocks first in the sequence: the host mixes the two so that the layer's tiles fill their rounds of the
+    // chip evenly (a 3-row tile is the same stage loop less the multiplies of the fourth row).
+    auto decode = [&](int s) {
         const int pbx = s / g.kTiles, kt = s - pbx * g.kTiles;
         const int pb = pbx * 8 + xcd;
         const int rb = pb / g.colBlocks, cb = pb - rb * g.colBlocks;
+        if (g.b3 > 0) {
+            const int n4 = g.N * g.a4;
+            if (rb < n4) {
+                const int n0 = rb / g.a4;
+                return Tile{kt * P::KT, cb * g.BC, n0, (rb - n0 * g.a4) * g.BR, 4};
+            }
+            const int q = rb - n4, n0 = q / g.b3;
+            return Tile{kt * P::KT, cb * g.BC, n0, g.a4 * g.BR + (q - n0 * g.b3) * (g.BR / 4 * 3), 3};
+        }
         const long g0 = (long)rb * g.BR;
         const int n0 = (int)(g0 / g.Ho);
-        return Tile{kt * P::KT, cb * g.BC, n0, (int)(g0 - (long)n0 * g.Ho)};
+        return Tile{kt * P::KT, cb * g.BC, n0, (int)(g0 - (long)n0 * g.Ho), 4};
     };
 
     // ---- input tasks of this thread: (channel vector v, LDS row, column pair); what does not depend on the tile ----
@@ -155,48 +131,23 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     }
 
     // ---- request cursors: the stage whose input is requested next, and the stage whose filters are ----------------
-    // ph: 0 .. rounds-1 the full rounds, then rounds + index into pc_tab; left: stages left of the run's current part
-    // (a round's tile, a piece); s, cs: item and stage; kind: 0 / 1 / 2 for the three pieces, 1 for a round's tile,
-    // 3 past the end; open: the stage opens a tile or a part of one
     struct Cursor {
-        int s, cs, left, ph, kind;
-        bool open;
+        int s, cs;
+        bool valid;
     };
-    auto enter = [&](Cursor& c) __attribute__((always_inline)) {          // phase c.ph begins
-        c.open = true;
-        if (c.ph < rounds) {
-            c.s = s0 + c.ph * sstep;
+    auto advance = [&](Cursor& c) {
+        if (++c.cs == nst) {
             c.cs = 0;
-            c.left = nst;
-            c.kind = 1;
-            return;
-        }
-        const int4 e = pc_tab[min(c.ph - rounds, 3)];
-        c.s = __builtin_amdgcn_readfirstlane(e.x);
-        c.cs = __builtin_amdgcn_readfirstlane(e.y);
-        c.left = __builtin_amdgcn_readfirstlane(e.z);
-        c.kind = __builtin_amdgcn_readfirstlane(e.w);
-    };
-    auto advance = [&](Cursor& c) __attribute__((always_inline)) {
-        c.open = false;
-        if (--c.left == 0) {
-            ++c.ph;
-            enter(c);
-        } else if (++c.cs == nst) {                          // (whole tiles of the run: the next item)
-            c.cs = 0;
-            ++c.s;
-            c.open = true;
+            c.s += sstep;
+            c.valid = c.s < send;
         }
     };
-    Cursor cx{0, 0, 0, 0, 1, true}, cf{0, 0, 0, 0, 1, true}, cc{0, 0, 0, 0, 1, true};
-    enter(cx);
-    enter(cf);
-    enter(cc);
+    Cursor cx{s0, 0, true}, cf{s0, 0, true};
     unsigned xoff[NTASK];                                    // byte offset from (image n0, the stage's first channel), a multiple
                                                              // of 4 | bit 0: the pair lies inside the image
     const char* xs = nullptr;                                // image n0, first channel of the stage to request
     const unsigned hw2 = (unsigned)(HW * 2);
-    auto prep_x = [&](const Tile& t) __attribute__((always_inline)) {
+    auto prep_x = [&](const Tile& t) {
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
             const int sl = min((tid + 512 * q) >> 1, g.LR * g.PW - 1);           // NHWC source: the task's pixel slot
@@ -234,11 +185,11 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     }
     const char* const w9b = reinterpret_cast<const char*>(W9);
     const unsigned fstep = (unsigned)(2 * g.Kp * 16);
-    auto f_request = [&](const Cursor& c, int slot) __attribute__((always_inline)) {        // the filter rows of stage c into ring slot `slot`
+    auto f_request = [&](const Cursor& c, int slot) {        // the filter rows of stage c into ring slot `slot`
         const int pbx = c.s / g.kTiles, kt = c.s - pbx * g.kTiles;
         const uint64_t base = reinterpret_cast<uint64_t>(w9b) + (uint64_t)kt * P::KT * 16 + (uint64_t)c.cs * fstep;
 #pragma unroll
-        for (int q = 0; q < P::NF; ++q) dma_row(uniform64(base + frow_src[q]), lane_off, d16r_smem + slot * P::FB + frow_dst[q]);
+        for (int q = 0; q < P::NF; ++q) dma_row(base + frow_src[q], lane_off, d16r_smem + slot * P::FB + frow_dst[q]);
     };
     uint32_t raw[XN ? 1 : NTASK][8];
     uint4 rawn[XN ? NTASK : 1];                            // NHWC source: the 8 channels of a task's pixel
@@ -246,7 +197,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     int req_cs = 0;                                          // the stage (inside its tile) whose input was requested last
     // piece 8q + e of a stage's input requests: channel e of task q.  A stage's second channel vector may lie past
     // C: the first one is loaded instead, and masked when it is written
-    auto x_piece = [&](int idx) __attribute__((always_inline)) {
+    auto x_piece = [&](int idx) {
         if (idx == 0) req_cs = cx.cs;
         if constexpr (XN) {
             const int v = tid & 1;
@@ -263,7 +214,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         raw[XN ? 0 : q][e] = *reinterpret_cast<const uint32_t*>(xs + poff[q]);
         poff[q] += hw2;
     };
-    auto x_commit = [&](int xslot) __attribute__((always_inline)) {                         // the stage requested through x_piece into input slot xslot
+    auto x_commit = [&](int xslot) {                         // the stage requested through x_piece into input slot xslot
 #pragma unroll
         for (int q = 0; q < NTASK; ++q) {
             if ((ldsw[q] & 3) == 0) continue;
@@ -292,16 +243,18 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     int yoff[4];                                             // element offset of (n, k0, oh, ow) in y per row of the wave, < 0: no pixel
     int k0c = 0;                                             // first filter of this wave
     int pc0 = 0;                                             // NHWC: first output column of this wave
-    auto prep_pix = [&](const Tile& t) __attribute__((always_inline)) {
+    bool r4 = true;                                          // the waves of the tile own 4 rows (else 3: row 3 of a wave is not computed, not stored)
+    auto prep_pix = [&](const Tile& t) {
         k0c = t.k0 + wf * 64;
+        r4 = t.R == 4;
         const long g0 = (long)t.n0 * g.Ho + t.oh0;
         const int col = 32 * wc + l32;
         const bool colok = t.c0 + col < g.Wo;
-        const int ohp = t.oh0 + 4 * wr;                      // the wave's four rows lie in one image: Ho is a multiple of 4
+        const int ohp = t.oh0 + t.R * wr;                    // the wave's rows lie in one image: Ho is a multiple of 4 (of a block's rows, with 3-row blocks mixed in)
         int dn = 0;
         for (int k = 1; k <= g.maxcross; ++k) dn += ohp >= k * g.Ho ? 1 : 0;
         const int oh = ohp - dn * g.Ho;
-        const bool rowok = g0 + 4 * wr < g.G;
+        const bool rowok = g0 + t.R * wr < g.G;
         const int L = rowok ? dn * Hp + oh - t.oh0 : 0;
         xw_off = ((lh * P::XPLANE) + L * g.PW + (colok ? col : 0)) * 16;
         if constexpr (YN) {
@@ -336,24 +289,24 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     // multiplies.  The order is pinned: the pixel fragment of step t+2 and the filter fragments that the following
     // steps need are requested before the multiplies of step t, filter row r of the next column as soon as its last
     // use has issued.  service() -- everything else this wave does in a stage -- runs before step 0, 5, 9 or 14.
-    auto compute = [&](int fslot, int xslot, int site, auto&& service) __attribute__((always_inline)) {
+    auto compute = [&](int fslot, int xslot, int site, auto&& service) {
         const unsigned char* fs = d16r_smem + fslot * P::FB + (lh * P::KT + wf * 64 + l32) * 16;
         const unsigned char* xrow[6];                        // the wave's six input rows, this lane's column
 #pragma unroll
         for (int r = 0; r < 6; ++r) xrow[r] = xsm + xslot * P::XB + xw_off + r * g.PW * 16;
         vec a[3][2], b[3];
-        auto lda = [&](int r, int s) __attribute__((always_inline)) {
+        auto lda = [&](int r, int s) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) a[r][i] = *reinterpret_cast<const vec*>(fs + (3 * r + s) * (2 * P::KT * 16) + i * 512);
         };
         const int dsb = g.ds * 16;                           // bytes between the tap columns of a fragment
-        auto ldb = [&](int t) __attribute__((always_inline)) { b[t % 3] = *reinterpret_cast<const vec*>(xrow[t % 6] + (DIL ? (t / 6) * dsb : (t / 6) * 16)); };
+        auto ldb = [&](int t) { b[t % 3] = *reinterpret_cast<const vec*>(xrow[t % 6] + (DIL ? (t / 6) * dsb : (t / 6) * 16)); };
         lda(0, 0);
         ldb(0);
         lda(1, 0);
         ldb(1);
         lda(2, 0);
-        auto step = [&](int t) __attribute__((always_inline)) {
+        auto step = [&](int t) {
             const int s = t / 6, rho = t % 6;
             if (t + 2 < 18) ldb(t + 2);
             if (rho == 4 && s < 2) lda(0, s + 1);
@@ -364,6 +317,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             for (int j = 0; j < 4; ++j) {
                 const int r = rho - j;
                 if (r < 0 || r > 2) continue;
+                if (j == 3 && !r4) continue;                 // (uniform)
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
                     if constexpr (YN) Mma<T>::run(b[t % 3], a[r][i], acc[i][j]);
@@ -392,11 +346,11 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     // a wave exist together, so a lane stores all its values or none.
     const unsigned kstride2 = (ep.pool ? (unsigned)((g.Ho >> 1) * (g.Wo >> 1)) : (unsigned)(g.Ho * g.Wo)) * 2u;   // bytes between the planes of two filters
     const bool odd = lane & 1;
-    auto stores = [&]() __attribute__((always_inline)) {
+    auto stores = [&]() {
         if (k0c >= g.K || yoff[0] < 0) return;
         // (opaque to the optimiser: called from inside the stage loop, the 64 store addresses of a tile would be
         // loop invariants, computed ahead of the loop and kept in registers)
-        unsigned ks = __builtin_amdgcn_readfirstlane(kstride2);
+        unsigned ks = kstride2;
         asm volatile("" : "+s"(ks));
         char* const yb = reinterpret_cast<char*>(y);
         if constexpr (YN) {
@@ -404,7 +358,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             // k0c + 32*i + l32.  Two neighbouring lanes hold neighbouring filters and exchange values, so that each
             // stores one 4-byte pair of filters -- the even lane for the pixel of register r, the odd lane for that of
             // register r+1: per instruction the 16 even (odd) lanes of a half write 64 contiguous bytes of one pixel.
-            unsigned kp = __builtin_amdgcn_readfirstlane((unsigned)g.K * 2u);                // bytes between two pixels of y
+            unsigned kp = (unsigned)g.K * 2u;                // bytes between two pixels of y
             asm volatile("" : "+s"(kp));
             // (the two filter halves of a pixel, 64 + 64 bytes of one 128-byte line, are stored one right after the other)
             float bk[2] = {0.f, 0.f};
@@ -443,6 +397,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                 const bool pok = pc0 + 8 * (r2 >> 2) + 4 * lh + (r2 & 3) < g.Wo;    // (Wo is even: the pair's pixels exist together)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
+                    if (j == 3 && !r4) continue;             // (uniform: a 3-row tile)
 #pragma unroll
                     for (int i = 0; i < 2; ++i) {
                         float v0 = acc[i][j][r2] + bk[i], v1 = acc[i][j][r2 + 1] + bk[i];
@@ -503,6 +458,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
+                    if (j == 3 && !r4) continue;             // (uniform: a 3-row tile)
                     float v0 = acc[i][j][r2] + b0, v1 = acc[i][j][r2 + 1] + b1;
                     if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
                     const float got = swap_lane_pairs(odd ? v0 : v1);
@@ -517,13 +473,13 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
 
     // the filters of the stage after the next, into the ring slot that was read last in the previous stage (a ring of
     // two: the next stage's, into the other slot)
-    auto f_next = [&](int fslot) __attribute__((always_inline)) {
-        if (!(cf.kind < 3)) return false;
+    auto f_next = [&](int fslot) {
+        if (!cf.valid) return false;
         f_request(cf, P::NFR == 2 ? fslot ^ 1 : (fslot == 0 ? 2 : fslot - 1));
         advance(cf);
         return true;
     };
-    auto zero_acc = [&]() __attribute__((always_inline)) {
+    auto zero_acc = [&]() {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -533,14 +489,14 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     };
     // wait until at most `newest` of this wave's memory requests are outstanding (loads return in order, so those
     // are the ones issued last), and for its LDS writes; then the workgroup's barrier
-    auto wait_only = [&](int newest) __attribute__((always_inline)) {
+    auto wait_only = [&](int newest) {
         if (newest == 0) __builtin_amdgcn_s_waitcnt(0x0070);
         else if (newest == P::NF) __builtin_amdgcn_s_waitcnt(0x0070 | P::NF);
         else if (newest == NX) __builtin_amdgcn_s_waitcnt(0x0070 | (NX & 0xF) | ((NX >> 4) << 14));
         else __builtin_amdgcn_s_waitcnt(0x0070 | ((NX + P::NF) & 0xF) | (((NX + P::NF) >> 4) << 14));
         asm volatile("" ::: "memory");
     };
-    auto wait_barrier = [&](int newest) __attribute__((always_inline)) {
+    auto wait_barrier = [&](int newest) {
         wait_only(newest);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -559,106 +515,38 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     const int site = (wave >> 2) == 0 ? 2 + (wave & 1) : (wave & 1);
     f_request(cf, 0);
     advance(cf);
-    if (P::NFR > 2 && (cf.kind < 3)) {
+    if (P::NFR > 2 && cf.valid) {
         f_request(cf, 1);
         advance(cf);
     }
     bool pending = false;                                    // a requested stage waits in registers
-    auto x_request = [&]() __attribute__((always_inline)) {
-        if (cx.open) {                                       // the stage opens a tile (or a part of one, at stage cx.cs)
+    bool need_prep = true;                                   // the stage to request next opens a tile
+    auto x_request = [&]() {
+        if (need_prep) {
             prep_x(decode(cx.s));
-            xs += (size_t)cx.cs * (XN ? (size_t)32 : (size_t)16 * HW * 2);
+            need_prep = false;
         }
 #pragma unroll
         for (int i = 0; i < NX; ++i) x_piece(i);
         pending = true;
         xs += XN ? (size_t)32 : (size_t)16 * HW * 2;                           // the next 16 channels
         advance(cx);
+        need_prep = cx.cs == 0;
     };
     x_request();
     x_commit(0);
     pending = false;
-    if ((cx.kind < 3)) x_request();
+    if (cx.valid) x_request();
     wait_barrier(pending ? NX : 0);
 
-    // A block of partial sums is [32 register quads][512 threads] of 16 bytes; a thread walks its column with a running
-    // pointer (pitch opaque: 32 addresses computed from constants would be loop invariants of the stage loop, kept
-    // in registers across it).  The data travel as plain stores and loads: writer and reader run on the same XCD (its
-    // L2 is where both meet: stores write through the CU's L1, and the reader's CU -- one persistent workgroup per CU
-    // -- has never touched these lines since its L1 was invalidated at the kernel's start); only the arrival counter
-    // is an atomic, incremented after the writer's stores have been acknowledged (vmcnt) and its waves have met.
-    // this workgroup's accumulators to its block of scratch
-    auto park = [&]() __attribute__((always_inline)) {
-        floatx4* p = reinterpret_cast<floatx4*>(part + (size_t)slot_me * (128 * 512)) + tid;
-        unsigned pitch = 512;
-        asm volatile("" : "+s"(pitch));
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-#pragma unroll
-                for (int q = 0; q < 16; q += 4) {
-                    *p = floatx4{acc[i][j][q], acc[i][j][q + 1], acc[i][j][q + 2], acc[i][j][q + 3]};
-                    p += pitch;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): this wave's values have reached the L2
-    };
-    // the first stages of a tile that the next workgroup continues are done: the owner's counter, once every wave's
-    // values are in the L2
-    auto hand_over = [&]() __attribute__((always_inline)) {
-        __syncthreads();
-        if (tid == 0) {
-            const int pend = (rb / nst + 1) * nst;           // the tile ends here; its owner holds stage pend - 1
-            const int owner = (int)(((long)pend * sstep - 1) / Tx);
-            __hip_atomic_fetch_add(&cnt[xcd * sstep + owner], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    };
-    // the last stages of a tile that previous workgroups began are done: their partial sums are added, in workgroup
-    // order.  The parts of a tile are computed side by side; the owner needs the others' sums only now, at the end of
-    // its part -- which is the end of its run, so this is done behind the stage loop, where nothing of the loop's
-    // pipeline (input on its way, fragments, cursors) competes for registers.
-    auto gather = [&]() __attribute__((always_inline)) {
-        const int pbeg = ra / nst * nst;                     // the tile begins here, in workgroup `first`
-        const int first = (int)(((long)(pbeg + 1) * sstep - 1) / Tx);
-        if (tid == 0) {
-            int spins = 0;
-            while (__hip_atomic_load(&cnt[slot_me], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < s0 - first && spins < spin_limit) {
-                __builtin_amdgcn_s_sleep(32);
-                ++spins;
-            }
-            __hip_atomic_store(&cnt[slot_me], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     // zero for the next launch
-        }
-        __syncthreads();
-        unsigned pitch = 512;
-        asm volatile("" : "+s"(pitch));
-#pragma unroll 1
-        for (int c = first; c < s0; ++c) {
-            const floatx4* p = reinterpret_cast<const floatx4*>(part + (size_t)(xcd * sstep + c) * (128 * 512)) + tid;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                floatx4 v[16];                               // half a block in flight at a time
-#pragma unroll
-                for (int t = 0; t < 16; ++t) {
-                    v[t] = __builtin_nontemporal_load(p);
-                    p += pitch;
-                }
-#pragma unroll
-                for (int t = 0; t < 16; ++t)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][t >> 2][4 * (t & 3) + e] += v[t][e];
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-
     int fslot = 0, xslot = 0;
-    const int total = rounds * nst + (rb - ra);
+    const int ntiles = (send - s0 + sstep - 1) / sstep;
+    int s = s0, cs = 0;
+    const int total = ntiles * nst;
 #pragma unroll 1
     for (int it = 0; it < total; ++it) {
-        if (cc.open) {
-            prep_pix(decode(cc.s));
+        if (cs == 0) {
+            prep_pix(decode(s));
             zero_acc();
         }
         bool xreq = false, freq = false;
@@ -670,21 +558,16 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             // (a filter ring of two: the filters requested now are read in the next stage, so they go first and
             // only the input requests may still be on their way at the stage's end)
             if (P::NFR == 2) f_next(fslot);
-            if ((cx.kind < 3)) {
+            if (cx.valid) {
                 x_request();
                 xreq = true;
             }
             if (P::NFR > 2) freq = f_next(fslot);
         });
         const int newest = (xreq ? NX : 0) + (freq ? P::NF : 0);
-        if (cc.left == 1 || cc.cs == nst - 1) {              // the tile, or this workgroup's part of it, is complete
+        if (cs == nst - 1) {
             wait_only(newest);                               // before the stores: they would count as the newest requests
-            if (cc.kind == 0) {
-                park();
-                hand_over();
-            } else if (cc.kind != 2) {
-                stores();
-            }
+            stores();
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         } else {
@@ -692,11 +575,10 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         }
         fslot = fslot == P::NFR - 1 ? 0 : fslot + 1;
         xslot ^= 1;
-        if (it + 1 < total) advance(cc);
-    }
-    if (cc.kind == 2) {                                      // the run ended with the end of a shared tile
-        gather();
-        stores();
+        if (++cs == nst) {
+            cs = 0;
+            s += sstep;
+        }
     }
 }
 

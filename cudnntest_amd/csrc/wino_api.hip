@@ -856,6 +856,7 @@ bool direct16_plan(const Geometry& g, int npg, bool rows, D16Geom* d) {
     d->colBlocks = (g.Wo + BC - 1) / BC;
     d->rowBlocks = (int)((G + BR - 1) / BR);
     d->maxcross = (g.Ho + BR - 2) / g.Ho;
+    d->a4 = 0; d->b3 = 0;
     d->kTiles = (g.K + D16_KT - 1) / D16_KT;
     d->CQ = (int)round_up(g.C, 32) / 8;
     d->Kp = (int)round_up(g.K, D16_KT);
@@ -896,6 +897,7 @@ bool direct16_rows_plan(const Geometry& gl, D16Geom* d) {
     d->colBlocks = (g.Wo + BC - 1) / BC;
     d->rowBlocks = (int)((G + BR - 1) / BR);
     d->maxcross = maxcross;
+    d->a4 = 0; d->b3 = 0;
     d->kTiles = (g.K + P::KT - 1) / P::KT;
     d->CQ = (int)round_up(g.C, 16) / 8;
     d->Kp = (int)round_up(g.K, P::KT);
@@ -904,41 +906,66 @@ bool direct16_rows_plan(const Geometry& gl, D16Geom* d) {
 }
 inline int direct16_rows_wf(const Geometry& g) { return (g.K % 128 == 0 || g.K > 256) ? 2 : 1; }
 
-// Scratch of the 8-wave direct kernel for the workgroups that share a tile: one block of partial sums per workgroup
-// (128 registers x 512 threads) and an arrival counter each (the arena's first 4 KB).
-struct D16Share {
-    float* part = nullptr;
-    int* cnt = nullptr;
-};
-constexpr size_t kD16PartPerWg = (size_t)128 * 512 * sizeof(float);
-size_t direct16_part_bytes() { return (size_t)(device_cus() / 8 * 8) * kD16PartPerWg; }
+// Blocks whose waves own 3 rows mixed in with the 4-row ones.  A layer is a handful of tiles per CU, and rounds of
+// whole tiles leave a good part of the chip idle in the last one (N = 32, C = K = 256, 56 x 56: 448 tiles on 256 CUs, two
+// rounds for 1.75 rounds of work).  A 3-row tile is three quarters of the multiplies: cut every image into a4 blocks of
+// 4-row waves and b3 of 3-row waves, 4-row blocks first, and the same layer is 512 tiles, one of each kind to a CU:
+// 7 units instead of 8.  The cost of a cut is taken as the largest sum of rows-per-wave over a workgroup's tiles,
+// dealt round-robin; a cut is taken when it saves at least 6 %.  (Pooling needs whole row pairs in a wave: no cut.)
+long direct16_deal_cost(long t4, long t3, long wgs) {
+    long worst = 0;
+    const long total = t4 + t3;
+    const long probe[5] = {0, t4 % wgs, (t4 % wgs + wgs - 1) % wgs, total % wgs, (total % wgs + wgs - 1) % wgs};
+    for (long j : probe) {
+        if (j >= total) continue;
+        const long n = (total - j + wgs - 1) / wgs, n4 = j < t4 ? (t4 - j + wgs - 1) / wgs : 0;
+        worst = std::max(worst, 4 * n4 + 3 * (n - n4));
+    }
+    return worst;
+}
+void direct16_row_mix(D16Geom* d, bool pool) {
+    const int S = d->BR / 4;
+    if (pool || d->Ho % S != 0) return;
+    const long per = (long)d->colBlocks * d->kTiles, cus = std::max(8, device_cus() / 8 * 8);
+    const long plain_tiles = (long)d->rowBlocks * per;
+    const long plain = direct16_deal_cost(plain_tiles, 0, std::min(cus, (plain_tiles + 7) / 8 * 8));
+    long best = plain;
+    int best_b = 0;
+    const int units = d->Ho / S;                             // = 4 a4 + 3 b3
+    for (int b = 1; 3 * b <= units; ++b) {
+        if ((units - 3 * b) % 4 != 0) continue;
+        const int a = (units - 3 * b) / 4;
+        const long t4 = (long)d->N * a * per, t3 = (long)d->N * b * per;
+        if ((t4 + t3) / per >= (1L << 28) / d->colBlocks) break;
+        const long cost = direct16_deal_cost(t4, t3, std::min(cus, (t4 + t3 + 7) / 8 * 8));
+        if (cost < best) {
+            best = cost;
+            best_b = b;
+        }
+    }
+    if (best_b == 0 || best * 100 > plain * 94) return;
+    d->b3 = best_b;
+    d->a4 = (units - 3 * best_b) / 4;
+    d->rowBlocks = d->N * (d->a4 + d->b3);
+    d->maxcross = 0;
+}
 
 template <typename T, int WF, bool XN = false, bool YN = XN, bool DIL = false>
-int launch_direct16_rows_t(const D16Geom& d, const Epilogue& ep, const void* x, const void* W9, void* y, const D16Share& sh,
-                           hipStream_t st) {
+int launch_direct16_rows_t(const D16Geom& planned, const Epilogue& ep, const void* x, const void* W9, void* y, hipStream_t st) {
+    D16Geom d = planned;
+    direct16_row_mix(&d, ep.pool != 0);
     static std::atomic<bool> attr_set{false};    // (per instantiation; setting it twice from two threads is harmless)
     if (!attr_set.load(std::memory_order_acquire)) {
         HIP_TRY(hipFuncSetAttribute((const void*)direct16_rows_kernel<T, WF, XN, YN, DIL>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     D16R<WF, DIL>::LDS));
         attr_set.store(true, std::memory_order_release);
     }
-    // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs.  The
-    // tiles left over after the full rounds are shared out by stages (partial sums through scratch) when they would
-    // occupy at most half of the workgroups: sharing costs a workgroup about six stage times (its accumulators out and
-    // in, two or three partial tiles to set up instead of one), so a last round that is three quarters full is better
-    // left alone (measured at N = 32 in bf16, shared against whole: C = K = 256 at 56 x 56, 24 tiles over 32 workgroups
-    // of an XCD, 136 against 129 us; C = K = 512 at 28 x 28, 28 over 32, 131 against 125 us).
+    // persistent grid: one workgroup of 8 waves per CU (or as many as there are tiles), a multiple of the 8 XCDs
     const long tiles = (long)d.rowBlocks * d.colBlocks * d.kTiles;
-    const long per_xcd = ((long)d.rowBlocks * d.colBlocks + 7) / 8 * d.kTiles;      // tiles of the XCD with the most
-    const long sx_all = std::max<long>(1, device_cus() / 8);
-    const long left_over = per_xcd % sx_all;
-    // (a run of at least four stages to every workgroup, or the kernel deals the left-over tiles out whole anyway)
-    const bool share = sh.part && left_over > 0 && 2 * left_over <= sx_all && left_over * (d.CQ / 2) >= 4 * sx_all &&
-                       sx_all * 8 <= (long)(kCounterBytes / sizeof(int));
-    const long sx = share ? sx_all : std::max<long>(1, std::min<long>(sx_all, (tiles + 7) / 8));
+    const long blocks = std::max<long>(8, std::min<long>(device_cus(), (tiles + 7) / 8 * 8) / 8 * 8);
     constexpr int kLds = D16R<WF, DIL>::LDS;
-    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN, DIL>), dim3((unsigned)(sx * 8)), dim3(512), kLds, st, (const T*)x,
-                       (const T*)W9, (T*)y, d, ep, share ? sh.part : nullptr, share ? sh.cnt : nullptr, 1 << 22);
+    hipLaunchKernelGGL((direct16_rows_kernel<T, WF, XN, YN, DIL>), dim3((unsigned)blocks), dim3(512), kLds, st, (const T*)x,
+                       (const T*)W9, (T*)y, d, ep);
     LAUNCH_CHECK("direct16_rows");
     return WINO_OK;
 }
@@ -994,7 +1021,7 @@ int launch_direct16_t(const D16Geom& d, const Epilogue& ep, const void* x, const
 // for tensors of the same alignment.
 enum { D16_PACK_RUN = 0, D16_PACK = 1, D16_RUN = 2 };
 int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x,
-                    const void* w, void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN, const D16Share& sh = D16Share{}) {
+                    const void* w, void* W9, void* y, hipStream_t st, int mode = D16_PACK_RUN) {
     const bool nhwc = layout == WINO_NHWC, ynhwc = dst == WINO_NHWC, chwn = layout == WINO_CHWN;
     if (chwn != (dst == WINO_CHWN)) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: CHWN tensors on both sides or on neither");
     if (misaligned(x, nhwc ? 16 : 4))
@@ -1028,16 +1055,16 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
         LAUNCH_CHECK("direct16_pack");                                                                             \
     }                                                                                                              \
     if (mode == D16_PACK) return WINO_OK;                                                                          \
-    if (chwn) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, false, true>(d, ep, x, W9, y, sh, st);         \
-                return launch_direct16_rows_t<T, 1, false, false, true>(d, ep, x, W9, y, sh, st); }                    \
-    if (nhwc && ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, true>(d, ep, x, W9, y, sh, st);        \
-                         return launch_direct16_rows_t<T, 1, true, true>(d, ep, x, W9, y, sh, st); }                   \
-    if (nhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, false>(d, ep, x, W9, y, sh, st);                \
-                return launch_direct16_rows_t<T, 1, true, false>(d, ep, x, W9, y, sh, st); }                           \
-    if (ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, true>(d, ep, x, W9, y, sh, st);               \
-                 return launch_direct16_rows_t<T, 1, false, true>(d, ep, x, W9, y, sh, st); }                          \
-    if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, sh, st);                                  \
-    if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, sh, st);                                             \
+    if (chwn) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, false, true>(d, ep, x, W9, y, st);         \
+                return launch_direct16_rows_t<T, 1, false, false, true>(d, ep, x, W9, y, st); }                    \
+    if (nhwc && ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, true>(d, ep, x, W9, y, st);        \
+                         return launch_direct16_rows_t<T, 1, true, true>(d, ep, x, W9, y, st); }                   \
+    if (nhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, true, false>(d, ep, x, W9, y, st);                \
+                return launch_direct16_rows_t<T, 1, true, false>(d, ep, x, W9, y, st); }                           \
+    if (ynhwc) { if (wf == 2) return launch_direct16_rows_t<T, 2, false, true>(d, ep, x, W9, y, st);               \
+                 return launch_direct16_rows_t<T, 1, false, true>(d, ep, x, W9, y, st); }                          \
+    if (big && wf == 2) return launch_direct16_rows_t<T, 2>(d, ep, x, W9, y, st);                                  \
+    if (big) return launch_direct16_rows_t<T, 1>(d, ep, x, W9, y, st);                                             \
     if (rows) return launch_direct16_t<T, 4, true>(d, ep, x, W9, y, st);                                           \
     if (npg == 4) return launch_direct16_t<T, 4, false>(d, ep, x, W9, y, st);                                      \
     if (npg == 2) return launch_direct16_t<T, 2, false>(d, ep, x, W9, y, st);                                      \
@@ -1237,20 +1264,11 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (!direct16_ok(src, dst, dtype, flags, g))
             return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for pad 0 and 1: for C <= 4, and for 2-byte NCHW tensors with "
                                               "C a multiple of 8 and an even width (pooling: output height a multiple of 4, K a multiple of 64, a large layer)");
-        // counters, the re-ordered bank, and the partial sums of workgroups that share a tile (left out, and the
-        // tiles run whole, where a fixed scratch buffer has no room for them)
         void* base = nullptr;
-        const size_t bank = (direct16_bank_bytes(g) + 255) / 256 * 256;
-        const bool share = !ss.fixed || kCounterBytes + bank + direct16_part_bytes() <= ss.fixed_bytes;
-        const int rcb = ss.get(kCounterBytes + bank + (share ? direct16_part_bytes() : 0), &base);
+        const int rcb = ss.get(kCounterBytes + direct16_bank_bytes(g), &base);
         if (rcb) return rcb;
-        D16Share sh;
-        if (share) {
-            sh.part = (float*)((char*)base + kCounterBytes + bank);
-            sh.cnt = (int*)base;
-        }
         StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-        return launch_direct16(src, dst, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream, D16_PACK_RUN, sh);
+        return launch_direct16(src, dst, dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, y, (hipStream_t)stream);
     }
     if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4)
         return conv_f4_impl(ss, src, dst, dtype, algo, flags, bias, N, C, K, H, W, pad, x, w, Upre, y, stream);
@@ -1781,14 +1799,8 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
         } else if (L.W9 && !misaligned(in, 4) && (!misaligned(out, 4) || (L.flags & WINO_FLAG_POOL2)) &&
                    auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in, out)) {
             // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
-            void* base = nullptr;                           // the partial sums of workgroups that share a tile: the arena
-            rc = arena_get(kCounterBytes + direct16_part_bytes(), &base);
-            if (rc) return rc;
-            D16Share sh;
-            sh.part = (float*)((char*)base + kCounterBytes);
-            sh.cnt = (int*)base;
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-            rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN, sh);
+            rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
         } else {
             rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
                            L.wraw, L.U, bias, out, stream);
@@ -1930,7 +1942,6 @@ int wino_stack_forward_graph(wino_stack_t* s, const void* x, void* y, void* stre
         Geometry g;
         if (!make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g)) return fail(WINO_ERR_INVALID, "bad layer shape");
         need = std::max(need, scratch_layout(g, s->dtype).total);
-        if (L.W9) need = std::max(need, kCounterBytes + direct16_part_bytes());
         Geometry g4;
         if (L.U4 && make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4))
             need = std::max(need, scratch_layout(g4, s->dtype, auto_f4_algo(s->dtype, g4)).total);

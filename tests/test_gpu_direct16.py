@@ -185,16 +185,15 @@ def test_chwn_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
         assert err <= (1e-3 if dtype == ops.F16 else 5e-3), err
 
 
-@pytest.mark.parametrize("shape,layout", [((46, 256, 128, 56, 56), ops.NCHW), ((46, 256, 128, 56, 56), ops.NHWC),
-                                          ((10, 512, 128, 56, 56), ops.NCHW), ((44, 256, 256, 56, 56), ops.NHWC),
-                                          ((24, 256, 256, 56, 56), ops.CHWN)])
-def test_left_over_tiles_shared_out_by_stages(oracle, shape, layout):
-    """Layers whose last round of tiles would occupy at most half of the workgroups: the 8-wave kernel cuts the stage
-    sequence of those tiles into equal runs, workgroups leave partial sums of the tiles they share in scratch and the
-    tile's owner adds them in a fixed order.  One full round and nine tiles more per XCD; a fraction of a round only
-    (every workgroup holds parts of tiles); two filter tiles, two rounds and fourteen tiles; a CHWN layer.  Small integers: exact whatever the order of the sums --
-    the staged Winograd pipeline's bits, the oracle's planes, three times in a row (the arrival counters return to
-    zero)."""
+@pytest.mark.parametrize("shape,layout", [((32, 64, 256, 56, 56), ops.NCHW), ((32, 64, 256, 56, 56), ops.NHWC),
+                                          ((32, 32, 128, 112, 112), ops.NCHW), ((32, 64, 256, 56, 56), ops.CHWN),
+                                          ((20, 48, 128, 60, 56), ops.NCHW)])
+def test_layers_whose_images_are_cut_into_4_row_and_3_row_blocks(oracle, shape, layout):
+    """Layers whose tiles would leave a good part of the chip idle in their last round: the 8-wave kernel's host side
+    cuts every image into blocks whose waves own 4 rows and blocks whose waves own 3 (the VGG geometries at N = 32 with
+    fewer channels: 56 x 56 with two filter tiles, 448 tiles -> 256 + 256; 112 x 112, 896 -> 512 + 512; the CHWN layer as
+    one wide image; an image height that is a multiple of 4 but not of 8).  Small integers: the staged Winograd
+    pipeline's bits, and the oracle's on the first and last image."""
     N, C, K, H, W = shape
     dtype = ops.BF16
     x = synth.small_ints(N * C * H * W, sum(shape), -1, 1).reshape(N, C, H, W)
@@ -202,14 +201,17 @@ def test_left_over_tiles_shared_out_by_stages(oracle, shape, layout):
     bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
     xd, wd, bd = dev(synth.act_to_layout(x, layout), dtype), dev(synth.flt_to_layout(w, layout), dtype), dev(bias, dtype)
     ref = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=bd)
+    got = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
+    assert torch.equal(got, ref)
     ks = sorted({0, K // 2, K - 1})
-    for rep in range(3):
-        got = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_DIRECT, relu=True, bias=bd)
-        assert torch.equal(got, ref), rep
     g = synth.act_from_layout(host(got), layout)
     for n in (0, N - 1):
         want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], 1) + bias[ks][None, :, None, None], 0)
         assert np.array_equal(g[n:n + 1][:, ks], rounded(want.astype(np.float32), dtype, oracle)), n
+    if layout != ops.CHWN:                                     # pooled: whole row pairs in a wave, so no cut -- the same values, pooled
+        pooled = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+        want = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True)
+        assert torch.equal(pooled, want)
 
 
 def test_chwn_layers_the_8_wave_kernel_does_not_take():
