@@ -633,9 +633,16 @@ int launch_f4_input(int layout, int order, const Geometry& g, const void* x, voi
             if (in_blocks + extra < (1L << 31) && (size_t)NQ * plane <= 65536) {
                 const int stepC = 256 / (g.H * g.W), stepH = (256 - stepC * g.H * g.W) / g.W,
                           stepW = 256 - stepC * g.H * g.W - stepH * g.W;
-                hipLaunchKernelGGL((input_transform_nchw_small_kernel<float, 1, 4>), dim3((unsigned)(in_blocks + extra)), dim3(256),
-                                   (size_t)NQ * plane, st, (const float*)x, (float*)V, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp,
-                                   NQ, groups, (int)in_blocks, stepC, stepH, stepW, fj);
+                // rows in 16-byte pieces where they consist of them and a thread's share is at most 16
+                const bool quad = g.W % 4 == 0 && !misaligned(x, 16) && (long)NQ * CV * g.H * (g.W / 4) <= 16 * 256;
+                if (quad)
+                    hipLaunchKernelGGL((input_transform_nchw_small_kernel<float, 1, 4, true>), dim3((unsigned)(in_blocks + extra)), dim3(256),
+                                       (size_t)NQ * plane, st, (const float*)x, (float*)V, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp,
+                                       NQ, groups, (int)in_blocks, stepC, stepH, stepW, fj);
+                else
+                    hipLaunchKernelGGL((input_transform_nchw_small_kernel<float, 1, 4>), dim3((unsigned)(in_blocks + extra)), dim3(256),
+                                       (size_t)NQ * plane, st, (const float*)x, (float*)V, g.C, g.H, g.W, g.pad, g.th, g.tw, g.Pp, g.Cp,
+                                       NQ, groups, (int)in_blocks, stepC, stepH, stepW, fj);
                 LAUNCH_CHECK("f4_input_transform_nchw_small");
                 return WINO_OK;
             }
