@@ -71,27 +71,30 @@ WORKLOADS = {
 # script (the summary file holds the counters and the copy-kernel scale factor), keyed by
 # (workload, layout, dtype, resolved algo): (bytes, summary under profiles/).
 MEASURED_TRAFFIC = {
-    # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_spread_kernel): 320.9 MB fetched + 231.2 MB written
+    # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_spread_kernel): 320.8 MB fetched + 231.2 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged_f4"):
         (552.1e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
-    # 636.1 MB fetched + 111.2 MB written (partial sums of the cut-up last round included)
+    # gemm_rows_f4_kernel: 1435.0 MB fetched (a patch's rows of V once per filter tile, most of it from the L2) + 515.0 MB written
+    ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue_f4"):
+        (1949.9e6, "profiles/epilogue_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    # gemm_rows_kernel (partial sums of the cut-up last round included)
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue"):
-        (747.2e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_counters.txt"),
-    # 483.1 MB fetched + 411.0 MB written
+        (746.9e6, "profiles/epilogue_fp32_nchw_vgg16_conv3_N32_counters.txt"),
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged"):
-        (894.1e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_counters.txt"),
-    # 581.5 MB fetched + 411.0 MB written
+        (896.8e6, "profiles/staged_fp32_nchw_vgg16_conv3_N32_counters.txt"),
     ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "f32", "fused"):
-        (992.6e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_counters.txt"),
-    # direct16_rows_kernel: 83.1 + 51.4 MB; 325.3 + 209.2 MB
+        (994.6e6, "profiles/fused_fp32_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # direct16_rows_kernel: 93.6 + 51.4 MB
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "direct"):
-        (134.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv3_N32_counters.txt"),
+        (145.0e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv3_N32_counters.txt"),
     ("vgg16_conv1_2_N32_C64_K64_H224", "NCHW", "bf16", "direct"):
-        (534.5e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv1_2_N32_counters.txt"),
-    # the same kernel from NHWC tensors: 86.3 + 51.4 MB
+        (533.6e6, "profiles/direct16_rows_bf16_nchw_vgg16_conv1_2_N32_counters.txt"),
+    # the same kernel from NHWC tensors, and from CHWN ones (one image of width W * N: 4-row blocks read 6 input rows)
     ("vgg16_conv3_N32_C256_K256_H56", "NHWC", "bf16", "direct"):
-        (137.7e6, "profiles/direct16_rows_bf16_nhwc_vgg16_conv3_N32_counters.txt"),
-    # gemm_rows_kernel in bf16: 271.5 MB fetched + 56.9 MB written
+        (145.7e6, "profiles/direct16_rows_bf16_nhwc_vgg16_conv3_N32_counters.txt"),
+    ("vgg16_conv3_N32_C256_K256_H56", "CHWN", "bf16", "direct"):
+        (235.0e6, "profiles/direct16_rows_bf16_chwn_vgg16_conv3_N32_counters.txt"),
+    # gemm_rows_kernel in bf16
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "bf16", "epilogue"):
         (328.4e6, "profiles/epilogue_bf16_nchw_vgg16_conv3_N32_counters.txt"),
 }
@@ -109,7 +112,7 @@ OTHER_CONFIGS = [
     ("cfg5_vgg16_all13_N32_bf16_CHWN", "vgg16_all13", "bf16", "CHWN"),
 ]
 KERNEL_OF = {"epilogue_f4": "gemm_rows_f4_kernel", "staged": "gemm_128x128_kernel / gemm_128x128_walk_kernel / gemm_128x128_walk_spread_kernel", "epilogue": "gemm_rows_kernel", "fused": "fused_rows_kernel",
-             "staged_f4": "gemm_128x128_walk_spread_kernel / gemm_128x128_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel"}
+             "staged_f4": "gemm_128x128_walk_spread_kernel / gemm_128x128_kernel", "direct": "direct16_rows_kernel / direct_small_c kernel / direct_few_pixels_kernel"}
 
 
 def main():

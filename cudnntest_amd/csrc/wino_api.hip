@@ -874,8 +874,11 @@ bool direct16_plan(const Geometry& g, int npg, bool rows, D16Geom* d) {
 // The 8-wave kernel of direct16_rows.hpp: blocks of 32/WF rows x 32 columns whose waves own 4 consecutive rows of one
 // image.  WF = 2 (128 filters per tile) when that wastes no filters, else 1.
 // DIL: a CHWN layer taken as ONE image of width W * N whose tap columns lie N elements apart (direct16_rows.hpp).
+// xn: the source is NHWC.  With 64-filter tiles its blocks stay 128 columns wide and 8 rows high on wider images: a stage
+// takes 32 of a pixel's bytes, and the taller block reads 10 input rows for 8 instead of 6 for 4 (C = K = 64, 224 x 224
+// at N = 32 in bf16: 210 -> 178 us; from NCHW, where a row of a block is one contiguous run, the wide block stays: 195 against 199).
 template <int WF, bool DIL = false>
-bool direct16_rows_plan(const Geometry& gl, D16Geom* d) {
+bool direct16_rows_plan(const Geometry& gl, D16Geom* d, bool xn = false) {
     typedef D16R<WF, DIL> P;
     Geometry g = gl;
     int ds = 1;
@@ -890,15 +893,21 @@ bool direct16_rows_plan(const Geometry& gl, D16Geom* d) {
     const long G = (long)g.N * g.Ho;
     if (g.Ho % 4 != 0 || g.K % 64 != 0 || g.Wo % 2 != 0) return false;
     // the block's waves (4 rows x 32 columns each) side by side until they span the image, the rest stacked
-    int WC = 1;
-    while (WC < P::WP && 32 * WC < g.Wo) WC *= 2;
-    const int BR = 4 * (P::WP / WC), BC = 32 * WC;
-    if (G < BR) return false;
-    const int maxcross = g.Ho % BR == 0 ? 0 : (g.Ho + BR - 2) / g.Ho;     // images a block's rows can span beyond the first
-    const int PW = std::min(BC, (g.Wo + 1) / 2 * 2) + 2 * ds; // slots of an LDS row: the block's columns (or the image's) + the two tap columns
+    int WC = 0, BR = 0, BC = 0, maxcross = 0, PW = 0, LR = 0, PP = 0;
     const int padw = g.pad * ds;                              // zero columns left of a row; pairs start at even columns
-    const int LR = BR + 2 + 2 * maxcross, PP = (PW + (padw & 1) + 1) / 2;
-    if (LR * PW > P::XPLANE || 2 * LR * PP > P::NTASK * 512 || LR > 255 || PW > 2048) return false;
+    for (int wc_cap : {xn && WF == 1 ? 4 : P::WP, P::WP}) {   // (the narrower block first where it is preferred; the wide one if its rows do not fit)
+        WC = 1;
+        while (WC < wc_cap && 32 * WC < g.Wo) WC *= 2;
+        BR = 4 * (P::WP / WC);
+        BC = 32 * WC;
+        if (G < BR) return false;
+        maxcross = g.Ho % BR == 0 ? 0 : (g.Ho + BR - 2) / g.Ho;           // images a block's rows can span beyond the first
+        PW = std::min(BC, (g.Wo + 1) / 2 * 2) + 2 * ds;     // slots of an LDS row: the block's columns (or the image's) + the two tap columns
+        LR = BR + 2 + 2 * maxcross;
+        PP = (PW + (padw & 1) + 1) / 2;
+        if (!(LR * PW > P::XPLANE || 2 * LR * PP > P::NTASK * 512 || LR > 255 || PW > 2048)) break;
+        if (wc_cap == P::WP) return false;
+    }
     d->N = g.N; d->C = g.C; d->K = g.K; d->H = g.H; d->W = g.W; d->pad = g.pad; d->Ho = g.Ho; d->Wo = g.Wo;
     d->BR = BR; d->BC = BC; d->WC = WC; d->PW = PW; d->LR = LR; d->PP = PP; d->ds = ds;
     d->colBlocks = (g.Wo + BC - 1) / BC;
@@ -980,9 +989,9 @@ int launch_direct16_rows_t(const D16Geom& planned, const Epilogue& ep, const voi
 size_t direct16_bank_bytes(const Geometry& g) { return (size_t)9 * round_up(g.C, 32) * round_up(g.K, 128) * 2; }
 
 // whether a layer runs on the 8-wave kernel (given 4-byte aligned tensors); chwn: as one image of width W * N
-bool direct16_big(const Geometry& g, D16Geom* d, bool chwn = false) {
+bool direct16_big(const Geometry& g, D16Geom* d, bool chwn = false, bool xn = false) {
     const bool plan = chwn ? (direct16_rows_wf(g) == 2 ? direct16_rows_plan<2, true>(g, d) : direct16_rows_plan<1, true>(g, d))
-                           : (direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, d) : direct16_rows_plan<1>(g, d));
+                           : (direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, d, xn) : direct16_rows_plan<1>(g, d, xn));
     return plan && (long)d->rowBlocks * d->colBlocks * d->kTiles >= device_cus() / 2;
 }
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
@@ -995,7 +1004,7 @@ bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g)
     }
     if (src == WINO_NHWC || dst == WINO_NHWC) {
         // an NHWC side: the 8-wave kernel only; offsets inside a block's images are 32-bit
-        if (!direct16_big(g, &d)) return false;
+        if (!direct16_big(g, &d, false, src == WINO_NHWC)) return false;
         return src == WINO_NHWC ? (long)(d.maxcross + 1) * g.C * g.H * g.W * 2 < (1L << 32)
                                 : g.W % 2 == 0 && (long)g.C * g.H * g.W * 2 * 8 < (1L << 32);
     }
@@ -1038,7 +1047,7 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
     // the chip short of tiles
     int npg = 4, wf = direct16_rows_wf(g);
     const bool pool = (flags & WINO_FLAG_POOL2) != 0;        // (pooled values are stored one by one: no alignment asked of y)
-    const bool big = (pool || !misaligned(y, 4)) && !(chwn && pool) && direct16_big(g, &d, chwn);
+    const bool big = (pool || !misaligned(y, 4)) && !(chwn && pool) && direct16_big(g, &d, chwn, nhwc);
     if (chwn && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of CHWN tensors: the 8-wave kernel's layer shapes, an even batch, no pooling, y 4-byte aligned");
     if ((nhwc || ynhwc) && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of NHWC tensors: the 8-wave kernel's layer shapes, y 4-byte aligned");
     if (pool && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: pooling needs the 8-wave kernel's layer shapes");
@@ -1141,7 +1150,7 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
         // 7 x 7 blocks of a filter tile leave a quarter of the chip idle: 121 against 72, 225 against 128 us)
         return planc && g.Ho >= 48 && g.Wo >= 48 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus();
     }
-    const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d) : direct16_rows_plan<1>(g, &d);
+    const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d, src == WINO_NHWC) : direct16_rows_plan<1>(g, &d, src == WINO_NHWC);
     if (plan8 && g.Ho >= 28 && g.Wo >= 28 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus()) return true;
     if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 48 || g.Wo < 48) return false;
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
