@@ -181,16 +181,21 @@ __global__ __launch_bounds__(256) void direct_small_c_kernel(const T* __restrict
 // instructions a CU can take (about one per 16 clocks, whatever its width), so a wave fetches a group with as few
 // as the layout allows and hands the elements to the lanes that multiply them through LDS of its own:
 //   * the input patch of a group, 4 channels x 6 x 10 elements (zeros where the padding is), is 4 loads per lane;
-//   * the filter block, 32 filters x 36 elements, is contiguous per filter in a [K][C][3][3] bank: 5 loads of 16
-//     bytes per lane (any other order, or C not a multiple of 4: 18 loads of one element);
+//     where the channels are the contiguous axis (XW: NHWC) a pixel's 4 channels are one load of 16 bytes, one
+//     load per lane;
+//   * the filter block, 32 filters x 36 elements, in 16-byte pieces, 5 loads per lane: a [K][C][3][3] bank holds a
+//     filter's 36 elements of a group contiguously (FM = 1), a [K][3][3][C] bank the 4 channels of a (filter, tap)
+//     (FM = 2), a [C][3][3][K] bank 4 filters of a (channel, tap) (FM = 3); any other order, or C (FM = 3: C or
+//     K) not a multiple of 4: 18 loads of one element (FM = 0);
 //   * the waves' partial sums meet in LDS and each wave stores two of the 16 filter rows of the sum (bias, ReLU).
 // Any layout on either side (element strides), any padding; the partial sums are added in wave order, so results do
-// not depend on the launch.
+// not depend on the launch.  The order in which a group's 36 products enter the sum follows the bank (FM = 2: tap
+// major), so results of different layouts agree to rounding, not bit for bit.
 constexpr int DFP_NE = 18;                  // multiplies per group of 4 channels
 constexpr int DFP_ROW = 37;                 // floats per filter in the wave's strip of LDS (36 + 1: the 32 lanes of a read hit 32 banks)
 constexpr int DFP_PATCH = 4 * 6 * 10;       // a group's input patch: 4 channels x (4 + 2) rows x (8 + 2) columns
 
-template <typename T>
+template <typename T, int FM, bool XW>
 __global__ __launch_bounds__(512) void direct_few_pixels_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                                 T* __restrict__ y, ActStrides xs, FltStrides ws,
                                                                 ActStrides ys, int N, int C, int K, int H, int W, int pad,
@@ -216,33 +221,46 @@ __global__ __launch_bounds__(512) void direct_few_pixels_kernel(const T* __restr
 
     // Input patch as loaded: element 64 j + lane of [4][6][10], j < 4: byte offset in x relative to the group's
     // first channel (0 and a zero mask where the element lies in the padding or past the patch).
-    unsigned offx[4], mx[4];
+    // XW: lane p < 60 loads the 4 channels of pixel p of [6][10] as one piece.
+    constexpr int NX = XW ? 1 : 4;
+    unsigned offx[NX], mx[NX];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NX; ++j) {
         const int p = 64 * j + lane;
-        const int c = (p * 1093) >> 16, rem = p - 60 * c;                    // p / 60, p % 60 (p < 256)
+        const int c = XW ? 0 : (p * 1093) >> 16, rem = p - 60 * c;            // p / 60, p % 60 (p < 256)
         const int rr = (rem * 205) >> 11, cc = rem - 10 * rr;                 // rem / 10, rem % 10 (rem < 64)
         const int ih = oh0 - pad + rr, iw = ow0 - pad + cc;
-        const bool in = p < DFP_PATCH && ih >= 0 && ih < H && iw >= 0 && iw < W;
+        const bool in = p < (XW ? 60 : DFP_PATCH) && ih >= 0 && ih < H && iw >= 0 && iw < W;
         offx[j] = in ? (unsigned)((int)(n * xs.n + c * xs.c + ih * xs.h + iw * xs.w) * (int)sizeof(T)) : 0u;
         mx[j] = in ? 0xFFFFFFFFu : 0u;
     }
     __syncthreads();
-    // Filter block as loaded: a bank in [K][C][3][3] order holds a filter's 36 elements of a group contiguously:
-    // 16-byte piece 64 j + lane of the [32][9] pieces, j < 5.  Any other order: element 64 j + lane of [32][36],
-    // j < 18.  Byte offset in w relative to the group's first channel, mask (filters past K), place in the strip.
-    const bool wide = ws.s == 1 && ws.r == 3 && ws.c == 9 && (C & 3) == 0;
-    unsigned offw[NE], mw[NE];
-    int sidx[NE];
+    // Filter block as loaded.  FM = 1, 2: 16-byte piece 64 j + lane of the [32 filters][9] pieces of a group, j < 5
+    // (FM = 1: elements 4 part .. 4 part + 3 of the filter's 36; FM = 2: the 4 channels of tap `part`).  FM = 3:
+    // piece 64 j + lane of [36 (channel, tap)][8]: filters 4 piece .. 4 piece + 3.  FM = 0: element 64 j + lane of
+    // [32][36], j < 18.  Byte offset in w relative to the group's first channel, mask (filters past K), place in
+    // the strip: a filter's row holds position 9 c + tap (FM = 2: 4 tap + c) of the group.
+    constexpr bool wide = FM != 0;
+    constexpr int NW = wide ? 5 : NE;
+    unsigned offw[NW], mw[NW];
+    int sidx[NW];
 #pragma unroll
-    for (int j = 0; j < NE; ++j) {
+    for (int j = 0; j < NW; ++j) {
         const int idx = 64 * j + lane;
-        if (wide) {
+        if (FM == 1 || FM == 2) {
             const int fk = (idx * 7282) >> 16, part = idx - 9 * fk;           // idx / 9, idx % 9 (idx < 320)
-            const bool fok = j < 5 && fk < 32 && kt * 32 + fk < K;
-            offw[j] = fok ? (unsigned)(((kt * 32 + fk) * (int)ws.k + 4 * part) * (int)sizeof(T)) : 0u;
+            const bool fok = fk < 32 && kt * 32 + fk < K;
+            const int at = FM == 1 ? 4 * part : (part / 3) * (int)ws.r + (part % 3) * (int)ws.s;
+            offw[j] = fok ? (unsigned)(((kt * 32 + fk) * (int)ws.k + at) * (int)sizeof(T)) : 0u;
             mw[j] = fok ? 0xFFFFFFFFu : 0u;
             sidx[j] = fk < 32 ? fk * DFP_ROW + 4 * part : 0;
+        } else if (FM == 3) {
+            const int row = idx >> 3, piece = idx & 7;                         // (channel, tap) 9 c + tap, filters 4 piece ..
+            const bool fok = row < 36 && kt * 32 + 4 * piece < K;              // (K a multiple of 4)
+            const int c = (row * 57) >> 9, tap = row - 9 * c;                  // row / 9 (row < 40)
+            offw[j] = fok ? (unsigned)((c * (int)ws.c + (tap / 3) * (int)ws.r + (tap % 3) * (int)ws.s + kt * 32 + 4 * piece) * (int)sizeof(T)) : 0u;
+            mw[j] = fok ? 0xFFFFFFFFu : 0u;
+            sidx[j] = row < 36 ? 4 * piece * DFP_ROW + row : 0;
         } else {
             const int fk = (idx * 1821) >> 16, fkk = idx - 36 * fk;           // idx / 36, idx % 36 (idx < 1152)
             const bool fok = kt * 32 + fk < K;
@@ -259,19 +277,24 @@ __global__ __launch_bounds__(512) void direct_few_pixels_kernel(const T* __restr
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
     // the group on its way: 4 patch elements; 5 filter pieces of 4 elements (wide) or 18 elements
-    T rb[4];
     struct alignas(4) T4 { T v[4]; };
+    T rb[4];
+    T4 rb4;
     T4 rw4[5];
-    T rw[NE];
+    T rw[NW];
     int cleft = 0;                                            // channels of that group that exist, counted from the wave's first
     int crem = C - wave * 4;
     auto load = [&]() __attribute__((always_inline)) {        // the group at xg, wg; the pointers move on
         cleft = crem;
+        if (XW) {
+            rb4 = *reinterpret_cast<const T4*>(xg + offx[0]);                 // (C a multiple of 4: the group's channels exist)
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            // (a channel past C: the first element of the group's first channel is read instead, and masked)
-            const int c = ((64 * j + lane) * 1093) >> 16;
-            rb[j] = *reinterpret_cast<const T*>(xg + (c < crem ? offx[j] : 0u));
+            for (int j = 0; j < 4; ++j) {
+                // (a channel past C: the first element of the group's first channel is read instead, and masked)
+                const int c = ((64 * j + lane) * 1093) >> 16;
+                rb[j] = *reinterpret_cast<const T*>(xg + (c < crem ? offx[j] : 0u));
+            }
         }
         if (wide) {
 #pragma unroll
@@ -290,15 +313,27 @@ __global__ __launch_bounds__(512) void direct_few_pixels_kernel(const T* __restr
     float* const mine = strip[wave];
     float* const mypatch = patch[wave];
     float a[NE], b[NE];
-    // the group that has arrived -> the wave's strip and patch -> a, b: multiply e of a lane takes reduction index
-    // 18 lh + e of the group, (channel 2 lh + e / 9, tap e % 9)
+    // the group that has arrived -> the wave's strip and patch -> a, b: multiply e of a lane takes (channel
+    // 2 lh + e / 9, tap e % 9) of the group (FM = 2: channel 2 lh + e % 2, tap e / 2)
     auto stage = [&]() __attribute__((always_inline)) {
+        if (XW) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int p = 64 * j + lane, c = (p * 1093) >> 16;
-            if (p < DFP_PATCH) mypatch[p] = __uint_as_float(__float_as_uint(to_f32(rb[j])) & (c < cleft ? mx[j] : 0u));
+            for (int i = 0; i < 4; ++i)
+                if (lane < 60) mypatch[60 * i + lane] = __uint_as_float(__float_as_uint(to_f32(rb4.v[i])) & mx[0]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int p = 64 * j + lane, c = (p * 1093) >> 16;
+                if (p < DFP_PATCH) mypatch[p] = __uint_as_float(__float_as_uint(to_f32(rb[j])) & (c < cleft ? mx[j] : 0u));
+            }
         }
-        if (wide) {
+        if (FM == 3) {
+#pragma unroll
+            for (int j = 0; j < 5; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (j < 4 || lane < 32) mine[sidx[j] + i * DFP_ROW] = __uint_as_float(__float_as_uint(to_f32(rw4[j].v[i])) & mw[j]);
+        } else if (wide) {
 #pragma unroll
             for (int j = 0; j < 5; ++j)
 #pragma unroll
@@ -314,12 +349,13 @@ __global__ __launch_bounds__(512) void direct_few_pixels_kernel(const T* __restr
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const float* ar = mine + l32 * DFP_ROW + 18 * lh;
+        const float* ar = mine + l32 * DFP_ROW + (FM == 2 ? 2 : 18) * lh;
         const float* br = mypatch + 120 * lh + py * 10 + px;
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
-            a[e] = ar[e];
-            b[e] = br[(e / 9) * 60 + ((e % 9) / 3) * 10 + e % 3];
+            const int ec = FM == 2 ? e % 2 : e / 9, et = FM == 2 ? e / 2 : e % 9;       // channel (of the half's two), tap
+            a[e] = ar[FM == 2 ? 4 * et + ec : e];
+            b[e] = br[ec * 60 + (et / 3) * 10 + et % 3];
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();

@@ -822,14 +822,31 @@ bool direct_few_ok(int dtype, unsigned flags, const Geometry& g) {
            (long)g.N * g.C * g.H * g.W < (1L << 29) && (long)g.N * g.K * g.Ho * g.Wo < (1L << 29) &&
            (long)g.K * g.C * 9 < (1L << 29);                                                 // 32-bit byte offsets
 }
+// Which 16-byte pieces the filter bank offers (FM of the kernel): a [K][C][3][3] bank 1, [K][3][3][C] 2, [C][3][3][K] 3,
+// when the pieces are whole (C, for the last order also K, a multiple of 4); otherwise 0, one element per load.
+int direct_few_filter_mode(int src, const Geometry& g) {
+    if (g.C % 4) return 0;
+    if (src == WINO_NCHW) return 1;
+    if (src == WINO_NHWC) return 2;
+    return g.K % 4 ? 0 : 3;
+}
 int launch_direct_few(int src, int dst, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
                       void* y, hipStream_t st) {
     const int tiles_y = (g.Ho + 3) / 4, tiles_x = (g.Wo + 7) / 8, PT = g.N * tiles_y * tiles_x;
     const ActStrides xs = act_strides(src, g.N, g.C, g.H, g.W), ys = act_strides(dst, g.N, g.K, g.Ho, g.Wo);
     const FltStrides fs = flt_strides(src, g.K, g.C);
-    hipLaunchKernelGGL(direct_few_pixels_kernel<float>, dim3((unsigned)direct_few_units(g)), dim3(512), 0, st, (const float*)x,
-                       (const float*)w, (float*)y, xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, tiles_y, tiles_x, PT,
-                       make_epilogue(flags, bias));
+    const dim3 grid((unsigned)direct_few_units(g));
+    const Epilogue ep = make_epilogue(flags, bias);
+#define WINO_DFP(FM, XW)                                                                                                     \
+    hipLaunchKernelGGL((direct_few_pixels_kernel<float, FM, XW>), grid, dim3(512), 0, st, (const float*)x, (const float*)w, \
+                       (float*)y, xs, fs, ys, g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, tiles_y, tiles_x, PT, ep)
+    switch (direct_few_filter_mode(src, g)) {
+        case 1: WINO_DFP(1, false); break;
+        case 2: WINO_DFP(2, true); break;                  // (NHWC with C a multiple of 4: a pixel's channels in pieces as well)
+        case 3: WINO_DFP(3, false); break;
+        default: WINO_DFP(0, false); break;
+    }
+#undef WINO_DFP
     LAUNCH_CHECK("direct_few_pixels");
     return WINO_OK;
 }
@@ -1156,15 +1173,20 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
     return tiles >= 2L * device_cus();
 }
-// Small fp32 layers go to the one-launch direct kernel while its cost -- rounds of the chip times groups of 32
-// channels -- stays small (measured against the fastest Winograd pipeline, NCHW: N = 1, C = K = 64, H = 56: 8.6
-// against 17.2 us; N = 2: 13.8 against 20.4; N = 1, C = K = 128, H = 28: 11.1 against 17.3; H = 56: 21.3 against
-// 23.4; N = 1, C = K = 256, H = 28: 19.8 against 23.5; N = 4, C = K = 64, H = 56: 26.2 against 27.1; beyond that the
-// Winograd pipelines win: N = 2, C = K = 256, H = 28: 37.6 against 27.0; N = 1, C = K = 512, H = 14: 36.5 against 25.9).
-bool auto_direct_few(int dtype, unsigned flags, const Geometry& g) {
+// Small fp32 layers go to the one-launch direct kernel while its cost stays small: a round of the chip costs a fixed
+// part (the first group's trip to memory, the sum over the waves, the stores) and a part per group of 32 channels.
+// Measured against the fastest Winograd pipeline with the bank read in 16-byte pieces (times of calls issued one
+// by one from Python, about 5 us above back-to-back launches; (rounds, groups)): N = 1, C = K = 64, H = 56 (1, 2):
+// 13.5 against 19.8 us, from NHWC 12.1 against 19.9; N = 2 (2, 2): 16.8 against 23.1; N = 4 (4, 2): 29.6 against
+// 29.9, NHWC 25.3 against 26.8; N = 1, C = K = 128, H = 22 (1, 4): 13.2 against 18.6; N = 4 (2, 4): 23.5 against
+// 23.4; N = 8 (3, 4): 33.5 against 28.0; N = 4, C = K = 256, H = 14 (1, 8): 22.4 against 27.0, NHWC 26.0 against
+// 25.5; N = 8 (2, 8): 41.0 against 30.7; N = 1, C = K = 512, H = 7 (1, 16): 33.1 against 29.4; N = 8, C = K = 32,
+// H = 56 (4, 1): 22.1 against 27.8.  With one element per load (C not a multiple of 4) the kernel takes about twice
+// as long per group: N = 2, C = K = 64, H = 56 (2, 2): 32 against 22; N = 1, C = K = 128, H = 22: 26 against 19.
+bool auto_direct_few(int src, int dtype, unsigned flags, const Geometry& g) {
     if (!direct_few_ok(dtype, flags, g)) return false;
-    const long rounds = (direct_few_units(g) + device_cus() - 1) / device_cus();
-    return rounds * ((g.C + 31) / 32) <= 8;
+    const long rounds = (direct_few_units(g) + device_cus() - 1) / device_cus(), groups = (g.C + 31) / 32;
+    return direct_few_filter_mode(src, g) ? rounds * (1 + groups) <= 10 : rounds * groups <= 2;
 }
 // fp32 layers with a long reduction and enough 4x4 tiles run faster through the F(4x4,3x3) pipeline, product tensor
 // and all: 2.25 multiplies per output instead of 4, and a transformed input of 2.25x the tensor instead of 4x.
@@ -1179,23 +1201,11 @@ bool auto_f4(int dtype, const Geometry& g) {
     const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
     return tiles4 >= 512;
 }
-// which of the two F(4x4) pipelines then runs (g4: the layer's F(4x4) geometry)
-int auto_f4_algo(int dtype, const Geometry& g4) {
-    F4RowsPlan plan;
-    (void)plan;
-    (void)dtype;
-    (void)g4;
-    return WINO_ALGO_STAGED_F4;
-}
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y, bool have_w) {
     if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x, y)) return WINO_ALGO_DIRECT;
-    if (have_w && auto_direct_few(dtype, flags, g)) return WINO_ALGO_DIRECT;
-    if (have_w && auto_f4(dtype, g)) {
-        Geometry g4;
-        make_geometry(dtype, g.N, g.C, g.K, g.H, g.W, g.pad, &g4, 4);
-        return auto_f4_algo(dtype, g4);
-    }
+    if (have_w && auto_direct_few(src, dtype, flags, g)) return WINO_ALGO_DIRECT;
+    if (have_w && auto_f4(dtype, g)) return WINO_ALGO_STAGED_F4;
     const int algo = pick_algo(src, dtype, g);
     return algo == WINO_ALGO_FUSED && g.pad > 1 ? WINO_ALGO_EPILOGUE : algo;   // the single kernel masks one ring of padding
 }
@@ -1810,7 +1820,7 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
         make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g);
         make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4);
         if (L.U4) {
-            rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, auto_f4_algo(s->dtype, g4), L.flags, s->N, L.C, L.K,
+            rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, WINO_ALGO_STAGED_F4, L.flags, s->N, L.C, L.K,
                            L.H, L.W, 1, in, nullptr, L.U4, bias, out, stream);
         } else if (L.W9 && !misaligned(in, 4) && (!misaligned(out, 4) || (L.flags & WINO_FLAG_POOL2)) &&
                    auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in, out)) {
@@ -1882,7 +1892,7 @@ int wino_stack_create(int dtype, int N, int C, int H, int W, int nlayers, const 
         if (e == hipSuccess) e = hipMalloc(&L.bias, (size_t)L.K * es);
         // a copy of the bank itself for the layers AUTO may run without Winograd (C <= 4; 2-byte layers; small fp32 layers)
         const bool direct16_layer = dtype != WINO_F32 && (L.layout_in == WINO_CHWN) == (L.layout_out == WINO_CHWN) && L.C % 8 == 0;
-        if (e == hipSuccess && (L.C <= 4 || direct16_layer || auto_direct_few(dtype, L.flags, g)))
+        if (e == hipSuccess && (L.C <= 4 || direct16_layer || auto_direct_few(L.layout_in, dtype, L.flags, g)))
             e = hipMalloc(&L.wraw, (size_t)9 * L.K * L.C * es);
         // what AUTO runs outside the F(2x2) kernels gets its filters prepared once as well
         if (e == hipSuccess && L.algo == WINO_ALGO_AUTO && auto_f4(dtype, g)) {
@@ -1960,7 +1970,7 @@ int wino_stack_forward_graph(wino_stack_t* s, const void* x, void* y, void* stre
         need = std::max(need, scratch_layout(g, s->dtype).total);
         Geometry g4;
         if (L.U4 && make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g4, 4))
-            need = std::max(need, scratch_layout(g4, s->dtype, auto_f4_algo(s->dtype, g4)).total);
+            need = std::max(need, scratch_layout(g4, s->dtype, WINO_ALGO_STAGED_F4).total);
     }
     void* base = nullptr;
     int rc = arena_get(need, &base);

@@ -87,14 +87,15 @@ def test_direct_with_the_largest_filter_bank_that_fits_lds(oracle, dtype):
         assert np.array_equal(y, oracle.direct_conv(x, w, 1))
 
 
-FEW_SHAPES = [(1, 64, 64, 12, 16), (2, 7, 40, 6, 6), (1, 130, 70, 9, 11), (3, 36, 100, 13, 5), (1, 5, 33, 7, 20), (1, 8, 32, 3, 3)]
+FEW_SHAPES = [(1, 64, 64, 12, 16), (2, 7, 40, 6, 6), (1, 130, 70, 9, 11), (3, 36, 100, 13, 5), (1, 5, 33, 7, 20), (1, 8, 32, 3, 3), (2, 12, 30, 5, 9)]
 
 
 @pytest.mark.parametrize("shape", FEW_SHAPES)
 def test_fp32_layers_with_few_pixels_bit_exact_on_integers(oracle, shape):
     """direct_few_pixels_kernel: any number of channels in fp32 while the layer has few output pixels.  Channel counts
-    that are and are not multiples of 4 (16-byte and element-wise filter loads), of 32 (the waves' share of the
-    reduction), filter counts off the tile of 32, images off the 4 x 8 pixel tile, all nine layout pairs, pad 0 to 3."""
+    that are and are not multiples of 4 (16-byte and element-wise filter loads; from CHWN the pieces run along the
+    filters, so K = 30 takes the element-wise path there), of 32 (the waves' share of the reduction), filter counts off
+    the tile of 32, images off the 4 x 8 pixel tile, all nine layout pairs, pad 0 to 3."""
     N, C, K, H, W = shape
     x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
     w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
