@@ -52,6 +52,19 @@ template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
     return bf16_t{__builtin_bit_cast(uint16_t, (__bf16)f)};
 }
 
+// two values rounded to T (nearest even), a in the low half of the result
+template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b);
+template <> __device__ __forceinline__ unsigned pack2<bf16_t>(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(unsigned, __builtin_convertvector((f32x2){a, b}, bf16x2));
+}
+template <> __device__ __forceinline__ unsigned pack2<f16_t>(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(unsigned, __builtin_convertvector((f32x2){a, b}, f16x2));
+}
+
 // What the output stage applies to the 2x2 outputs of a tile before storing them:
 //     y = pool2x2( relu( conv + bias[k] ) )        (each step optional)
 // bias holds K elements of the tensor's element type.  With pool the destination has
@@ -64,6 +77,11 @@ struct Epilogue {
 };
 template <typename T> __device__ __forceinline__ float bias_of(const Epilogue& ep, int k) {
     return ep.bias ? to_f32(static_cast<const T*>(ep.bias)[k]) : 0.f;
+}
+
+// v with its lanes swapped pairwise (0 <-> 1, 2 <-> 3, ...)
+__device__ __forceinline__ float swap_lane_pairs(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
 }
 
 // v with its bits ANDed by m (m is all ones or zero).  Opaque to the optimiser on purpose:

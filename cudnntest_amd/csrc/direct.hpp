@@ -559,4 +559,205 @@ __global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restri
     }
 }
 
+// The same for NCHW tensors on both sides with an even width, as tiles.  The kernel above is bound by its memory
+// instructions twice over: it gathers a pixel's taps with sixteen 2-byte loads and stores its sums 2 bytes at a time
+// (48 memory instructions per 32 pixels x 64 filters; a CU takes about one per 16 clocks whatever its width), and the
+// 64-byte runs a wave writes per filter are half cache lines whose other half arrives from another CU: written as
+// this kernel's stores and nothing else, that pattern moves 3.5 TB/s, whole 128-byte lines 4.7 (N = 32, 224 x 224,
+// K = 64, 205 MB of y: 58 against 44 us).  Here every WAVE takes tiles of 4 rows x 64 columns, one after the
+// other, on its own:
+//   * a tile's input, C x 6 rows x 68 columns, comes in as aligned 4-byte pairs (10 loads per lane for C = 3, zeros
+//     where the padding is) and goes to LDS of the wave's own; a lane then gathers its taps with 2-byte LDS reads.
+//     The next tile's pairs are requested before the current tile's multiplies, so no wave waits for memory, and
+//     there is no workgroup barrier in the loop;
+//   * a row of the tile is two multiplies of 32 columns; the upper half of the first result and the lower half of
+//     the second change places (v_permlane32_swap), so that a register holds ONE filter for the row's 64 columns;
+//     neighbouring lanes then swap one of two sums (rounded and packed first: one DPP move, one byte permute) and
+//     every lane stores a 4-byte pair: an instruction writes two filters x 128 contiguous bytes;
+//   * the sum starts at the bias (the matrix instruction's third operand), ReLU is one instruction per value.
+// The filter bank is staged once per workgroup, as above.  Same products as above; the bias enters the sum first.
+constexpr int DSC_WR = 4;                           // output rows of a wave's tile
+constexpr int DSC_WC = 64;                          // output columns
+constexpr int DSC_PR = DSC_WR + 2;                  // input rows
+constexpr int DSC_PP = 34;                          // 4-byte pairs of an input row: 66 columns from an even one
+constexpr int dsc_loads(int ne) { return ne == 1 ? 4 : ne == 2 ? 10 : 13; }   // loads per lane of a tile's input: C = 1 (204 pairs), 2 or 3 (612), 4 (816)
+__host__ inline size_t direct16_tiles_lds_bytes(int C, int K) {
+    const size_t base = direct16_lds_bytes(C, K);
+    return base ? base + 4 * (size_t)C * DSC_PR * DSC_PP * 4 : 0;
+}
+
+template <typename T, int NE>
+__global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                     T* __restrict__ y, int N, int C, int K, int H, int W,
+                                                                     int pad, int Ho, int Wo, int tiles_y, int tiles_x,
+                                                                     int ntiles, Epilogue ep) {
+    static_assert(sizeof(T) == 2, "2-byte tensors");
+    typedef typename Mma<T>::vec vec;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem16t[];
+    const int KT = (K + 31) / 32;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int nk = 9 * C;
+    const int npairs = C * DSC_PR * DSC_PP;
+    vec* sW = reinterpret_cast<vec*>(smem16t);                                   // [KT][NE][64]
+    float* sB = reinterpret_cast<float*>(smem16t + (size_t)KT * NE * 64 * 16);  // [KT * 32] bias
+    unsigned* sP = reinterpret_cast<unsigned*>(sB + KT * 32) + wave * npairs;    // this wave's [C][6][34] pairs
+
+    for (int i = tid; i < KT * NE * 64; i += 256) {
+        const int ln = i & 63, e = (i >> 6) % NE, kt = (i >> 6) / NE;
+        const int k = kt * 32 + (ln & 31);
+        T v8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int kk = 16 * e + 8 * (ln >> 5) + j;
+            const bool ok = k < K && kk < nk;
+            const T v = w[ok ? k * nk + kk : 0];                                   // [K][C][3][3]: tap kk of filter k
+            v8[j] = ok ? v : from_f32<T>(0.f);
+        }
+        vec pk;
+        __builtin_memcpy(&pk, v8, 16);
+        sW[i] = pk;
+    }
+    for (int i = tid; i < KT * 32; i += 256) sB[i] = i < K ? bias_of<T>(ep, i) : 0.f;
+    __syncthreads();
+
+    // a lane's taps in the tile's patch: byte offset of (channel, row r, column s) relative to its pixel's first
+    // column; taps past 9 C read the pixel itself and are masked (bit 8 e + j of tapmask: a real tap)
+    int off[NE][8];
+    unsigned tapmask = 0;
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int kk = 16 * e + 8 * lh + j;
+            const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
+            off[e][j] = kk < nk ? ((c * DSC_PR + r) * DSC_PP * 2 + q) * 2 : 0;
+            tapmask |= kk < nk ? 1u << (8 * e + j) : 0u;
+        }
+    constexpr int DSC_NL = dsc_loads(NE);
+    const int rounds = (npairs + 63) / 64;                                       // wave-uniform
+    const char* xb = reinterpret_cast<const char*>(x);
+    char* yb = reinterpret_cast<char*>(y);
+    const unsigned plane_y = (unsigned)Ho * (unsigned)Wo * 2u;                    // bytes of a filter's plane of y
+    const unsigned psel = (lane & 1) ? 0x03020706u : 0x05040100u;                 // (own pair, neighbour's pair) -> what the lane stores
+
+    // the wave's tiles: every (4 x workgroups)-th, columns fastest
+    const int wstride = (int)gridDim.x * 4;
+    int tile = (int)blockIdx.x * 4 + wave;
+    int n = 0, oh0 = 0, ow0 = 0;                                                  // of the tile whose input is on its way
+    unsigned v[DSC_NL], inside = 0;                                               // bit j: pair j lies inside the image
+    auto request = [&](int t) __attribute__((always_inline)) {
+        n = t / (tiles_y * tiles_x);
+        const int trem = t - n * tiles_y * tiles_x;
+        oh0 = (trem / tiles_x) * DSC_WR;
+        ow0 = (trem - (trem / tiles_x) * tiles_x) * DSC_WC;
+        const int ic0 = ow0 - pad - ((ow0 - pad) & 1);                           // first column of the patch: even, <= ow0 - pad
+        const int base = (n * C * H + oh0 - pad) * W + ic0;
+        inside = 0;
+#pragma unroll
+        for (int j = 0; j < DSC_NL; ++j) {
+            if (j < rounds) {                                                     // (uniform)
+                // pair 64 j + lane of [C][6][34]: channel, row, pair of the row (t < 1024)
+                const int t = 64 * j + lane;
+                const int c = (t * 1286) >> 18, rem = t - c * (DSC_PR * DSC_PP);  // t / 204
+                const int rr = (rem * 1928) >> 16, pp = rem - rr * DSC_PP;         // rem / 34 (rem < 204)
+                const int ih = oh0 - pad + rr, iw = ic0 + 2 * pp;
+                const bool in = t < npairs && ih >= 0 && ih < H && iw >= 0 && iw < W;   // (W even: both elements or neither)
+                v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)((base + (c * H + rr) * W + 2 * pp) * 2) : 0u));
+                inside |= in ? 1u << j : 0u;
+            }
+        }
+    };
+    if (tile < ntiles) request(tile);
+#pragma unroll 1
+    while (tile < ntiles) {
+        const int cn = n, coh0 = oh0, cow0 = ow0;                                 // the tile to compute
+        const int shift = (cow0 - pad) & 1;
+#pragma unroll
+        for (int j = 0; j < DSC_NL; ++j)
+            if (j < rounds && 64 * j + lane < npairs) sP[64 * j + lane] = v[j] & (0u - ((inside >> j) & 1u));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        tile += wstride;
+        if (tile < ntiles) request(tile);
+
+        const int ow = cow0 + lane;                                               // the lane's column once a register holds one filter
+        const bool pok = ow < Wo;                                                 // (Wo even, ow0 even: a pair is in or out)
+#pragma unroll 1
+        for (int g = 0; g < DSC_WR; ++g) {
+            const int oh = coh0 + g;
+            if (oh >= Ho) break;                                                  // wave-uniform
+            const unsigned char* pb = reinterpret_cast<const unsigned char*>(sP) + (g * DSC_PP * 2 + l32 + shift) * 2;
+            vec b[2][NE];                                                         // columns 0 .. 31 and 32 .. 63
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int e = 0; e < NE; ++e) {
+                    unsigned short raw[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        raw[j] = (unsigned short)(*reinterpret_cast<const unsigned short*>(pb + 64 * h + off[e][j]) & (0u - ((tapmask >> (8 * e + j)) & 1u)));
+                    __builtin_memcpy(&b[h][e], raw, 16);
+                }
+            // the lane's pair: columns ow & ~1 and the next one, of the filter it keeps (even lanes the first of two)
+            const unsigned yq = (unsigned)(((cn * K + (lane & 1)) * Ho + oh) * Wo + (ow & ~1)) * 2u;
+#pragma unroll 1
+            for (int kt = 0; kt < KT; ++kt) {
+                // register r of a lane: filter 8 (r / 4) + 4 lh + r % 4 of the tile; the sum starts at the bias
+                floatx16 acc[2];
+                const float* bk = sB + kt * 32 + 4 * lh;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const floatx4 bq = *reinterpret_cast<const floatx4*>(bk + 8 * q);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[0][4 * q + r] = acc[1][4 * q + r] = bq[r];
+                }
+                const vec* wk = sW + (size_t)kt * NE * 64 + lane;
+#pragma unroll
+                for (int e = 0; e < NE; ++e) {
+                    const vec a = wk[e * 64];
+                    Mma<T>::run(a, b[0][e], acc[0]);
+                    Mma<T>::run(a, b[1][e], acc[1]);
+                }
+                // registers 2i and 2i + 1 of half u (after the exchange of halves) are filters f and f + 1,
+                // f = 8 (i / 2) + 4 u + 2 (i % 2), for the row's 64 columns: rounded, packed, swapped with the
+                // neighbouring lane, and each lane keeps the two columns of one filter
+                auto put = [&](int i, bool check, bool relu) __attribute__((always_inline)) {
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[0][2 * i]), __float_as_uint(acc[1][2 * i]), false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[0][2 * i + 1]), __float_as_uint(acc[1][2 * i + 1]), false, false);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        float a0 = __uint_as_float(s0[u]), a1 = __uint_as_float(s1[u]);
+                        if (relu) {                                                // max(a, 0), 0 for a NaN (as fmaxf)
+                            asm("v_max_f32_e32 %0, 0, %1" : "=v"(a0) : "v"(a0));
+                            asm("v_max_f32_e32 %0, 0, %1" : "=v"(a1) : "v"(a1));
+                        }
+                        const unsigned own = pack2<T>(a0, a1);
+                        const unsigned nb = (unsigned)__builtin_amdgcn_mov_dpp((int)own, 0xB1, 0xF, 0xF, true);
+                        const unsigned out = __builtin_amdgcn_perm(nb, own, psel);
+                        const int f = kt * 32 + 8 * (i >> 1) + 4 * u + 2 * (i & 1);
+                        if (pok && (!check || f + (lane & 1) < K)) *reinterpret_cast<unsigned*>(yb + (yq + (unsigned)f * plane_y)) = out;
+                    }
+                };
+                // (every lane takes part in the exchanges; only the stores are conditional)
+                if (kt * 32 + 32 > K) {                                           // (wave-uniform: the bank's last, partial tile)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) put(i, true, ep.relu != 0);
+                } else if (ep.relu) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) put(i, false, true);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) put(i, false, false);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                   // (the tile's LDS reads before the next tile's writes)
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 }  // namespace wino

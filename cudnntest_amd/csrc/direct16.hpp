@@ -104,10 +104,6 @@ __global__ __launch_bounds__(64) void direct16_pack_kernel(const T* __restrict__
     }
 }
 
-// v with its lanes swapped pairwise (0 <-> 1, 2 <-> 3, ...)
-__device__ __forceinline__ float swap_lane_pairs(float v) {
-    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
-}
 
 // ROWS: the block is 16 rows x 32 columns (PW = 34), every wave owns 4 consecutive output rows of one image
 // (the host offers it when Ho is a multiple of 4), so pixel group j, filter row r reads input row j + r of the

@@ -35,6 +35,36 @@ def test_integers_bit_exact(oracle, shape, dtype):
             assert np.array_equal(host(got), want), (pad, src, dst)
 
 
+TILE_SHAPES = [(2, 3, 64, 40, 70), (1, 4, 70, 18, 34), (3, 1, 33, 17, 32), (2, 2, 40, 33, 66), (5, 3, 64, 16, 2)]
+
+
+@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", TILE_SHAPES)
+def test_two_byte_nchw_layers_as_tiles_bit_exact(oracle, shape, dtype):
+    """2-byte NCHW tensors with an even width run as tiles of 16 rows x 32 columns (input through LDS, 4-byte pairs
+    stored): several tiles each way with ragged last ones, one to four channels, filter counts off the tile of 32,
+    pad 0 and 1 (the patch starts at an even or an odd column), with and without bias and ReLU; a view that is only
+    2-byte aligned takes the gathering kernel and gives the same bits."""
+    N, C, K, H, W = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    for pad in (1, 0):
+        if H + 2 * pad < 3 or W + 2 * pad < 3:
+            continue
+        plain = oracle.direct_conv(x, w, pad)
+        got = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT)
+        assert np.array_equal(host(got), plain), pad
+        want = np.maximum(plain + bias[None, :, None, None], 0).astype(np.float32)
+        got = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
+        assert np.array_equal(host(got), want), pad
+        xd = dev(x, dtype)
+        shifted = torch.empty(xd.numel() + 1, dtype=xd.dtype, device="cuda")[1:].view(xd.shape)
+        shifted.copy_(xd)
+        got2 = ops.conv(shifted, dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
+        assert torch.equal(got2, got), pad
+
+
 @pytest.mark.parametrize("dtype", [ops.F32, ops.BF16])
 @pytest.mark.parametrize("layout", DST)
 def test_floats_within_tolerance_and_auto_takes_the_path(oracle, layout, dtype):
