@@ -760,4 +760,191 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
     }
 }
 
+// The same for NHWC tensors on both sides (K even): y is then a matrix [pixel][filter] whose rows are K contiguous
+// elements, and the gathering kernel writes it two bytes per lane, 64 bytes per pixel and instruction.  Per wave and
+// tile of 4 rows x 32 columns, as above; the differences:
+//   * an input row of a tile is ONE contiguous run of (32 + 2) x C elements: C x 17 + 1 aligned pairs a row (the run
+//     may start at an odd element; a row of the image starts and ends at an even one, so no pair straddles its edge);
+//   * the taps of a multiply are in the bank's order (tap major, channel minor: [K][3][3][C]), the pixels are the
+//     first operand, so a lane holds one filter and its registers the pixels;
+//   * two filter tiles are multiplied at a time; the upper half of the first result and the lower half of the second
+//     change places (v_permlane32_swap), so that a register holds ONE pixel for 64 filters; neighbouring lanes then
+//     swap one of two sums and every lane stores a 4-byte pair: an instruction writes the 64 filters of two
+//     neighbouring pixels, 256 contiguous bytes when K = 64.
+// Bias after the sum, as in the gathering kernel: same bits.
+constexpr int dsc_nhwc_loads(int ne) { return ne == 1 ? 2 : ne == 2 ? 5 : 7; }   // loads per lane of a tile's input: C = 1 (108 pairs), 2 or 3 (312), 4 (414)
+__host__ inline size_t direct16_tiles_nhwc_lds_bytes(int C, int K) {
+    const size_t base = direct16_lds_bytes(C, K + 32);                           // (filter tiles in pairs: one more when their number is odd)
+    return base ? base + 4 * (size_t)DSC_PR * (17 * C + 1) * 4 : 0;
+}
+
+template <typename T, int NE>
+__global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                          T* __restrict__ y, int N, int C, int K, int H,
+                                                                          int W, int pad, int Ho, int Wo, int tiles_y,
+                                                                          int tiles_x, int ntiles, Epilogue ep) {
+    static_assert(sizeof(T) == 2, "2-byte tensors");
+    typedef typename Mma<T>::vec vec;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem16n[];
+    const int KT2 = (K + 63) / 64;                                               // pairs of filter tiles
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int nk = 9 * C;
+    const int PPN = 17 * C + 1;                                                  // pairs of an input row of a tile
+    const int npairs = DSC_PR * PPN;
+    vec* sW = reinterpret_cast<vec*>(smem16n);                                   // [2 KT2][NE][64]
+    float* sB = reinterpret_cast<float*>(smem16n + (size_t)2 * KT2 * NE * 64 * 16);   // [64 KT2] bias
+    unsigned* sP = reinterpret_cast<unsigned*>(sB + KT2 * 64) + wave * npairs;   // this wave's [6][PPN] pairs
+
+    for (int i = tid; i < 2 * KT2 * NE * 64; i += 256) {
+        const int ln = i & 63, e = (i >> 6) % NE, kt = (i >> 6) / NE;
+        const int k = kt * 32 + (ln & 31);
+        T v8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int kk = 16 * e + 8 * (ln >> 5) + j;
+            const bool ok = k < K && kk < nk;
+            const T v = w[ok ? k * nk + kk : 0];                                   // [K][3][3][C]: element kk of filter k
+            v8[j] = ok ? v : from_f32<T>(0.f);
+        }
+        vec pk;
+        __builtin_memcpy(&pk, v8, 16);
+        sW[i] = pk;
+    }
+    for (int i = tid; i < KT2 * 64; i += 256) sB[i] = i < K ? bias_of<T>(ep, i) : 0.f;
+    __syncthreads();
+
+    // a lane's taps in the tile's patch: element kk = (3 r + s) C + c of a filter meets the input at row r, element
+    // s C + c past the pixel's first: byte offset relative to that; taps past 9 C read the pixel itself and are masked
+    int off[NE][8];
+    unsigned tapmask = 0;
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int kk = 16 * e + 8 * lh + j;
+            const int r = kk / (3 * C), rem = kk - r * 3 * C;
+            off[e][j] = kk < nk ? (r * PPN * 2 + rem) * 2 : 0;
+            tapmask |= kk < nk ? 1u << (8 * e + j) : 0u;
+        }
+    // the patch as loaded: pair 64 j + lane of [6][PPN], as row | pair of the row << 8 (row 255, never inside, past it)
+    constexpr int NL = dsc_nhwc_loads(NE);
+    unsigned prp[NL];
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const int t = 64 * j + lane;
+        const int rr = t / PPN, pp = t - rr * PPN;
+        prp[j] = t < npairs ? (unsigned)(rr | pp << 8) : 0xFFu;
+    }
+    const int rounds = (npairs + 63) / 64;                                       // wave-uniform
+    const char* xb = reinterpret_cast<const char*>(x);
+    char* yb = reinterpret_cast<char*>(y);
+    const unsigned psel = (lane & 1) ? 0x03020706u : 0x05040100u;                 // (own pair, neighbour's pair) -> what the lane stores
+    const int WC = W * C;                                                         // elements of an image row (even)
+
+    const int wstride = (int)gridDim.x * 4;
+    int tile = (int)blockIdx.x * 4 + wave;
+    int n = 0, oh0 = 0, ow0 = 0;                                                  // of the tile whose input is on its way
+    unsigned v[NL], inside = 0;                                                   // bit j: pair j lies inside the image
+    auto request = [&](int t) __attribute__((always_inline)) {
+        n = t / (tiles_y * tiles_x);
+        const int trem = t - n * tiles_y * tiles_x;
+        oh0 = (trem / tiles_x) * DSC_WR;
+        ow0 = (trem - (trem / tiles_x) * tiles_x) * 32;
+        const int e0 = (ow0 - pad) * C - (((ow0 - pad) * C) & 1);                // first element of the patch's rows: even
+        const int base = (n * H + oh0 - pad) * WC + e0;
+        inside = 0;
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            if (j < rounds) {                                                     // (uniform)
+                const int rr = prp[j] & 0xFF, pp = prp[j] >> 8;
+                const int ih = oh0 - pad + rr, ie = e0 + 2 * pp;
+                const bool in = ih >= 0 && ih < H && ie >= 0 && ie < WC;          // (a row starts and ends at an even element)
+                v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)((base + rr * WC + 2 * pp) * 2) : 0u));
+                inside |= in ? 1u << j : 0u;
+            }
+        }
+    };
+    if (tile < ntiles) request(tile);
+#pragma unroll 1
+    while (tile < ntiles) {
+        const int cn = n, coh0 = oh0, cow0 = ow0;                                 // the tile to compute
+        const int shift = ((cow0 - pad) * C) & 1;
+#pragma unroll
+        for (int j = 0; j < NL; ++j)
+            if (j < rounds && 64 * j + lane < npairs) sP[64 * j + lane] = v[j] & (0u - ((inside >> j) & 1u));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        tile += wstride;
+        if (tile < ntiles) request(tile);
+
+#pragma unroll 1
+        for (int g = 0; g < DSC_WR; ++g) {
+            const int oh = coh0 + g;
+            if (oh >= Ho) break;                                                  // wave-uniform
+            const unsigned char* pb = reinterpret_cast<const unsigned char*>(sP) + (g * PPN * 2 + l32 * C + shift) * 2;
+            vec a[NE];                                                            // the pixels' taps
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                unsigned short raw[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    raw[j] = (unsigned short)(*reinterpret_cast<const unsigned short*>(pb + off[e][j]) & (0u - ((tapmask >> (8 * e + j)) & 1u)));
+                __builtin_memcpy(&a[e], raw, 16);
+            }
+            // after the exchanges a lane keeps filters (lane & ~1, + 1) of one pixel: even lanes the pixel of the
+            // even register, odd lanes the next one
+            const unsigned yrow = (unsigned)((cn * Ho + oh) * Wo + cow0) * (unsigned)K * 2u + (unsigned)(lane & ~1) * 2u;
+#pragma unroll 1
+            for (int kp = 0; kp < KT2; ++kp) {
+                // register r of a lane: pixel 8 (r / 4) + 4 lh + r % 4 of the row's 32, filter 32 (2 kp + u) + l32
+                floatx16 acc[2];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = 0.f;
+                const vec* wk = sW + (size_t)(2 * kp) * NE * 64 + lane;
+#pragma unroll
+                for (int e = 0; e < NE; ++e) {
+                    Mma<T>::run(a[e], wk[e * 64], acc[0]);
+                    Mma<T>::run(a[e], wk[(NE + e) * 64], acc[1]);
+                }
+                const float bl = sB[kp * 64 + lane];                               // the bias of the filter the lane holds after the exchange
+                const bool kok = kp * 64 + (lane | 1) < K;                          // (K even: the lane's two filters exist together)
+                // registers 2i and 2i + 1 of half u (after the exchange of halves) are pixels p and p + 1,
+                // p = 8 (i / 2) + 4 u + 2 (i % 2), for 64 filters
+                auto put = [&](int i, bool relu) __attribute__((always_inline)) {
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[0][2 * i]), __float_as_uint(acc[1][2 * i]), false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[0][2 * i + 1]), __float_as_uint(acc[1][2 * i + 1]), false, false);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        float a0 = __uint_as_float(s0[u]) + bl, a1 = __uint_as_float(s1[u]) + bl;
+                        if (relu) {                                                // max(a, 0), 0 for a NaN (as fmaxf)
+                            asm("v_max_f32_e32 %0, 0, %1" : "=v"(a0) : "v"(a0));
+                            asm("v_max_f32_e32 %0, 0, %1" : "=v"(a1) : "v"(a1));
+                        }
+                        const unsigned own = pack2<T>(a0, a1);
+                        const unsigned nb = (unsigned)__builtin_amdgcn_mov_dpp((int)own, 0xB1, 0xF, 0xF, true);
+                        const unsigned out = __builtin_amdgcn_perm(nb, own, psel);
+                        const int p = 8 * (i >> 1) + 4 * u + 2 * (i & 1);           // (Wo even: pixels p and p + 1 exist together)
+                        if (kok && cow0 + p < Wo)
+                            *reinterpret_cast<unsigned*>(yb + (yrow + (unsigned)(p + (lane & 1)) * (unsigned)K * 2u + (unsigned)(kp * 128))) = out;
+                    }
+                };
+                // (every lane takes part in the exchanges; only the stores are conditional)
+                if (ep.relu) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) put(i, true);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) put(i, false);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                   // (the tile's LDS reads before the next tile's writes)
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 }  // namespace wino

@@ -805,6 +805,27 @@ int launch_direct_t(int src, int dst, unsigned flags, const void* bias, const Ge
             LAUNCH_CHECK("direct_small_c16_tiles");
             return WINO_OK;
         }
+        if (src == WINO_NHWC && dst == WINO_NHWC && g.W % 2 == 0 && g.K % 2 == 0 && !misaligned(x, 4) && !misaligned(y, 4) &&
+            direct16_tiles_nhwc_lds_bytes(g.C, g.K) <= 64 * 1024) {
+            // NHWC on both sides, rows and pixels of whole 4-byte pairs: tiles of 4 rows x 32 columns per wave, input
+            // through LDS, the 64 filters of two neighbouring pixels stored per instruction
+            const int tiles_y = (g.Ho + DSC_WR - 1) / DSC_WR, tiles_x = (g.Wo + 31) / 32;
+            const long ntiles = (long)g.N * tiles_y * tiles_x, resident = 8L * device_cus();
+            const long per = (ntiles + resident - 1) / resident;                 // tiles per wave
+            const dim3 tgrid((unsigned)((ntiles + 4 * per - 1) / (4 * per)));
+            const size_t ldst = direct16_tiles_nhwc_lds_bytes(g.C, g.K);
+#define DIRECT16_TILES(NE)                                                                                                   \
+    hipLaunchKernelGGL((direct_small_c16_tiles_nhwc_kernel<T, NE>), tgrid, block, ldst, st, (const T*)x, (const T*)w, (T*)y, g.N, \
+                       g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, tiles_y, tiles_x, (int)ntiles, ep)
+            switch (g.C) {
+            case 1: DIRECT16_TILES(1); break;
+            case 4: DIRECT16_TILES(3); break;
+            default: DIRECT16_TILES(2); break;
+            }
+#undef DIRECT16_TILES
+            LAUNCH_CHECK("direct_small_c16_tiles_nhwc");
+            return WINO_OK;
+        }
 #define DIRECT16_LAUNCH(NE)                                                                                          \
     if (dst == WINO_NHWC)                                                                                           \
         hipLaunchKernelGGL((direct_small_c16_kernel<T, NE, true>), grid, block, lds16, st, (const T*)x, (const T*)w, \

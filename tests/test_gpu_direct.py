@@ -35,33 +35,37 @@ def test_integers_bit_exact(oracle, shape, dtype):
             assert np.array_equal(host(got), want), (pad, src, dst)
 
 
-TILE_SHAPES = [(2, 3, 64, 40, 70), (1, 4, 70, 18, 34), (3, 1, 33, 17, 32), (2, 2, 40, 33, 66), (5, 3, 64, 16, 2)]
+TILE_SHAPES = [(2, 3, 64, 40, 70), (1, 4, 70, 18, 34), (3, 1, 33, 17, 32), (2, 2, 40, 33, 66), (5, 3, 64, 16, 2), (1, 3, 130, 9, 36)]
 
 
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC])
 @pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
 @pytest.mark.parametrize("shape", TILE_SHAPES)
-def test_two_byte_nchw_layers_as_tiles_bit_exact(oracle, shape, dtype):
-    """2-byte NCHW tensors with an even width run as tiles of 16 rows x 32 columns (input through LDS, 4-byte pairs
-    stored): several tiles each way with ragged last ones, one to four channels, filter counts off the tile of 32,
-    pad 0 and 1 (the patch starts at an even or an odd column), with and without bias and ReLU; a view that is only
-    2-byte aligned takes the gathering kernel and gives the same bits."""
+def test_two_byte_layers_as_tiles_bit_exact(oracle, shape, dtype, layout):
+    """2-byte NCHW (NHWC) tensors with an even width (and an even K) run as tiles of 4 rows x 64 (32) columns per wave
+    (input through LDS, sums exchanged between lanes, 4-byte pairs stored): several tiles each way with ragged last
+    ones, one to four channels, filter counts off the tile of 32 (K = 33 from NHWC: the gathering kernel), pad 0 and 1
+    (the patch starts at an even or an odd element), with and without bias and ReLU; a view that is only 2-byte
+    aligned takes the gathering kernel and gives the same bits."""
     N, C, K, H, W = shape
     x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
     w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
     bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    xs, ws = synth.act_to_layout(x, layout), synth.flt_to_layout(w, layout)
     for pad in (1, 0):
         if H + 2 * pad < 3 or W + 2 * pad < 3:
             continue
-        plain = oracle.direct_conv(x, w, pad)
-        got = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT)
+        plain = oracle.direct_conv(xs, ws, pad, layout, layout)
+        got = ops.conv(dev(xs, dtype), dev(ws, dtype), pad, layout, algo=ops.ALGO_DIRECT)
         assert np.array_equal(host(got), plain), pad
-        want = np.maximum(plain + bias[None, :, None, None], 0).astype(np.float32)
-        got = ops.conv(dev(x, dtype), dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
+        want = np.maximum(synth.act_from_layout(plain, layout) + bias[None, :, None, None], 0).astype(np.float32)
+        want = synth.act_to_layout(np.ascontiguousarray(want), layout)
+        got = ops.conv(dev(xs, dtype), dev(ws, dtype), pad, layout, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
         assert np.array_equal(host(got), want), pad
-        xd = dev(x, dtype)
+        xd = dev(xs, dtype)
         shifted = torch.empty(xd.numel() + 1, dtype=xd.dtype, device="cuda")[1:].view(xd.shape)
         shifted.copy_(xd)
-        got2 = ops.conv(shifted, dev(w, dtype), pad, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
+        got2 = ops.conv(shifted, dev(ws, dtype), pad, layout, algo=ops.ALGO_DIRECT, relu=True, bias=dev(bias, dtype))
         assert torch.equal(got2, got), pad
 
 
