@@ -511,9 +511,10 @@ __global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restri
         const unsigned yq = (unsigned)(n * ys.n + oh * ys.h + ow * ys.w + 4 * lh * ys.c);
 #pragma unroll 1
         for (int kt = 0; kt < KT; ++kt) {
+            // the sum starts at the bias (SWAP: a lane holds one filter; else register r is filter 8 (r / 4) + 4 lh + r % 4)
             floatx16 acc;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            for (int r = 0; r < 16; ++r) acc[r] = SWAP ? sB[kt * 32 + l32] : sB[kt * 32 + 8 * (r >> 2) + (r & 3) + 4 * lh];
             const vec* wk = sW + (size_t)kt * NE * 64 + lane;
             vec a[NE];
 #pragma unroll
@@ -525,24 +526,20 @@ __global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restri
             }
             if (SWAP) {
                 const int k = kt * 32 + l32;
-                const float bk = sB[k];
                 if (k < K) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const long pq = q0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                        float v = acc[r] + bk;
+                        float v = acc[r];
                         if (ep.relu) v = fmaxf(v, 0.f);
                         if (pq < Q) y[pq * K + k] = from_f32<T>(v);
                     }
                 }
                 continue;
             }
-            float bv[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) bv[r] = sB[kt * 32 + 8 * (r >> 2) + (r & 3) + 4 * lh];
             const T* yk = y + (size_t)kt * 32 * ys.c;
             auto put = [&](int r) {
-                float v = acc[r] + bv[r];
+                float v = acc[r];
                 if (ep.relu) v = fmaxf(v, 0.f);
                 const_cast<T*>(yk + (size_t)(8 * (r >> 2) + (r & 3)) * ys.c)[yq] = from_f32<T>(v);
             };
@@ -575,22 +572,27 @@ __global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restri
 //     neighbouring lanes then swap one of two sums (rounded and packed first: one DPP move, one byte permute) and
 //     every lane stores a 4-byte pair: an instruction writes two filters x 128 contiguous bytes;
 //   * the sum starts at the bias (the matrix instruction's third operand), ReLU is one instruction per value.
-// The filter bank is staged once per workgroup, as above.  Same products as above; the bias enters the sum first.
+// The filter bank is staged once per workgroup, as above.  Same products and the same bits as above.
+// DIL: CHWN tensors ([C][H][W][N], filters [C][3][3][K]) as ONE image of width W * N whose taps are N columns apart:
+// the batch is the contiguous axis of both tensors, so a row of 64 "columns" is two pixels x 32 images (N = 32), the
+// zero padding is pad * N columns wide, and everything else is the NCHW kernel.
 constexpr int DSC_WR = 4;                           // output rows of a wave's tile
 constexpr int DSC_WC = 64;                          // output columns
 constexpr int DSC_PR = DSC_WR + 2;                  // input rows
 constexpr int DSC_PP = 34;                          // 4-byte pairs of an input row: 66 columns from an even one
-constexpr int dsc_loads(int ne) { return ne == 1 ? 4 : ne == 2 ? 10 : 13; }   // loads per lane of a tile's input: C = 1 (204 pairs), 2 or 3 (612), 4 (816)
-__host__ inline size_t direct16_tiles_lds_bytes(int C, int K) {
+constexpr int DSC_DS = 32;                          // DIL: columns between taps, at most
+// loads per lane of a tile's input: C = 1 (204 pairs), 2 or 3 (612), 4 (816); DIL: rows of up to 33 + 32 pairs
+constexpr int dsc_loads(int ne, bool dil) { return dil ? (ne == 1 ? 7 : ne == 2 ? 19 : 25) : (ne == 1 ? 4 : ne == 2 ? 10 : 13); }
+__host__ inline size_t direct16_tiles_lds_bytes(int C, int K, int ds = 1) {
     const size_t base = direct16_lds_bytes(C, K);
-    return base ? base + 4 * (size_t)C * DSC_PR * DSC_PP * 4 : 0;
+    return base ? base + 4 * (size_t)C * DSC_PR * (33 + ds) * 4 : 0;
 }
 
-template <typename T, int NE>
+template <typename T, int NE, bool DIL>
 __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                                      T* __restrict__ y, int N, int C, int K, int H, int W,
-                                                                     int pad, int Ho, int Wo, int tiles_y, int tiles_x,
-                                                                     int ntiles, Epilogue ep) {
+                                                                     int pad, int ds, int Ho, int Wo, int tiles_y,
+                                                                     int tiles_x, int ntiles, Epilogue ep) {
     static_assert(sizeof(T) == 2, "2-byte tensors");
     typedef typename Mma<T>::vec vec;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem16t[];
@@ -600,7 +602,9 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
     const int nk = 9 * C;
-    const int npairs = C * DSC_PR * DSC_PP;
+    const int PP = DIL ? 33 + ds : DSC_PP;                                       // pairs of an input row of a tile: 64 + 2 ds columns from an even one
+    const int padw = pad * ds;                                                   // zero columns left of a row
+    const int npairs = C * DSC_PR * PP;
     vec* sW = reinterpret_cast<vec*>(smem16t);                                   // [KT][NE][64]
     float* sB = reinterpret_cast<float*>(smem16t + (size_t)KT * NE * 64 * 16);  // [KT * 32] bias
     unsigned* sP = reinterpret_cast<unsigned*>(sB + KT * 32) + wave * npairs;    // this wave's [C][6][34] pairs
@@ -613,7 +617,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
         for (int j = 0; j < 8; ++j) {
             const int kk = 16 * e + 8 * (ln >> 5) + j;
             const bool ok = k < K && kk < nk;
-            const T v = w[ok ? k * nk + kk : 0];                                   // [K][C][3][3]: tap kk of filter k
+            const T v = w[ok ? (DIL ? kk * K + k : k * nk + kk) : 0];              // [K][C][3][3] (DIL: [C][3][3][K]): tap kk of filter k
             v8[j] = ok ? v : from_f32<T>(0.f);
         }
         vec pk;
@@ -633,10 +637,22 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
         for (int j = 0; j < 8; ++j) {
             const int kk = 16 * e + 8 * lh + j;
             const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
-            off[e][j] = kk < nk ? ((c * DSC_PR + r) * DSC_PP * 2 + q) * 2 : 0;
+            off[e][j] = kk < nk ? ((c * DSC_PR + r) * PP * 2 + q * ds) * 2 : 0;
             tapmask |= kk < nk ? 1u << (8 * e + j) : 0u;
         }
-    constexpr int DSC_NL = dsc_loads(NE);
+    constexpr int DSC_NL = dsc_loads(NE, DIL);
+    // DIL: the patch as loaded, pair 64 j + lane of [C][6][PP], as channel | row << 4 | pair of the row << 8 (row 15,
+    // never inside the image, past the patch)
+    unsigned pd[DIL ? DSC_NL : 1];
+    if (DIL) {
+#pragma unroll
+        for (int j = 0; j < DSC_NL; ++j) {
+            const int t = 64 * j + lane;
+            const int c = t / (DSC_PR * PP), rem = t - c * (DSC_PR * PP);
+            const int rr = rem / PP, pp = rem - rr * PP;
+            pd[j] = t < npairs ? (unsigned)(c | rr << 4 | pp << 8) : 0xF0u;
+        }
+    }
     const int rounds = (npairs + 63) / 64;                                       // wave-uniform
     const char* xb = reinterpret_cast<const char*>(x);
     char* yb = reinterpret_cast<char*>(y);
@@ -653,7 +669,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
         const int trem = t - n * tiles_y * tiles_x;
         oh0 = (trem / tiles_x) * DSC_WR;
         ow0 = (trem - (trem / tiles_x) * tiles_x) * DSC_WC;
-        const int ic0 = ow0 - pad - ((ow0 - pad) & 1);                           // first column of the patch: even, <= ow0 - pad
+        const int ic0 = ow0 - padw - ((ow0 - padw) & 1);                         // first column of the patch: even, <= ow0 - padw
         const int base = (n * C * H + oh0 - pad) * W + ic0;
         inside = 0;
 #pragma unroll
@@ -661,8 +677,13 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
             if (j < rounds) {                                                     // (uniform)
                 // pair 64 j + lane of [C][6][34]: channel, row, pair of the row (t < 1024)
                 const int t = 64 * j + lane;
-                const int c = (t * 1286) >> 18, rem = t - c * (DSC_PR * DSC_PP);  // t / 204
-                const int rr = (rem * 1928) >> 16, pp = rem - rr * DSC_PP;         // rem / 34 (rem < 204)
+                int c = (t * 1286) >> 18, rem = t - c * (DSC_PR * DSC_PP);        // t / 204
+                int rr = (rem * 1928) >> 16, pp = rem - rr * DSC_PP;               // rem / 34 (rem < 204)
+                if (DIL) {
+                    c = pd[j] & 15;
+                    rr = (pd[j] >> 4) & 15;
+                    pp = pd[j] >> 8;
+                }
                 const int ih = oh0 - pad + rr, iw = ic0 + 2 * pp;
                 const bool in = t < npairs && ih >= 0 && ih < H && iw >= 0 && iw < W;   // (W even: both elements or neither)
                 v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)((base + (c * H + rr) * W + 2 * pp) * 2) : 0u));
@@ -674,7 +695,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
 #pragma unroll 1
     while (tile < ntiles) {
         const int cn = n, coh0 = oh0, cow0 = ow0;                                 // the tile to compute
-        const int shift = (cow0 - pad) & 1;
+        const int shift = (cow0 - padw) & 1;
 #pragma unroll
         for (int j = 0; j < DSC_NL; ++j)
             if (j < rounds && 64 * j + lane < npairs) sP[64 * j + lane] = v[j] & (0u - ((inside >> j) & 1u));
@@ -690,7 +711,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
         for (int g = 0; g < DSC_WR; ++g) {
             const int oh = coh0 + g;
             if (oh >= Ho) break;                                                  // wave-uniform
-            const unsigned char* pb = reinterpret_cast<const unsigned char*>(sP) + (g * DSC_PP * 2 + l32 + shift) * 2;
+            const unsigned char* pb = reinterpret_cast<const unsigned char*>(sP) + (g * PP * 2 + l32 + shift) * 2;
             vec b[2][NE];                                                         // columns 0 .. 31 and 32 .. 63
 #pragma unroll
             for (int h = 0; h < 2; ++h)
@@ -765,13 +786,12 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
 // tile of 4 rows x 32 columns, as above; the differences:
 //   * an input row of a tile is ONE contiguous run of (32 + 2) x C elements: C x 17 + 1 aligned pairs a row (the run
 //     may start at an odd element; a row of the image starts and ends at an even one, so no pair straddles its edge);
-//   * the taps of a multiply are in the bank's order (tap major, channel minor: [K][3][3][C]), the pixels are the
-//     first operand, so a lane holds one filter and its registers the pixels;
+//   * the pixels are the first operand of a multiply, so a lane holds one filter and its registers the pixels;
 //   * two filter tiles are multiplied at a time; the upper half of the first result and the lower half of the second
 //     change places (v_permlane32_swap), so that a register holds ONE pixel for 64 filters; neighbouring lanes then
 //     swap one of two sums and every lane stores a 4-byte pair: an instruction writes the 64 filters of two
 //     neighbouring pixels, 256 contiguous bytes when K = 64.
-// Bias after the sum, as in the gathering kernel: same bits.
+// The sums start at the bias, as in the gathering kernel: same bits.
 constexpr int dsc_nhwc_loads(int ne) { return ne == 1 ? 2 : ne == 2 ? 5 : 7; }   // loads per lane of a tile's input: C = 1 (108 pairs), 2 or 3 (312), 4 (414)
 __host__ inline size_t direct16_tiles_nhwc_lds_bytes(int C, int K) {
     const size_t base = direct16_lds_bytes(C, K + 32);                           // (filter tiles in pairs: one more when their number is odd)
@@ -806,7 +826,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const 
         for (int j = 0; j < 8; ++j) {
             const int kk = 16 * e + 8 * (ln >> 5) + j;
             const bool ok = k < K && kk < nk;
-            const T v = w[ok ? k * nk + kk : 0];                                   // [K][3][3][C]: element kk of filter k
+            const T v = w[ok ? k * nk + (kk % 9) * C + kk / 9 : 0];                 // [K][3][3][C]: tap kk = 9 c + 3 r + s of filter k
             v8[j] = ok ? v : from_f32<T>(0.f);
         }
         vec pk;
@@ -816,8 +836,9 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const 
     for (int i = tid; i < KT2 * 64; i += 256) sB[i] = i < K ? bias_of<T>(ep, i) : 0.f;
     __syncthreads();
 
-    // a lane's taps in the tile's patch: element kk = (3 r + s) C + c of a filter meets the input at row r, element
-    // s C + c past the pixel's first: byte offset relative to that; taps past 9 C read the pixel itself and are masked
+    // a lane's taps in the tile's patch, in the gathering kernel's order: tap kk = 9 c + 3 r + s meets the input at
+    // row r, element s C + c past the pixel's first: byte offset relative to that; taps past 9 C read the pixel itself
+    // and are masked
     int off[NE][8];
     unsigned tapmask = 0;
 #pragma unroll
@@ -825,8 +846,8 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const 
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int kk = 16 * e + 8 * lh + j;
-            const int r = kk / (3 * C), rem = kk - r * 3 * C;
-            off[e][j] = kk < nk ? (r * PPN * 2 + rem) * 2 : 0;
+            const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
+            off[e][j] = kk < nk ? (r * PPN * 2 + q * C + c) * 2 : 0;
             tapmask |= kk < nk ? 1u << (8 * e + j) : 0u;
         }
     // the patch as loaded: pair 64 j + lane of [6][PPN], as row | pair of the row << 8 (row 255, never inside, past it)
@@ -901,16 +922,19 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const 
 #pragma unroll 1
             for (int kp = 0; kp < KT2; ++kp) {
                 // register r of a lane: pixel 8 (r / 4) + 4 lh + r % 4 of the row's 32, filter 32 (2 kp + u) + l32
+                // (the sums start at the bias of the lane's filter)
                 floatx16 acc[2];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = 0.f;
+                for (int r = 0; r < 16; ++r) {
+                    acc[0][r] = sB[kp * 64 + l32];
+                    acc[1][r] = sB[kp * 64 + 32 + l32];
+                }
                 const vec* wk = sW + (size_t)(2 * kp) * NE * 64 + lane;
 #pragma unroll
                 for (int e = 0; e < NE; ++e) {
                     Mma<T>::run(a[e], wk[e * 64], acc[0]);
                     Mma<T>::run(a[e], wk[(NE + e) * 64], acc[1]);
                 }
-                const float bl = sB[kp * 64 + lane];                               // the bias of the filter the lane holds after the exchange
                 const bool kok = kp * 64 + (lane | 1) < K;                          // (K even: the lane's two filters exist together)
                 // registers 2i and 2i + 1 of half u (after the exchange of halves) are pixels p and p + 1,
                 // p = 8 (i / 2) + 4 u + 2 (i % 2), for 64 filters
@@ -919,7 +943,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const 
                     const auto s1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[0][2 * i + 1]), __float_as_uint(acc[1][2 * i + 1]), false, false);
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
-                        float a0 = __uint_as_float(s0[u]) + bl, a1 = __uint_as_float(s1[u]) + bl;
+                        float a0 = __uint_as_float(s0[u]), a1 = __uint_as_float(s1[u]);
                         if (relu) {                                                // max(a, 0), 0 for a NaN (as fmaxf)
                             asm("v_max_f32_e32 %0, 0, %1" : "=v"(a0) : "v"(a0));
                             asm("v_max_f32_e32 %0, 0, %1" : "=v"(a1) : "v"(a1));

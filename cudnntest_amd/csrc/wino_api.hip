@@ -783,19 +783,25 @@ int launch_direct_t(int src, int dst, unsigned flags, const void* bias, const Ge
     if constexpr (sizeof(T) == 2) {
         // 2-byte tensors: the 16-bit matrix instruction, 16 taps each
         const size_t lds16 = direct16_lds_bytes(g.C, g.K);
-        if (src == WINO_NCHW && dst == WINO_NCHW && g.W % 2 == 0 && !misaligned(x, 4) && !misaligned(y, 4) &&
-            direct16_tiles_lds_bytes(g.C, g.K) <= 64 * 1024) {
+        const bool chwn_tiles = src == WINO_CHWN && dst == WINO_CHWN && g.N <= DSC_DS && ((long)g.W * g.N) % 2 == 0;
+        if (((src == WINO_NCHW && dst == WINO_NCHW && g.W % 2 == 0) || chwn_tiles) && !misaligned(x, 4) && !misaligned(y, 4) &&
+            direct16_tiles_lds_bytes(g.C, g.K, chwn_tiles ? g.N : 1) <= 64 * 1024) {
             // NCHW on both sides, rows of whole 4-byte pairs: tiles of 4 rows x 64 columns per wave, input through LDS,
             // whole cache lines stored; the tiles are dealt evenly to two workgroups per CU (the kernel's registers
-            // leave room for two waves a SIMD)
-            const int tiles_y = (g.Ho + DSC_WR - 1) / DSC_WR, tiles_x = (g.Wo + DSC_WC - 1) / DSC_WC;
-            const long ntiles = (long)g.N * tiles_y * tiles_x, resident = 8L * device_cus();
+            // leave room for two waves a SIMD).  CHWN on both sides: one image of width W * N, taps N columns apart.
+            const int ds = chwn_tiles ? g.N : 1, n1 = chwn_tiles ? 1 : g.N, w1 = g.W * ds, wo1 = g.Wo * ds;
+            const int tiles_y = (g.Ho + DSC_WR - 1) / DSC_WR, tiles_x = (wo1 + DSC_WC - 1) / DSC_WC;
+            const long ntiles = (long)n1 * tiles_y * tiles_x, resident = 8L * device_cus();
             const long per = (ntiles + resident - 1) / resident;                 // tiles per wave
             const dim3 tgrid((unsigned)((ntiles + 4 * per - 1) / (4 * per)));
-            const size_t ldst = direct16_tiles_lds_bytes(g.C, g.K);
-#define DIRECT16_TILES(NE)                                                                                              \
-    hipLaunchKernelGGL((direct_small_c16_tiles_kernel<T, NE>), tgrid, block, ldst, st, (const T*)x, (const T*)w, (T*)y, g.N, \
-                       g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, tiles_y, tiles_x, (int)ntiles, ep)
+            const size_t ldst = direct16_tiles_lds_bytes(g.C, g.K, ds);
+#define DIRECT16_TILES(NE)                                                                                                 \
+    if (chwn_tiles)                                                                                                        \
+        hipLaunchKernelGGL((direct_small_c16_tiles_kernel<T, NE, true>), tgrid, block, ldst, st, (const T*)x, (const T*)w,  \
+                           (T*)y, n1, g.C, g.K, g.H, w1, g.pad, ds, g.Ho, wo1, tiles_y, tiles_x, (int)ntiles, ep);          \
+    else                                                                                                                   \
+        hipLaunchKernelGGL((direct_small_c16_tiles_kernel<T, NE, false>), tgrid, block, ldst, st, (const T*)x, (const T*)w, \
+                           (T*)y, n1, g.C, g.K, g.H, w1, g.pad, ds, g.Ho, wo1, tiles_y, tiles_x, (int)ntiles, ep)
             switch (g.C) {
             case 1: DIRECT16_TILES(1); break;
             case 4: DIRECT16_TILES(3); break;
