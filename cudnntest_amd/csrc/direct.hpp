@@ -170,6 +170,166 @@ __global__ __launch_bounds__(256) void direct_small_c_kernel(const T* __restrict
     }
 }
 
+// The same for fp32 NCHW tensors on both sides with an even width, as tiles: the kernel above gathers a pixel's taps
+// with NE loads of one element per 32 pixels and filter tile -- 27 loads next to 32 stores for C = 3, K = 64, and a
+// CU takes about one memory instruction per 16 clocks whatever its width.  Here every WAVE takes tiles of 4 rows x 32
+// columns, one after the other, on its own: a tile's input, C x 6 rows x 36 columns, comes in as aligned 8-byte
+// pairs (6 loads per lane for C = 3, zeros where the padding is) and goes to LDS of the wave's own, the next tile's
+// requested before the current tile's multiplies (no workgroup barrier in the loop); a lane then reads its taps
+// from LDS.  The stores are those of the kernel above (a lane's 32 pixels of a filter are 128 contiguous bytes).
+// Same products in the same multiply slots, bias after the sum: the same bits as above.  (N = 32, 224 x 224, K = 64:
+// 125 -> 115 us; 411 MB of y, and store instructions and multiplies of a wave add up rather than overlap.  CHWN
+// tensors as one image of width W * N, which pays in 16 bits, were slower here than the kernel above: 130 against 117.)
+constexpr int DSF_WR = 4;                           // output rows of a wave's tile
+constexpr int DSF_PR = DSF_WR + 2;                  // input rows
+constexpr int DSF_PP = 18;                          // 8-byte pairs of an input row: 34 columns from an even one
+// loads per lane of a tile's input (pairs of [C][6][18]) by NE = ceil(9 C / 2)
+constexpr int dsf_loads(int ne) { return ne == 5 ? 2 : ne == 9 ? 4 : ne == 14 ? 6 : 7; }
+__host__ inline size_t direct_tiles_lds_bytes(int C, int K) {
+    const size_t base = direct_lds_bytes(C, K);
+    return base ? base + 4 * (size_t)C * DSF_PR * DSF_PP * 8 : 0;
+}
+
+template <int NE>
+__global__ __launch_bounds__(256) void direct_small_c_tiles_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                   float* __restrict__ y, int N, int C, int K, int H, int W,
+                                                                   int pad, int Ho, int Wo, int tiles_y, int tiles_x,
+                                                                   int ntiles, Epilogue ep) {
+    extern __shared__ __attribute__((aligned(16))) float smemt[];
+    const int KT = (K + 31) / 32;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int nk = 9 * C;
+    constexpr int PP = DSF_PP;
+    const int npairs = C * DSF_PR * PP;
+    float* sW = smemt;                                                           // [KT][NE][64]: lane (lh, l32) holds W[kt*32 + l32][2e + lh]
+    float* sB = smemt + (size_t)KT * NE * 64;                                    // [KT*32] bias
+    float* sP = sB + KT * 32 + wave * npairs * 2;                                // this wave's [C][6][2 PP] elements
+
+    for (int i = tid; i < KT * NE * 64; i += 256) {
+        const int ln = i & 63, e = (i >> 6) % NE, kt = (i >> 6) / NE;
+        const int k = kt * 32 + (ln & 31), kk = 2 * e + (ln >> 5);
+        const bool ok = k < K && kk < nk;
+        const float v = w[ok ? k * nk + kk : 0];                                   // [K][C][3][3]: tap kk of filter k
+        sW[i] = ok ? v : 0.f;
+    }
+    for (int i = tid; i < KT * 32; i += 256) sB[i] = i < K ? bias_of<float>(ep, i) : 0.f;
+    __syncthreads();
+
+    // a lane's taps in the tile's patch: element offset of (channel, row r, column s) relative to its pixel's first
+    // column; a tap past 9 C reads the pixel itself and is masked
+    int off[NE];
+    unsigned tapmask = 0;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        const int kk = 2 * e + lh;
+        const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
+        off[e] = kk < nk ? (c * DSF_PR + r) * PP * 2 + q : 0;
+        tapmask |= kk < nk ? 1u << e : 0u;
+    }
+    // the patch as loaded: pair 64 j + lane of [C][6][PP], as channel | row << 4 | pair of the row << 8 (row 15,
+    // never inside the image, past the patch)
+    constexpr int NL = dsf_loads(NE);
+    unsigned pd[NL];
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const int t = 64 * j + lane;
+        const int c = t / (DSF_PR * PP), rem = t - c * (DSF_PR * PP);
+        const int rr = rem / PP, pp = rem - rr * PP;
+        pd[j] = t < npairs ? (unsigned)(c | rr << 4 | pp << 8) : 0xF0u;
+    }
+    const int rounds = (npairs + 63) / 64;                                       // wave-uniform
+    const char* xb = reinterpret_cast<const char*>(x);
+    char* yb = reinterpret_cast<char*>(y);
+    const unsigned plane_y = (unsigned)Ho * (unsigned)Wo * 4u;                    // bytes of a filter's plane of y
+
+    const int wstride = (int)gridDim.x * 4;
+    int tile = (int)blockIdx.x * 4 + wave;
+    int n = 0, oh0 = 0, ow0 = 0;                                                  // of the tile whose input is on its way
+    uint2 v[NL];
+    unsigned inside = 0;                                                          // bit j: pair j lies inside the image
+    auto request = [&](int t) __attribute__((always_inline)) {
+        n = t / (tiles_y * tiles_x);
+        const int trem = t - n * tiles_y * tiles_x;
+        oh0 = (trem / tiles_x) * DSF_WR;
+        ow0 = (trem - (trem / tiles_x) * tiles_x) * 32;
+        const int ic0 = ow0 - pad - ((ow0 - pad) & 1);                           // first column of the patch: even, <= ow0 - pad
+        const int base = (n * C * H + oh0 - pad) * W + ic0;
+        inside = 0;
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            if (j < rounds) {                                                     // (uniform)
+                const int c = pd[j] & 15, rr = (pd[j] >> 4) & 15, pp = pd[j] >> 8;
+                const int ih = oh0 - pad + rr, iw = ic0 + 2 * pp;
+                const bool in = ih >= 0 && ih < H && iw >= 0 && iw < W;           // (W even: both elements or neither)
+                v[j] = *reinterpret_cast<const uint2*>(xb + (in ? (unsigned)((base + (c * H + rr) * W + 2 * pp) * 4) : 0u));
+                inside |= in ? 1u << j : 0u;
+            }
+        }
+    };
+    if (tile < ntiles) request(tile);
+#pragma unroll 1
+    while (tile < ntiles) {
+        const int cn = n, coh0 = oh0, cow0 = ow0;                                 // the tile to compute
+        const int shift = (cow0 - pad) & 1;
+#pragma unroll
+        for (int j = 0; j < NL; ++j)
+            if (j < rounds && 64 * j + lane < npairs) {
+                const unsigned m = 0u - ((inside >> j) & 1u);
+                reinterpret_cast<uint2*>(sP)[64 * j + lane] = make_uint2(v[j].x & m, v[j].y & m);
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        tile += wstride;
+        if (tile < ntiles) request(tile);
+
+        const int ow = cow0 + l32;
+        const bool pok = ow < Wo;
+#pragma unroll 1
+        for (int g = 0; g < DSF_WR; ++g) {
+            const int oh = coh0 + g;
+            if (oh >= Ho) break;                                                  // wave-uniform
+            const float* pb = sP + g * PP * 2 + l32 + shift;
+            float b[NE];
+#pragma unroll
+            for (int e = 0; e < NE; ++e) b[e] = __uint_as_float(__float_as_uint(pb[off[e]]) & (0u - ((tapmask >> e) & 1u)));
+            // this lane's pixel, filter 4 lh
+            unsigned yq = (unsigned)(((cn * K + 4 * lh) * Ho + oh) * Wo + ow) * 4u;
+#pragma unroll 1
+            for (int kt = 0; kt < KT; ++kt) {
+                floatx16 acc;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+                const float* wk = sW + (size_t)kt * NE * 64 + lane;
+#pragma unroll
+                for (int e = 0; e < NE; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wk[e * 64], b[e], acc, 0, 0, 0);
+                // register r: filter 8 (r / 4) + 4 lh + r % 4 of the tile
+                const float* bk = sB + kt * 32 + 4 * lh;
+                unsigned o = yq;
+                auto put = [&](int r, bool check) __attribute__((always_inline)) {
+                    float val = acc[r] + bk[8 * (r >> 2) + (r & 3)];
+                    if (ep.relu) val = fmaxf(val, 0.f);
+                    if (pok && (!check || kt * 32 + 8 * (r >> 2) + (r & 3) + 4 * lh < K)) *reinterpret_cast<float*>(yb + o) = val;
+                    o += ((r & 3) == 3 ? 5u : 1u) * plane_y;
+                };
+                if (kt * 32 + 32 <= K) {                                          // wave-uniform: all 32 filters of the tile exist
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) put(r, false);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) put(r, true);
+                }
+                yq += 32u * plane_y;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                   // (the tile's LDS reads before the next tile's writes)
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // Direct 3x3 convolution for layers with FEW OUTPUT PIXELS and a reduction of any length (a batch of one image: the
 // reference's sweep starts at layer 1-2 with batch 1, comparison/layoutCompare.cu:38-46).  Such a layer is a few
 // microseconds of arithmetic; through the Winograd pipelines it is three dependent launches, each of which starts,

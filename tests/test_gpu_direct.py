@@ -39,14 +39,15 @@ TILE_SHAPES = [(2, 3, 64, 40, 70), (1, 4, 70, 18, 34), (3, 1, 33, 17, 32), (2, 2
 
 
 @pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
-@pytest.mark.parametrize("dtype", [ops.F16, ops.BF16])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16, ops.BF16])
 @pytest.mark.parametrize("shape", TILE_SHAPES)
-def test_two_byte_layers_as_tiles_bit_exact(oracle, shape, dtype, layout):
-    """2-byte NCHW (NHWC) tensors with an even width (and an even K) run as tiles of 4 rows x 64 (32) columns per wave
+def test_few_channel_layers_as_tiles_bit_exact(oracle, shape, dtype, layout):
+    """fp32 NCHW tensors with an even width run as tiles of 4 rows x 32 columns per wave (input through LDS).
+    2-byte NCHW (NHWC) tensors with an even width (and an even K) run as tiles of 4 rows x 64 (32) columns per wave
     (input through LDS, sums exchanged between lanes, 4-byte pairs stored), CHWN tensors of up to 32 images as one
     NCHW image of width W * N with taps N columns apart (batches of 1, 2, 3 and 5): several tiles each way with ragged
     last ones, one to four channels, filter counts off the tile of 32 (K = 33 from NHWC: the gathering kernel), pad 0 and 1
-    (the patch starts at an even or an odd element), with and without bias and ReLU; a view that is only 2-byte
+    (the patch starts at an even or an odd element), with and without bias and ReLU; a view that is only element
     aligned takes the gathering kernel and gives the same bits."""
     N, C, K, H, W = shape
     x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
