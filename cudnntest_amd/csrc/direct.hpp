@@ -719,9 +719,9 @@ __global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restri
 // The same for NCHW tensors on both sides with an even width, as tiles.  The kernel above is bound by its memory
 // instructions twice over: it gathers a pixel's taps with sixteen 2-byte loads and stores its sums 2 bytes at a time
 // (48 memory instructions per 32 pixels x 64 filters; a CU takes about one per 16 clocks whatever its width), and the
-// 64-byte runs a wave writes per filter are half cache lines whose other half arrives from another CU: written as
-// this kernel's stores and nothing else, that pattern moves 3.5 TB/s, whole 128-byte lines 4.7 (N = 32, 224 x 224,
-// K = 64, 205 MB of y: 58 against 44 us).  Here every WAVE takes tiles of 4 rows x 64 columns, one after the
+// 64-byte runs a wave writes per filter are half cache lines whose other half arrives from another wave: written as
+// stores and nothing else (cli/store_pattern.hip), that pattern moves 3.9 TB/s, whole 128-byte lines 4.4 (N = 32,
+// 224 x 224, K = 64, 205 MB of y: 53 against 46 us).  Here every WAVE takes tiles of 4 rows x 64 columns, one after the
 // other, on its own:
 //   * a tile's input, C x 6 rows x 68 columns, comes in as aligned 4-byte pairs (10 loads per lane for C = 3, zeros
 //     where the padding is) and goes to LDS of the wave's own; a lane then gathers its taps with 2-byte LDS reads.
