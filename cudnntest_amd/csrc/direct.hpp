@@ -264,7 +264,7 @@ __global__ __launch_bounds__(256) void direct_small_c_tiles_kernel(const float* 
                 const int c = pd[j] & 15, rr = (pd[j] >> 4) & 15, pp = pd[j] >> 8;
                 const int ih = oh0 - pad + rr, iw = ic0 + 2 * pp;
                 const bool in = ih >= 0 && ih < H && iw >= 0 && iw < W;           // (W even: both elements or neither)
-                v[j] = *reinterpret_cast<const uint2*>(xb + (in ? (unsigned)((base + (c * H + rr) * W + 2 * pp) * 4) : 0u));
+                v[j] = *reinterpret_cast<const uint2*>(xb + (in ? (unsigned)(base + (c * H + rr) * W + 2 * pp) * 4u : 0u));
                 inside |= in ? 1u << j : 0u;
             }
         }
@@ -846,7 +846,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_kernel(const T* __
                 }
                 const int ih = oh0 - pad + rr, iw = ic0 + 2 * pp;
                 const bool in = t < npairs && ih >= 0 && ih < H && iw >= 0 && iw < W;   // (W even: both elements or neither)
-                v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)((base + (c * H + rr) * W + 2 * pp) * 2) : 0u));
+                v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)(base + (c * H + rr) * W + 2 * pp) * 2u : 0u));
                 inside |= in ? 1u << j : 0u;
             }
         }
@@ -1043,7 +1043,7 @@ __global__ __launch_bounds__(256) void direct_small_c16_tiles_nhwc_kernel(const 
                 const int rr = prp[j] & 0xFF, pp = prp[j] >> 8;
                 const int ih = oh0 - pad + rr, ie = e0 + 2 * pp;
                 const bool in = ih >= 0 && ih < H && ie >= 0 && ie < WC;          // (a row starts and ends at an even element)
-                v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)((base + rr * WC + 2 * pp) * 2) : 0u));
+                v[j] = *reinterpret_cast<const unsigned*>(xb + (in ? (unsigned)(base + rr * WC + 2 * pp) * 2u : 0u));
                 inside |= in ? 1u << j : 0u;
             }
         }

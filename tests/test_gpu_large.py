@@ -50,3 +50,28 @@ def test_more_than_2_31_elements_per_operand(oracle, layout):
     # leave the scratch arena at its usual size for the tests that follow
     del ys, y, xl
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("Nl", [208, 334])
+def test_first_layer_with_byte_offsets_past_2_31(oracle, Nl):
+    """The few-channel direct kernels address x and y with 32-bit byte offsets off a scalar base; the library offers
+    them up to 2^30 elements a tensor.  208 and 334 images of 3 x 224 x 224 into 64 filters in fp32: y holds 668 M and
+    1073 M elements (the last below 2^30 by a thousandth), byte offsets past 2^31 and up to 4.29 GB.  The tiled
+    kernel against the oracle on the last image, and against the gathering kernel (an element-aligned view of x) over
+    the whole tensor.  (2-byte tensors of 2^30 elements end below 2^31 bytes.)"""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * 2 ** 30:
+        pytest.skip("needs 16 GB of free device memory")
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.rand((Nl, 3, 224, 224), device="cuda", generator=g) * 2 - 1
+    w = torch.randn((64, 3, 3, 3), device="cuda", generator=g) * 0.2
+    assert 2 ** 31 < Nl * 64 * 224 * 224 * 4 < 2 ** 32 and Nl * 64 * 224 * 224 < 2 ** 30
+    y = ops.conv(x, w, 1, algo=ops.ALGO_DIRECT)
+    want = oracle.direct_conv_f32(host(x[Nl - 1:]), host(w), 1)
+    assert oracle.rel_l2(host(y[Nl - 1:]), want) <= 1e-6
+    shifted = torch.empty(x.numel() + 1, dtype=x.dtype, device="cuda")[1:].view(x.shape)
+    shifted.copy_(x)
+    y2 = ops.conv(shifted, w, 1, algo=ops.ALGO_DIRECT)
+    assert all(torch.equal(y[i:i + 16], y2[i:i + 16]) for i in range(0, Nl, 16))
+    del x, y, y2, shifted
+    torch.cuda.empty_cache()
