@@ -138,12 +138,15 @@ __global__ __launch_bounds__(256) void direct_small_c_kernel(const T* __restrict
                 const int k = kt * 32 + l32;
                 const float bk = sB[k];
                 if (k < K) {
+                    // element offsets fit 32 bits (the host checks the tensor sizes): one scalar base, a running offset
+                    unsigned o = ((unsigned)q0 + 4u * lh) * (unsigned)K + (unsigned)k;
+                    const bool whole = q0 + 32 <= Q;                              // wave-uniform: all 32 pixels of the group exist
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const long pq = q0 + 8 * (r >> 2) + 4 * lh + (r & 3);
                         float v = acc[r] + bk;
                         if (ep.relu) v = fmaxf(v, 0.f);
-                        if (pq < Q) y[pq * K + k] = from_f32<T>(v);
+                        if (whole || q0 + 8 * (r >> 2) + 4 * lh + (r & 3) < Q) y[o] = from_f32<T>(v);
+                        o += ((r & 3) == 3 ? 5u : 1u) * (unsigned)K;
                     }
                 }
                 continue;
@@ -687,12 +690,14 @@ __global__ __launch_bounds__(256) void direct_small_c16_kernel(const T* __restri
             if (SWAP) {
                 const int k = kt * 32 + l32;
                 if (k < K) {
+                    unsigned o = ((unsigned)q0 + 4u * lh) * (unsigned)K + (unsigned)k;   // (element offsets fit 32 bits)
+                    const bool whole = q0 + 32 <= Q;                              // wave-uniform: all 32 pixels of the group exist
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const long pq = q0 + 8 * (r >> 2) + 4 * lh + (r & 3);
                         float v = acc[r];
                         if (ep.relu) v = fmaxf(v, 0.f);
-                        if (pq < Q) y[pq * K + k] = from_f32<T>(v);
+                        if (whole || q0 + 8 * (r >> 2) + 4 * lh + (r & 3) < Q) y[o] = from_f32<T>(v);
+                        o += ((r & 3) == 3 ? 5u : 1u) * (unsigned)K;
                     }
                 }
                 continue;
