@@ -346,6 +346,7 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
     // a wave exist together, so a lane stores all its values or none.
     const unsigned kstride2 = (ep.pool ? (unsigned)((g.Ho >> 1) * (g.Wo >> 1)) : (unsigned)(g.Ho * g.Wo)) * 2u;   // bytes between the planes of two filters
     const bool odd = lane & 1;
+    const unsigned psel = odd ? 0x03020706u : 0x05040100u;   // (own pair, neighbour's pair) -> even lanes: both lanes' first value; odd lanes: both lanes' second
     auto stores = [&]() {
         if (k0c >= g.K || yoff[0] < 0) return;
         // (opaque to the optimiser: called from inside the stage loop, the 64 store addresses of a tile would be
@@ -402,10 +403,10 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                     for (int i = 0; i < 2; ++i) {
                         float v0 = acc[i][j][r2] + bk[i], v1 = acc[i][j][r2 + 1] + bk[i];
                         if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
-                        const float got = swap_lane_pairs(odd ? v0 : v1);
-                        const float lo = odd ? got : v0, hi = odd ? v1 : got;
-                        struct alignas(4) Pair { T a, b; };
-                        if (pok) *reinterpret_cast<Pair*>(yb + o[j] + (unsigned)(i * 64)) = Pair{from_f32<T>(lo), from_f32<T>(hi)};
+                        // (rounded and packed first; the neighbour's pair by one DPP move, the lane's two by one byte permute)
+                        const unsigned own = pack2<T>(v0, v1);
+                        const unsigned nb = (unsigned)__builtin_amdgcn_mov_dpp((int)own, 0xB1, 0xF, 0xF, true);
+                        if (pok) *reinterpret_cast<unsigned*>(yb + o[j] + (unsigned)(i * 64)) = __builtin_amdgcn_perm(nb, own, psel);
                     }
                     o[j] += ((r2 & 2) ? 6u : 2u) * kp;
                 }
@@ -461,10 +462,9 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                     if (j == 3 && !r4) continue;             // (uniform: a 3-row tile)
                     float v0 = acc[i][j][r2] + b0, v1 = acc[i][j][r2 + 1] + b1;
                     if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
-                    const float got = swap_lane_pairs(odd ? v0 : v1);
-                    const float lo = odd ? got : v0, hi = odd ? v1 : got;
-                    struct alignas(4) Pair { T a, b; };
-                    *reinterpret_cast<Pair*>(yb + o[j]) = Pair{from_f32<T>(lo), from_f32<T>(hi)};
+                    const unsigned own = pack2<T>(v0, v1);
+                    const unsigned nb = (unsigned)__builtin_amdgcn_mov_dpp((int)own, 0xB1, 0xF, 0xF, true);
+                    *reinterpret_cast<unsigned*>(yb + o[j]) = __builtin_amdgcn_perm(nb, own, psel);
                     o[j] += ((r2 & 2) ? 6u : 2u) * ks;
                 }
                 __builtin_amdgcn_sched_barrier(0);           // one register pair at a time
