@@ -52,6 +52,33 @@ struct D16Geom {
     long G;                // N * Ho output rows
 };
 
+// ---- 2x2 / stride-2 maximum of a [K][Ho][Wo][N] tensor of 2-byte elements ---------------------------------
+// The 8-wave kernel pools in its stores where a window's columns sit in neighbouring lanes; in a CHWN tensor they are N
+// elements apart, in different waves.  Such a layer is convolved unpooled (bias and ReLU applied) into scratch and this
+// kernel follows: a thread takes VEC images of one window.  max(round(v)) = round(max(v)): the same bits as a kernel
+// that pooled before it rounded.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void pool2_chwn_kernel(const T* __restrict__ t, T* __restrict__ y, int Ho, int Wo, int N,
+                                                         long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int nv = N / VEC, Hp = Ho >> 1, Wp = Wo >> 1;
+    const int n0 = (int)(i % nv) * VEC;
+    long r = i / nv;
+    const int pw = (int)(r % Wp);
+    r /= Wp;
+    const int ph = (int)(r % Hp);
+    const long k = r / Hp;
+    const T* src = t + ((k * Ho + 2 * ph) * Wo + 2 * pw) * (long)N + n0;
+    struct alignas(VEC * 2) Vec { T v[VEC]; };
+    const Vec a = *reinterpret_cast<const Vec*>(src), b = *reinterpret_cast<const Vec*>(src + N);
+    const Vec c = *reinterpret_cast<const Vec*>(src + (long)Wo * N), d = *reinterpret_cast<const Vec*>(src + (long)Wo * N + N);
+    Vec o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.v[e] = from_f32<T>(fmaxf(fmaxf(to_f32(a.v[e]), to_f32(b.v[e])), fmaxf(to_f32(c.v[e]), to_f32(d.v[e]))));
+    *reinterpret_cast<Vec*>(y + ((k * Hp + ph) * Wp + pw) * (long)N + n0) = o;
+}
+
 // ---- filter bank -> W9[tap][Cp/8][Kp][8] (zero padded) --------------------------------------------------
 // One thread per (filter, channel vector).  VEC = 1: the bank is [K][C][3][3] with C a multiple of 8 and a 16-byte
 // aligned base, so the 72 values of a thread are 144 contiguous, aligned bytes: nine 16-byte loads instead of 72

@@ -1085,7 +1085,8 @@ bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g)
     D16Geom d;
     if (dtype == WINO_F32 || g.C % 8 != 0 || g.pad > 1 || (long)g.N * g.K * g.Ho * g.Wo >= (1L << 31)) return false;
     if (src == WINO_CHWN || dst == WINO_CHWN) {
-        // CHWN on both sides: the 8-wave kernel only, no pooling (a pooling window's columns are N elements apart);
+        // CHWN on both sides: the 8-wave kernel only, no pooling in its stores (a pooling window's columns are N elements
+        // apart: direct16_chwn_pool_ok and a pooling kernel take such a layer);
         // 32-bit byte offsets inside a stage's 16 channel planes
         return src == dst && !(flags & WINO_FLAG_POOL2) && (long)g.H * g.W * g.N * 2 * 16 < (1L << 32) && direct16_big(g, &d, true);
     }
@@ -1177,6 +1178,33 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
 #undef D16_GO
 }
 
+// CHWN tensors with 2x2 pooling: the layer unpooled into `tmp` (room for direct16_unpooled_bytes), then the pooling kernel
+bool direct16_chwn_pool_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
+    return src == WINO_CHWN && dst == WINO_CHWN && (flags & WINO_FLAG_POOL2) &&
+           direct16_ok(src, dst, dtype, flags & ~(unsigned)WINO_FLAG_POOL2, g);
+}
+size_t direct16_unpooled_bytes(int dtype, const Geometry& g) {
+    return ((size_t)g.N * g.K * g.Ho * g.Wo * dtype_size(dtype) + 255) / 256 * 256;
+}
+template <typename T>
+int launch_pool2_chwn_t(const Geometry& g, const void* tmp, void* y, hipStream_t st) {
+    const int vec = g.N % 8 == 0 && !misaligned(y, 16) ? 8 : g.N % 2 == 0 && !misaligned(y, 4) ? 2 : 1;   // (tmp is scratch: aligned)
+    const long total = (long)g.K * (g.Ho / 2) * (g.Wo / 2) * (g.N / vec);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (vec == 8) hipLaunchKernelGGL((pool2_chwn_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, g.N, total);
+    else if (vec == 2) hipLaunchKernelGGL((pool2_chwn_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, g.N, total);
+    else hipLaunchKernelGGL((pool2_chwn_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, g.N, total);
+    LAUNCH_CHECK("pool2_chwn");
+    return WINO_OK;
+}
+int launch_direct16_chwn_pooled(int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
+                                void* W9, void* tmp, void* y, hipStream_t st, int mode) {
+    const int rc = launch_direct16(WINO_CHWN, WINO_CHWN, dtype, flags & ~(unsigned)WINO_FLAG_POOL2, bias, g, x, w, W9, tmp, st, mode);
+    if (rc || mode == D16_PACK) return rc;
+    if (dtype == WINO_F16) return launch_pool2_chwn_t<f16_t>(g, tmp, y, st);
+    return launch_pool2_chwn_t<bf16_t>(g, tmp, y, st);
+}
+
 int pick_algo(int layout, int dtype, const Geometry& g) {
     const long patches = ((g.P + GO_T - 1) / GO_T) * ((g.K + GO_T - 1) / GO_T);
     const bool nhwc = layout == WINO_NHWC;
@@ -1225,7 +1253,11 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
 // 98 us; NHWC tensors, 8-wave kernel only: 236 against 462, 92 against 150, 143 against 257, 73 against 96, 122
 // against 170, 68 against 79, 117 against 133 us).  x, y: the tensors if known (their alignment decides: with an NHWC
 // side only the 8-wave kernel runs, and it stores 4-byte pairs unless it pools).
+bool direct16_chwn_pool_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g);
 bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y) {
+    // (a pooled CHWN layer runs unpooled into scratch, then a pooling kernel: N = 32 in bf16, direct + pooling against the
+    // fastest Winograd pipeline with pooling in its output stage: 183 + 46 against 528 us at C = K = 64, H = 224)
+    if (direct16_chwn_pool_ok(src, dst, dtype, flags, g)) return auto_direct16(src, dst, dtype, flags & ~(unsigned)WINO_FLAG_POOL2, g, x, nullptr);
     if (!direct16_ok(src, dst, dtype, flags, g) || misaligned(x, src == WINO_NHWC ? 16 : 4)) return false;
     if ((src == WINO_NHWC || dst == WINO_NHWC) && !(flags & WINO_FLAG_POOL2) && misaligned(y, 4)) return false;
     D16Geom d;
@@ -1346,6 +1378,13 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     if (algo == WINO_ALGO_AUTO) {
         algo = resolve_auto(src, dst, dtype, flags, g, x, y, w != nullptr);
         if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4) Upre = nullptr;      // transformed filters handed in alongside w are F(2x2) ones
+        // (a pooled CHWN layer on the direct path keeps the unpooled tensor in scratch: with a fixed buffer too small
+        // for it the Winograd pipelines take the layer)
+        if (algo == WINO_ALGO_DIRECT && ss.fixed && direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
+            kCounterBytes + direct16_bank_bytes(g) + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) {
+            algo = pick_algo(src, dtype, g);
+            if (algo == WINO_ALGO_FUSED && g.pad > 1) algo = WINO_ALGO_EPILOGUE;
+        }
     }
     if (algo == WINO_ALGO_DIRECT) {
         if (!w) return fail(WINO_ERR_INVALID, "the direct path needs the filter bank, not its Winograd transform");
@@ -1356,6 +1395,15 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (direct_few_ok(dtype, flags, g)) {
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
             return launch_direct_few(src, dst, flags, bias, g, x, w, y, (hipStream_t)stream);
+        }
+        if (direct16_chwn_pool_ok(src, dst, dtype, flags, g)) {
+            const size_t bank = (direct16_bank_bytes(g) + 255) / 256 * 256;
+            void* base = nullptr;
+            const int rcb = ss.get(kCounterBytes + bank + direct16_unpooled_bytes(dtype, g), &base);
+            if (rcb) return rcb;
+            StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
+            return launch_direct16_chwn_pooled(dtype, flags, bias, g, x, w, (char*)base + kCounterBytes, (char*)base + kCounterBytes + bank, y,
+                                               (hipStream_t)stream, D16_PACK_RUN);
         }
         if (!direct16_ok(src, dst, dtype, flags, g))
             return fail(WINO_ERR_UNSUPPORTED, "the direct path is built for pad 0 and 1: for C <= 4, and for 2-byte NCHW tensors with "
@@ -1896,7 +1944,12 @@ static int stack_run(wino_stack* s, const void* x, void* y, void* stream) {
                    auto_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, g, in, out)) {
             // (the bank was packed for 4-byte aligned tensors; a caller's tensor that is not takes the general call)
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
-            rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
+            if (direct16_chwn_pool_ok(L.layout_in, L.layout_out, s->dtype, L.flags, g)) {
+                void* tmp = nullptr;
+                rc = arena_get(direct16_unpooled_bytes(s->dtype, g), &tmp);
+                if (!rc) rc = launch_direct16_chwn_pooled(s->dtype, L.flags, bias, g, in, nullptr, L.W9, tmp, out, (hipStream_t)stream, D16_RUN);
+            } else
+                rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, bias, g, in, nullptr, L.W9, out, (hipStream_t)stream, D16_RUN);
         } else {
             rc = conv_impl(ScratchSource{}, L.layout_in, L.layout_out, s->dtype, L.algo, L.flags, s->N, L.C, L.K, L.H, L.W, 1, in,
                            L.wraw, L.U, bias, out, stream);
@@ -2001,7 +2054,8 @@ int wino_stack_set_layer(wino_stack_t* s, int layer, const void* w, const void* 
     if (L.W9) {
         Geometry g;
         make_geometry(s->dtype, s->N, L.C, L.K, L.H, L.W, 1, &g);
-        rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, L.flags, nullptr, g, L.W9, w, L.W9, L.W9, (hipStream_t)stream, D16_PACK);   // (x, y: any aligned address)
+        const unsigned pflags = L.layout_in == WINO_CHWN ? L.flags & ~(unsigned)WINO_FLAG_POOL2 : L.flags;   // (a pooled CHWN layer runs unpooled)
+        rc = launch_direct16(L.layout_in, L.layout_out, s->dtype, pflags, nullptr, g, L.W9, w, L.W9, L.W9, (hipStream_t)stream, D16_PACK);   // (x, y: any aligned address)
         if (rc) return rc;
     }
     L.has_bias = bias != nullptr;

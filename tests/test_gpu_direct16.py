@@ -166,10 +166,13 @@ def test_chwn_tensors_on_the_8_wave_kernel(oracle, shape, dtype):
         for n in (0, N - 1):
             want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], pad) + bias[ks][None, :, None, None], 0)
             assert np.array_equal(host(got.permute(3, 0, 1, 2)[n:n + 1][:, ks]), rounded(want.astype(np.float32), dtype, oracle)), (rep, n)
-    # pooling windows span columns N elements apart: not in this kernel's stores; other layouts on one side neither
-    with pytest.raises(_lib.WinoError) as e:
-        ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
-    assert e.value.code == -2
+    # pooling windows span columns N elements apart, in different waves: the layer runs unpooled into scratch and a
+    # pooling kernel follows (rounding is monotonic: the same bits as pooling before the rounding)
+    pooled = ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+    assert tuple(pooled.shape) == (K, got.shape[1] // 2, got.shape[2] // 2, N)
+    assert torch.equal(pooled.permute(3, 0, 1, 2), torch.nn.functional.max_pool2d(nchw.float(), 2).to(nchw.dtype))
+    assert torch.equal(pooled, ops.conv(xd, wd, pad, ops.CHWN, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True))
+    # other layouts on one side: not built
     with pytest.raises(_lib.WinoError) as e:
         ops.conv(xd, wd, pad, ops.CHWN, ops.NCHW, algo=ops.ALGO_DIRECT)
     assert e.value.code == -2
@@ -208,10 +211,10 @@ def test_layers_whose_images_are_cut_into_4_row_and_3_row_blocks(oracle, shape, 
     for n in (0, N - 1):
         want = np.maximum(oracle.direct_conv(x[n:n + 1], w[ks], 1) + bias[ks][None, :, None, None], 0)
         assert np.array_equal(g[n:n + 1][:, ks], rounded(want.astype(np.float32), dtype, oracle)), n
-    if layout != ops.CHWN:                                     # pooled: whole row pairs in a wave, so no cut -- the same values, pooled
-        pooled = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
-        want = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True)
-        assert torch.equal(pooled, want)
+    # pooled: whole row pairs in a wave, so no cut (CHWN: the cut layer unpooled, then a pooling kernel) -- the same values, pooled
+    pooled = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_DIRECT, relu=True, bias=bd, pool=True)
+    want = ops.conv(xd, wd, 1, layout, algo=ops.ALGO_STAGED, relu=True, bias=bd, pool=True)
+    assert torch.equal(pooled, want)
 
 
 def test_chwn_layers_the_8_wave_kernel_does_not_take():
