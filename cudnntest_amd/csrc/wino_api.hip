@@ -1359,6 +1359,17 @@ int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo,
     DISPATCH_DTYPE(dtype, launch_f4_output<T>(dst, order, porder, flags, bias, N, K, g.Ho, g.Wo, g.Kp, g.P, g.Pp, Mo, y, st));
 }
 
+// What the automatic choice runs when its first choice does not fit a fixed scratch buffer: a pooled CHWN layer on the
+// direct path keeps the unpooled tensor in scratch; without room for it the Winograd pipelines take the layer.
+int auto_within(const ScratchSource& ss, int algo, int src, int dst, int dtype, unsigned flags, const Geometry& g) {
+    if (algo == WINO_ALGO_DIRECT && ss.fixed && direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
+        kCounterBytes + (direct16_bank_bytes(g) + 255) / 256 * 256 + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) {
+        algo = pick_algo(src, dtype, g);
+        if (algo == WINO_ALGO_FUSED && g.pad > 1) algo = WINO_ALGO_EPILOGUE;
+    }
+    return algo;
+}
+
 int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, unsigned flags, int N, int C, int K, int H,
               int W, int pad, const void* x, const void* w, const void* Upre, const void* bias, void* y, void* stream) {
     if (!valid_layout(src) || !valid_layout(dst)) return fail(WINO_ERR_INVALID, "unknown layout %d -> %d", src, dst);
@@ -1378,13 +1389,7 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
     if (algo == WINO_ALGO_AUTO) {
         algo = resolve_auto(src, dst, dtype, flags, g, x, y, w != nullptr);
         if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4) Upre = nullptr;      // transformed filters handed in alongside w are F(2x2) ones
-        // (a pooled CHWN layer on the direct path keeps the unpooled tensor in scratch: with a fixed buffer too small
-        // for it the Winograd pipelines take the layer)
-        if (algo == WINO_ALGO_DIRECT && ss.fixed && direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
-            kCounterBytes + direct16_bank_bytes(g) + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) {
-            algo = pick_algo(src, dtype, g);
-            if (algo == WINO_ALGO_FUSED && g.pad > 1) algo = WINO_ALGO_EPILOGUE;
-        }
+        algo = auto_within(ss, algo, src, dst, dtype, flags, g);
     }
     if (algo == WINO_ALGO_DIRECT) {
         if (!w) return fail(WINO_ERR_INVALID, "the direct path needs the filter bank, not its Winograd transform");
@@ -1521,6 +1526,7 @@ int conv_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (algo == WINO_ALGO_AUTO) {
             algo = resolve_auto(src, dst, dtype, flags, g, x, y, w != nullptr);
             if (algo == WINO_ALGO_STAGED_F4 || algo == WINO_ALGO_EPILOGUE_F4) Upre = nullptr;  // transformed filters handed in alongside w are F(2x2) ones
+            algo = auto_within(ss, algo, src, dst, dtype, flags, g);
         }
         passes = batch_passes(src, dst, dtype, algo, g);
     }

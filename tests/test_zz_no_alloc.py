@@ -84,3 +84,17 @@ def test_a_problem_beyond_the_buffer_is_refused():
     w.normal_(0, 0.05)
     ops.conv_noalloc(x, w, out, algo=ops.ALGO_FUSED)
     assert torch.equal(out, ops.conv(x, w, algo=ops.ALGO_FUSED))
+
+
+def test_pooled_chwn_layers_with_and_without_room_for_the_unpooled_tensor(oracle):
+    """A pooled 2-byte CHWN layer on the direct path keeps the unpooled tensor in scratch.  N = 32, C = K = 64: at 56 x 56
+    it fits the buffer (12.8 MB) and the call runs the same two kernels as wino_conv_ex; at 160 x 160 it does not
+    (105 MB), and the automatic choice falls back to a Winograd pipeline that fits -- small integers, so both are exact
+    and agree bit for bit."""
+    for H in (56, 160):
+        N, C, K = 32, 64, 64
+        x, w = synth.conv_inputs(N, C, K, H, H, seed=H, layout=ops.CHWN, integer=True)
+        bias = dev(synth.small_ints(K, seed=4, lo=-2, hi=2).astype(np.float32), ops.BF16)
+        got, want = both(dev(x, ops.BF16), dev(w, ops.BF16), bias, ops.CHWN, ops.ALGO_AUTO, relu=True, pool=True)
+        assert (N * K * H * H * 2 > LIMIT) == (H == 160)
+        assert torch.equal(got, want), H
