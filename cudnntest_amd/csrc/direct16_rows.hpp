@@ -248,7 +248,10 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         k0c = t.k0 + wf * 64;
         r4 = t.R == 4;
         const long g0 = (long)t.n0 * g.Ho + t.oh0;
-        const int col = 32 * wc + l32;
+        // DIL with pooling (32 images: a column group of 32 is one pixel column): a wave takes 16 images of TWO
+        // neighbouring pixel columns, lanes 0-15 the even one, so that a pooling window's columns are lanes 16 apart;
+        // the two waves of a pair take the two halves of the images
+        const int col = DIL && ep.pool ? ((wc & ~1) + ((l32 >> 4) & 1)) * 32 + 16 * (wc & 1) + (l32 & 15) : 32 * wc + l32;
         const bool colok = t.c0 + col < g.Wo;
         const int ohp = t.oh0 + t.R * wr;                    // the wave's rows lie in one image: Ho is a multiple of 4 (of a block's rows, with 3-row blocks mixed in)
         int dn = 0;
@@ -278,9 +281,11 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
             // 2x2 pooling: the wave's rows are two pooling rows (Ho is a multiple of 4), a lane pair is one pooling
             // column (Wo is even); yoff[0], yoff[1]: the two pooled rows, this pair's column
             const int Hq = g.Ho >> 1, Wq = g.Wo >> 1;
+            // (DIL: column = 32 pixel column + image; the pooled row holds 32 (pixel column / 2) + image)
+            const int pcol = DIL ? (((t.c0 + col) >> 6) << 5) + ((t.c0 + col) & 31) : (t.c0 + col) >> 1;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                yoff[j] = (int)((((long)(t.n0 + dn) * g.K + k0c) * Hq + (oh >> 1) + j) * Wq + ((t.c0 + col) >> 1));
+                yoff[j] = (int)((((long)(t.n0 + dn) * g.K + k0c) * Hq + (oh >> 1) + j) * Wq + pcol);
         }
     };
 
@@ -417,9 +422,11 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
         if (ep.pool) {
             // with pooling: the maximum over the two rows in registers, over the two columns with the neighbouring lane;
             // the even lane stores the pooled value of filter r, the odd lane that of filter r+1 (2 bytes each)
+            // (DIL: the window's other column is 16 lanes away; lanes 0-15 store filter r, lanes 16-31 filter r+1)
+            const bool second = DIL ? (l32 & 16) != 0 : odd;
             unsigned q[2];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) q[j] = (unsigned)yoff[j] * 2u + (unsigned)(4 * lh + (odd ? 1 : 0)) * ks;
+            for (int j = 0; j < 2; ++j) q[j] = (unsigned)yoff[j] * 2u + (unsigned)(4 * lh + (second ? 1 : 0)) * ks;
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -435,9 +442,14 @@ __global__ __launch_bounds__(512, 1) void direct16_rows_kernel(const T* __restri
                         float v0 = fmaxf(acc[i][2 * j][r2], acc[i][2 * j + 1][r2]) + b0;
                         float v1 = fmaxf(acc[i][2 * j][r2 + 1], acc[i][2 * j + 1][r2 + 1]) + b1;
                         if (ep.relu) { v0 = fmaxf(v0, 0.f); v1 = fmaxf(v1, 0.f); }
-                        v0 = fmaxf(v0, swap_lane_pairs(v0));
-                        v1 = fmaxf(v1, swap_lane_pairs(v1));
-                        *reinterpret_cast<T*>(yb + q[j]) = from_f32<T>(odd ? v1 : v0);
+                        if constexpr (DIL) {
+                            v0 = fmaxf(v0, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v0), 0x401F)));   // lane ^ 16
+                            v1 = fmaxf(v1, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v1), 0x401F)));
+                        } else {
+                            v0 = fmaxf(v0, swap_lane_pairs(v0));
+                            v1 = fmaxf(v1, swap_lane_pairs(v1));
+                        }
+                        *reinterpret_cast<T*>(yb + q[j]) = from_f32<T>(second ? v1 : v0);
                         q[j] += ((r2 & 2) ? 6u : 2u) * ks;
                     }
                     __builtin_amdgcn_sched_barrier(0);

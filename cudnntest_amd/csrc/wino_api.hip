@@ -1081,6 +1081,9 @@ bool direct16_big(const Geometry& g, D16Geom* d, bool chwn = false, bool xn = fa
                            : (direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, d, xn) : direct16_rows_plan<1>(g, d, xn));
     return plan && (long)d->rowBlocks * d->colBlocks * d->kTiles >= device_cus() / 2;
 }
+// A pooled CHWN layer in the 8-wave kernel's own stores: with 32 images a column group of 32 is one pixel column, and a
+// wave takes 16 images of two neighbouring pixel columns instead, so that a window's columns are lanes 16 apart.
+inline bool direct16_chwn_pools(const Geometry& g) { return g.N == 32 && g.Wo % 2 == 0; }
 bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
     D16Geom d;
     if (dtype == WINO_F32 || g.C % 8 != 0 || g.pad > 1 || (long)g.N * g.K * g.Ho * g.Wo >= (1L << 31)) return false;
@@ -1088,7 +1091,8 @@ bool direct16_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g)
         // CHWN on both sides: the 8-wave kernel only, no pooling in its stores (a pooling window's columns are N elements
         // apart: direct16_chwn_pool_ok and a pooling kernel take such a layer);
         // 32-bit byte offsets inside a stage's 16 channel planes
-        return src == dst && !(flags & WINO_FLAG_POOL2) && (long)g.H * g.W * g.N * 2 * 16 < (1L << 32) && direct16_big(g, &d, true);
+        return src == dst && (!(flags & WINO_FLAG_POOL2) || direct16_chwn_pools(g)) && (long)g.H * g.W * g.N * 2 * 16 < (1L << 32) &&
+               direct16_big(g, &d, true);
     }
     if (src == WINO_NHWC || dst == WINO_NHWC) {
         // an NHWC side: the 8-wave kernel only; offsets inside a block's images are 32-bit
@@ -1135,8 +1139,8 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
     // the chip short of tiles
     int npg = 4, wf = direct16_rows_wf(g);
     const bool pool = (flags & WINO_FLAG_POOL2) != 0;        // (pooled values are stored one by one: no alignment asked of y)
-    const bool big = (pool || !misaligned(y, 4)) && !(chwn && pool) && direct16_big(g, &d, chwn, nhwc);
-    if (chwn && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of CHWN tensors: the 8-wave kernel's layer shapes, an even batch, no pooling, y 4-byte aligned");
+    const bool big = (pool || !misaligned(y, 4)) && !(chwn && pool && !direct16_chwn_pools(g)) && direct16_big(g, &d, chwn, nhwc);
+    if (chwn && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of CHWN tensors: the 8-wave kernel's layer shapes, an even batch (pooling: 32 images, an even width), y 4-byte aligned");
     if ((nhwc || ynhwc) && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution of NHWC tensors: the 8-wave kernel's layer shapes, y 4-byte aligned");
     if (pool && !big) return fail(WINO_ERR_UNSUPPORTED, "direct convolution: pooling needs the 8-wave kernel's layer shapes");
     const bool rows = !big && direct16_plan(g, 4, true, &d) && (long)d.rowBlocks * d.colBlocks * d.kTiles >= 2L * device_cus();
@@ -1178,9 +1182,10 @@ int launch_direct16(int layout, int dst, int dtype, unsigned flags, const void* 
 #undef D16_GO
 }
 
-// CHWN tensors with 2x2 pooling: the layer unpooled into `tmp` (room for direct16_unpooled_bytes), then the pooling kernel
+// CHWN tensors with 2x2 pooling that the 8-wave kernel does not pool itself (batches other than 32): the layer unpooled
+// into `tmp` (room for direct16_unpooled_bytes), then the pooling kernel
 bool direct16_chwn_pool_ok(int src, int dst, int dtype, unsigned flags, const Geometry& g) {
-    return src == WINO_CHWN && dst == WINO_CHWN && (flags & WINO_FLAG_POOL2) &&
+    return src == WINO_CHWN && dst == WINO_CHWN && (flags & WINO_FLAG_POOL2) && !direct16_chwn_pools(g) &&
            direct16_ok(src, dst, dtype, flags & ~(unsigned)WINO_FLAG_POOL2, g);
 }
 size_t direct16_unpooled_bytes(int dtype, const Geometry& g) {

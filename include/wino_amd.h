@@ -90,9 +90,10 @@ typedef enum {
                                tile for every other CU; other NHWC layers are refused (WINO_ERR_UNSUPPORTED).
                                2-byte CHWN -> CHWN layers (comparison/wrapedConv_CHWN.cuh:16-82) run on the same kernel, taken as one
                                image of width W * N whose tap columns lie N elements apart: the same shape conditions, an
-                               even batch of at most 32 images (more where the rows are short), x and y 4-byte aligned; with
-                               2x2 pooling the layer runs unpooled into scratch (N*K*Ho*Wo elements) and a pooling kernel
-                               follows; other CHWN layers, and layers with CHWN on one side only, are refused.
+                               even batch of at most 32 images (more where the rows are short), x and y 4-byte aligned; 2x2
+                               pooling in the kernel's stores for 32 images and an even width, otherwise the layer runs
+                               unpooled into scratch (N*K*Ho*Wo elements) and a pooling kernel follows; other CHWN
+                               layers, and layers with CHWN on one side only, are refused.
                                Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (the
                                shape just named), not for C <= 4; needs the filter bank itself (not
                                wino_conv_prepared).
