@@ -333,6 +333,159 @@ __global__ __launch_bounds__(256) void direct_small_c_tiles_kernel(const float* 
     }
 }
 
+// The same for fp32 NHWC tensors on both sides (W * C even): an input row of a tile is ONE contiguous run of
+// (32 + 2) x C elements, 17 C + 1 aligned 8-byte pairs (the run may start at an odd element; a row of the image starts
+// and ends at an even one, so no pair straddles its edge); the pixels are the multiply's first operand, so a lane holds
+// one filter and its registers the pixels; two filter tiles are multiplied at a time and exchange register halves, so
+// that a store instruction writes 64 filters of one pixel, 256 contiguous bytes when K = 64.
+// Same products in the same multiply slots as the gathering kernel, bias after the sum: the same bits.
+constexpr int dsf_nhwc_loads(int ne) { return ne == 5 ? 2 : ne == 9 ? 4 : ne == 14 ? 5 : 7; }   // pairs of [6][17 C + 1] over 64 lanes
+__host__ inline size_t direct_tiles_nhwc_lds_bytes(int C, int K) {
+    const size_t base = direct_lds_bytes(C, K);
+    return base ? base + 4 * (size_t)DSF_PR * (17 * C + 1) * 8 : 0;
+}
+
+template <int NE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void direct_small_c_tiles_nhwc_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                        float* __restrict__ y, int N, int C, int K, int H, int W,
+                                                                        int pad, int Ho, int Wo, int tiles_y, int tiles_x,
+                                                                        int ntiles, Epilogue ep) {
+    extern __shared__ __attribute__((aligned(16))) float smemn[];
+    const int KT = (K + 31) / 32;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int nk = 9 * C;
+    const int PPN = 17 * C + 1;                                                  // pairs of an input row of a tile
+    const int npairs = DSF_PR * PPN;
+    float* sW = smemn;                                                           // [KT][NE][64]: lane (lh, l32) holds W[kt*32 + l32][2e + lh]
+    float* sB = smemn + (size_t)KT * NE * 64;                                    // [KT*32] bias
+    float* sP = sB + KT * 32 + wave * npairs * 2;                                // this wave's [6][2 PPN] elements
+
+    for (int i = tid; i < KT * NE * 64; i += 256) {
+        const int ln = i & 63, e = (i >> 6) % NE, kt = (i >> 6) / NE;
+        const int k = kt * 32 + (ln & 31), kk = 2 * e + (ln >> 5);
+        const bool ok = k < K && kk < nk;
+        const float v = w[ok ? k * nk + (kk % 9) * C + kk / 9 : 0];                // [K][3][3][C]: tap kk = 9 c + 3 r + s of filter k
+        sW[i] = ok ? v : 0.f;
+    }
+    for (int i = tid; i < KT * 32; i += 256) sB[i] = i < K ? bias_of<float>(ep, i) : 0.f;
+    __syncthreads();
+
+    // a lane's taps in the tile's patch: tap kk = 9 c + 3 r + s meets the input at row r, element s C + c past the
+    // pixel's first; a tap past 9 C reads the pixel itself and is masked
+    int off[NE];
+    unsigned tapmask = 0;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        const int kk = 2 * e + lh;
+        const int c = kk / 9, r = (kk % 9) / 3, q = kk % 3;
+        off[e] = kk < nk ? r * PPN * 2 + q * C + c : 0;
+        tapmask |= kk < nk ? 1u << e : 0u;
+    }
+    // the patch as loaded: pair 64 j + lane of [6][PPN], as row | pair of the row << 8 (row 255, never inside, past it)
+    constexpr int NL = dsf_nhwc_loads(NE);
+    unsigned prp[NL];
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        const int t = 64 * j + lane;
+        const int rr = t / PPN, pp = t - rr * PPN;
+        prp[j] = t < npairs ? (unsigned)(rr | pp << 8) : 0xFFu;
+    }
+    const int rounds = (npairs + 63) / 64;                                       // wave-uniform
+    const char* xb = reinterpret_cast<const char*>(x);
+    const int WC = W * C;                                                         // elements of an image row (even)
+
+    const int wstride = (int)gridDim.x * 4;
+    int tile = (int)blockIdx.x * 4 + wave;
+    int n = 0, oh0 = 0, ow0 = 0;                                                  // of the tile whose input is on its way
+    uint2 v[NL];
+    unsigned inside = 0;                                                          // bit j: pair j lies inside the image
+    auto request = [&](int t) __attribute__((always_inline)) {
+        n = t / (tiles_y * tiles_x);
+        const int trem = t - n * tiles_y * tiles_x;
+        oh0 = (trem / tiles_x) * DSF_WR;
+        ow0 = (trem - (trem / tiles_x) * tiles_x) * 32;
+        const int e0 = (ow0 - pad) * C - (((ow0 - pad) * C) & 1);                // first element of the patch's rows: even
+        const int base = (n * H + oh0 - pad) * WC + e0;
+        inside = 0;
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            if (j < rounds) {                                                     // (uniform)
+                const int rr = prp[j] & 0xFF, pp = prp[j] >> 8;
+                const int ih = oh0 - pad + rr, ie = e0 + 2 * pp;
+                const bool in = ih >= 0 && ih < H && ie >= 0 && ie < WC;          // (a row starts and ends at an even element)
+                v[j] = *reinterpret_cast<const uint2*>(xb + (in ? (unsigned)(base + rr * WC + 2 * pp) * 4u : 0u));
+                inside |= in ? 1u << j : 0u;
+            }
+        }
+    };
+    if (tile < ntiles) request(tile);
+#pragma unroll 1
+    while (tile < ntiles) {
+        const int cn = n, coh0 = oh0, cow0 = ow0;                                 // the tile to compute
+        const int shift = ((cow0 - pad) * C) & 1;
+#pragma unroll
+        for (int j = 0; j < NL; ++j)
+            if (j < rounds && 64 * j + lane < npairs) {
+                const unsigned m = 0u - ((inside >> j) & 1u);
+                reinterpret_cast<uint2*>(sP)[64 * j + lane] = make_uint2(v[j].x & m, v[j].y & m);
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        tile += wstride;
+        if (tile < ntiles) request(tile);
+
+#pragma unroll 1
+        for (int g = 0; g < DSF_WR; ++g) {
+            const int oh = coh0 + g;
+            if (oh >= Ho) break;                                                  // wave-uniform
+            const float* pb = sP + g * PPN * 2 + l32 * C + shift;
+            float b[NE];
+#pragma unroll
+            for (int e = 0; e < NE; ++e) b[e] = __uint_as_float(__float_as_uint(pb[off[e]]) & (0u - ((tapmask >> e) & 1u)));
+            // two filter tiles at a time; register r of a lane: pixel 8 (r / 4) + 4 lh + r % 4 of the row's 32 for the
+            // lane's filter of each tile; the upper half of the first tile's register and the lower half of the second's
+            // change places (v_permlane32_swap), and a register holds ONE pixel for 64 filters: a store instruction
+            // writes 256 contiguous bytes when K = 64
+            const unsigned yrow = (unsigned)((cn * Ho + oh) * Wo + cow0) * (unsigned)K;
+#pragma unroll 1
+            for (int kp = 0; kp < KT; kp += 2) {
+                floatx16 acc0, acc1;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc0[r] = 0.f, acc1[r] = 0.f;
+                const float* wk = sW + (size_t)kp * NE * 64 + lane;
+                const bool two = kp + 1 < KT;                                     // (uniform)
+#pragma unroll
+                for (int e = 0; e < NE; ++e) acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(b[e], wk[e * 64], acc0, 0, 0, 0);
+                if (two) {
+#pragma unroll
+                    for (int e = 0; e < NE; ++e) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(b[e], wk[(NE + e) * 64], acc1, 0, 0, 0);
+                }
+                const int k = kp * 32 + lane;
+                const float bk = k < KT * 32 ? sB[k] : 0.f;
+                const bool kok = k < K;
+                unsigned o = yrow + (unsigned)k;                                  // element offsets fit 32 bits (the host checks the sizes)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc0[r]), __float_as_uint(acc1[r]), false, false);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {                                 // pixel 8 (r / 4) + 4 u + r % 4
+                        float val = __uint_as_float(sw[u]) + bk;
+                        if (ep.relu) val = fmaxf(val, 0.f);
+                        if (kok && cow0 + 8 * (r >> 2) + 4 * u + (r & 3) < Wo) y[o + (unsigned)(4 * u) * (unsigned)K] = val;
+                    }
+                    o += ((r & 3) == 3 ? 5u : 1u) * (unsigned)K;
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                   // (the tile's LDS reads before the next tile's writes)
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // Direct 3x3 convolution for layers with FEW OUTPUT PIXELS and a reduction of any length (a batch of one image: the
 // reference's sweep starts at layer 1-2 with batch 1, comparison/layoutCompare.cu:38-46).  Such a layer is a few
 // microseconds of arithmetic; through the Winograd pipelines it is three dependent launches, each of which starts,

@@ -867,6 +867,27 @@ int launch_direct_t(int src, int dst, unsigned flags, const void* bias, const Ge
             LAUNCH_CHECK("direct_small_c_tiles");
             return WINO_OK;
         }
+        if (src == WINO_NHWC && dst == WINO_NHWC && ((long)g.W * g.C) % 2 == 0 && !misaligned(x, 8) &&
+            direct_tiles_nhwc_lds_bytes(g.C, g.K) <= 64 * 1024) {
+            // NHWC on both sides, rows of whole 8-byte pairs: tiles of 4 rows x 32 columns per wave, input through LDS
+            const int tiles_y = (g.Ho + DSF_WR - 1) / DSF_WR, tiles_x = (g.Wo + 31) / 32;
+            const long ntiles = (long)g.N * tiles_y * tiles_x, resident = 16L * device_cus();
+            const long per = (ntiles + resident - 1) / resident;                 // tiles per wave
+            const dim3 tgrid((unsigned)((ntiles + 4 * per - 1) / (4 * per)));
+            const size_t ldst = direct_tiles_nhwc_lds_bytes(g.C, g.K);
+#define DIRECT_TILES_N(NE)                                                                                                     \
+    hipLaunchKernelGGL((direct_small_c_tiles_nhwc_kernel<NE>), tgrid, block, ldst, st, (const float*)x, (const float*)w, (float*)y, \
+                       g.N, g.C, g.K, g.H, g.W, g.pad, g.Ho, g.Wo, tiles_y, tiles_x, (int)ntiles, ep)
+            switch (g.C) {
+            case 1: DIRECT_TILES_N(5); break;
+            case 2: DIRECT_TILES_N(9); break;
+            case 3: DIRECT_TILES_N(14); break;
+            default: DIRECT_TILES_N(18); break;
+            }
+#undef DIRECT_TILES_N
+            LAUNCH_CHECK("direct_small_c_tiles_nhwc");
+            return WINO_OK;
+        }
         switch (g.C) {
         case 1: DIRECT_LAUNCH(5); break;
         case 2: DIRECT_LAUNCH(9); break;
