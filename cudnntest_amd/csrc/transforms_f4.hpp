@@ -265,19 +265,23 @@ __global__ __launch_bounds__(256) void input_transform_f4_vec_kernel(const float
 // ---- input transform, fp32 NHWC source, batch-major tiles: a row of tiles staged in LDS ------------------------
 // In NHWC the channels of a pixel are contiguous and the pixels of a tile are not: a thread per (tile, channel)
 // gathers 4-byte pieces 4 pixels apart.  Here a workgroup takes one image, one tile row, a block of at most 14 tile
-// columns and 32 channels: the 6 x (4*tiles + 2) pixels it needs are loaded 16 bytes per lane, 8 lanes per pixel
-// (128 contiguous bytes; every load unconditional from a clamped address and masked afterwards -- all twelve issued
+// columns and CC channels: the 6 x (4*tiles + 2) pixels it needs are loaded 16 bytes per lane, CC/4 lanes per pixel
+// (every load unconditional from a clamped address and masked afterwards -- all of a lane's loads issued
 // before the first mask, under a branch that is uniform for the workgroup: with the loads inside a per-lane branch
 // the compiler waits for each one before it issues the next, 91 against 73 us on N = 32, C = 256, 56 x 56), and
-// stored to LDS with a pixel pitch of 33 words.  Then one thread per (channel of a vector,
+// stored to LDS with a pixel pitch of CC + 1 words.  Then one thread per (channel of a vector,
 // tile, channel vector), channel fastest as in the layout-generic kernel: its 36 LDS reads hit distinct banks across
 // the wave (bank = 4*tile + channel + const), and the 4 lanes of a vector and the 16 tiles of a wave write 256
 // contiguous bytes of each coordinate plane of V.
-constexpr int F4N_CC = 32, F4N_PITCH = 33, F4N_TCB = 14;
+// Blocks of 16 channels (64-byte pieces of a pixel, 24 KB of LDS, six workgroups to a CU) against 32 and 8, one run,
+// N = 32, C = 256, 56 x 56: 71 us against 75.5 and 79.
+constexpr int F4N_CC = 16, F4N_TCB = 14;
+template <int CC>
 __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const float* __restrict__ x, float* __restrict__ V,
                                                                        int N, int C, int H, int W, int pad, int th,
                                                                        int tw, long Pp, int Cp, int colBlocks, FilterJob fj) {
-    __shared__ float sm[6 * (4 * F4N_TCB + 2) * F4N_PITCH];
+    constexpr int PITCH = CC + 1, L = CC / 4, PP = 256 / L, NQ = (6 * (4 * F4N_TCB + 2) + PP - 1) / PP;   // lanes of a pixel, pixels of a pass, passes
+    __shared__ float sm[6 * (4 * F4N_TCB + 2) * PITCH];
     const int zjob = gridDim.z - N;                          // 1 with a filter job: slice 0, dispatched first
     if (zjob && blockIdx.z == 0) {
         filter_job_f4<float>(fj);
@@ -299,24 +303,24 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
         }
     }
     const int ty = bx / colBlocks, cb = bx - ty * colBlocks;
-    const int c0 = by * F4N_CC;
+    const int c0 = by * CC;
     const int tx0 = cb * F4N_TCB, ntx = min(F4N_TCB, tw - tx0);
     const int wlb = 4 * ntx + 2;                             // pixel columns of the block
     const int h0 = 4 * ty - pad, w0 = 4 * tx0 - pad;
     // ---- pixels -> LDS
-    const int npix = 6 * wlb;                                // <= 348: twelve passes of 32 pixels at most
-    const int ch4 = tid & 7, pl = tid >> 3;                  // 16-byte piece of the 32 channels; pixel of a pass
+    const int npix = 6 * wlb;                                // <= 348: NQ passes of PP pixels at most
+    const int ch4 = tid & (L - 1), pl = tid / L;             // 16-byte piece of the CC channels; pixel of a pass
     const unsigned inv_wlb = (65536u + (unsigned)wlb - 1u) / (unsigned)wlb;      // pix / wlb = pix * inv_wlb >> 16 for pix < 348
     const char* const xn = reinterpret_cast<const char*>(x) + (size_t)n * H * W * C * sizeof(float);   // the image (uniform)
     const int c = c0 + 4 * ch4;
-    const bool vec = (C & 3) == 0 && c0 + F4N_CC <= C;         // uniform: every lane of the workgroup loads 16 bytes
-    float4 raw[12];
-    unsigned keep[12];
+    const bool vec = (C & 3) == 0 && c0 + CC <= C;         // uniform: every lane of the workgroup loads 16 bytes
+    float4 raw[NQ];
+    unsigned keep[NQ];
     if (vec) {
         // (all loads first, unconditionally, from clamped addresses; the masks afterwards: the loads are in flight together)
 #pragma unroll
-        for (int q = 0; q < 12; ++q) {
-            const int pix = min(pl + 32 * q, npix - 1);
+        for (int q = 0; q < NQ; ++q) {
+            const int pix = min(pl + PP * q, npix - 1);
             const int r = (int)(((unsigned)pix * inv_wlb) >> 16), col = pix - r * wlb;
             const int ih = h0 + r, iw = w0 + col;
             const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
@@ -326,12 +330,12 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
             raw[q] = *reinterpret_cast<const float4*>(xn + off);
         }
 #pragma unroll
-        for (int q = 0; q < 12; ++q)
+        for (int q = 0; q < NQ; ++q)
             raw[q] = make_float4(mask_keep(raw[q].x, keep[q]), mask_keep(raw[q].y, keep[q]), mask_keep(raw[q].z, keep[q]), mask_keep(raw[q].w, keep[q]));
     } else {
 #pragma unroll
-        for (int q = 0; q < 12; ++q) {
-            const int pix = min(pl + 32 * q, npix - 1);
+        for (int q = 0; q < NQ; ++q) {
+            const int pix = min(pl + PP * q, npix - 1);
             const int r = (int)(((unsigned)pix * inv_wlb) >> 16), col = pix - r * wlb;
             const int ih = h0 + r, iw = w0 + col;
             const bool ok = ih >= 0 && ih < H && iw >= 0 && iw < W;
@@ -345,17 +349,17 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
         }
     }
 #pragma unroll
-    for (int q = 0; q < 12; ++q) {
-        const int pix = pl + 32 * q;
+    for (int q = 0; q < NQ; ++q) {
+        const int pix = pl + PP * q;
         if (pix < npix) {
-            float* d = sm + pix * F4N_PITCH + 4 * ch4;
+            float* d = sm + pix * PITCH + 4 * ch4;
             d[0] = raw[q].x; d[1] = raw[q].y; d[2] = raw[q].z; d[3] = raw[q].w;
         }
     }
     __syncthreads();
     // ---- tiles
     const size_t vplane_bytes = (size_t)Cp * Pp * sizeof(float);
-    const int nvec = min(F4N_CC, Cp - c0) / 4;               // channel vectors of this workgroup (Cp is a multiple of 16)
+    const int nvec = min(CC, Cp - c0) / 4;               // channel vectors of this workgroup (Cp is a multiple of 16)
     const long p0 = ((long)n * th + ty) * tw + tx0;
     const unsigned inv_ntx = (65536u + (unsigned)ntx - 1u) / (unsigned)ntx;
     // a thread's 36 stores: a uniform plane base that moves on by a plane, and one 32-bit offset (a plane is < 2^32 bytes)
@@ -363,13 +367,13 @@ __global__ __launch_bounds__(256) void input_transform_f4_nhwc_kernel(const floa
     for (int idx = tid; idx < nvec * ntx * 4; idx += 256) {
         const int e = idx & 3, it = idx >> 2;
         const int ql = (int)(((unsigned)it * inv_ntx) >> 16), t = it - ql * ntx;
-        const float* src = sm + (4 * t) * F4N_PITCH + 4 * ql + e;
+        const float* src = sm + (4 * t) * PITCH + 4 * ql + e;
         float d[6][6], v[36];
 #pragma unroll
         for (int i = 0; i < 6; ++i) {
-            const float* row = src + i * wlb * F4N_PITCH;
+            const float* row = src + i * wlb * PITCH;
 #pragma unroll
-            for (int j = 0; j < 6; ++j) d[i][j] = row[j * F4N_PITCH];
+            for (int j = 0; j < 6; ++j) d[i][j] = row[j * PITCH];
         }
         input_tile_transform_f4(d, v);
         const unsigned voff = (unsigned)(((size_t)ql * Pp + t) * 16 + e * 4);

@@ -598,8 +598,8 @@ int launch_f4_input(int layout, int order, const Geometry& g, const void* x, voi
             if (rc) return rc;
         }
         if (ride) grid.z += 1;
-        hipLaunchKernelGGL(input_transform_f4_nhwc_kernel, grid, dim3(256), 0, st, (const float*)x, (float*)V, g.N, g.C, g.H, g.W,
-                           g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, ride ? fj : FilterJob{});
+        hipLaunchKernelGGL(input_transform_f4_nhwc_kernel<F4N_CC>, grid, dim3(256), 0, st, (const float*)x, (float*)V, g.N, g.C, g.H,
+                           g.W, g.pad, g.th, g.tw, g.Pp, g.Cp, colBlocks, ride ? fj : FilterJob{});
         LAUNCH_CHECK("f4_input_transform_nhwc");
         return WINO_OK;
     }
