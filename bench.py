@@ -74,6 +74,8 @@ MEASURED_TRAFFIC = {
     # the GEMM of the F(4x4) pipeline (gemm_128x128_walk_spread_kernel): 320.8 MB fetched + 231.2 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "staged_f4"):
         (552.1e6, "profiles/staged_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
+    ("vgg16_conv3_N32_C256_K256_H56", "NHWC", "f32", "staged_f4"):
+        (554.3e6, "profiles/staged_f4_fp32_nhwc_vgg16_conv3_N32_counters.txt"),   # 323.1 MB fetched + 231.2 MB written
     # gemm_rows_f4_kernel: 1435.0 MB fetched (a patch's rows of V once per filter tile, most of it from the L2) + 515.0 MB written
     ("vgg16_conv3_N32_C256_K256_H56", "NCHW", "f32", "epilogue_f4"):
         (1949.9e6, "profiles/epilogue_f4_fp32_nchw_vgg16_conv3_N32_counters.txt"),
