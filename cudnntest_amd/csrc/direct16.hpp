@@ -52,14 +52,15 @@ struct D16Geom {
     long G;                // N * Ho output rows
 };
 
-// ---- 2x2 / stride-2 maximum of a [K][Ho][Wo][N] tensor of 2-byte elements ---------------------------------
+// ---- 2x2 / stride-2 maximum of a tensor the direct kernels wrote unpooled ------------------------------------
 // The 8-wave kernel pools in its stores where a window's columns sit in neighbouring lanes; in a CHWN tensor they are N
-// elements apart, in different waves.  Such a layer is convolved unpooled (bias and ReLU applied) into scratch and this
-// kernel follows: a thread takes VEC images of one window.  max(round(v)) = round(max(v)): the same bits as a kernel
-// that pooled before it rounded.
+// elements apart, in different waves, and the kernels for layers of at most four channels do not pool.  Such a layer is
+// convolved unpooled (bias and ReLU applied) into scratch and one of these kernels follows.
+// max(round(v)) = round(max(v)): the same bits as a kernel that pooled before it rounded.
+// [outer][Ho][Wo][inner] (CHWN: K, N; NHWC: N, K): a thread takes VEC inner elements of one window.
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void pool2_chwn_kernel(const T* __restrict__ t, T* __restrict__ y, int Ho, int Wo, int N,
-                                                         long total) {
+__global__ __launch_bounds__(256) void pool2_inner_kernel(const T* __restrict__ t, T* __restrict__ y, int Ho, int Wo, int N,
+                                                          long total) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const int nv = N / VEC, Hp = Ho >> 1, Wp = Wo >> 1;
@@ -70,13 +71,34 @@ __global__ __launch_bounds__(256) void pool2_chwn_kernel(const T* __restrict__ t
     const int ph = (int)(r % Hp);
     const long k = r / Hp;
     const T* src = t + ((k * Ho + 2 * ph) * Wo + 2 * pw) * (long)N + n0;
-    struct alignas(VEC * 2) Vec { T v[VEC]; };
+    struct alignas(VEC * sizeof(T)) Vec { T v[VEC]; };
     const Vec a = *reinterpret_cast<const Vec*>(src), b = *reinterpret_cast<const Vec*>(src + N);
     const Vec c = *reinterpret_cast<const Vec*>(src + (long)Wo * N), d = *reinterpret_cast<const Vec*>(src + (long)Wo * N + N);
     Vec o;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) o.v[e] = from_f32<T>(fmaxf(fmaxf(to_f32(a.v[e]), to_f32(b.v[e])), fmaxf(to_f32(c.v[e]), to_f32(d.v[e]))));
     *reinterpret_cast<Vec*>(y + ((k * Hp + ph) * Wp + pw) * (long)N + n0) = o;
+}
+// [planes][Ho][Wo] (NCHW: N x K planes): a thread takes VEC neighbouring windows of a row pair, 2 VEC contiguous
+// elements of each row (VEC > 1: Wo a multiple of 2 VEC and both tensors aligned to the pieces).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void pool2_rows_kernel(const T* __restrict__ t, T* __restrict__ y, int Ho, int Wo, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int Hp = Ho >> 1, Wp = Wo >> 1, wv = Wp / VEC;
+    const int pw0 = (int)(i % wv) * VEC;
+    long r = i / wv;
+    const int ph = (int)(r % Hp);
+    const long plane = r / Hp;
+    const T* src = t + (plane * Ho + 2 * ph) * (long)Wo + 2 * pw0;
+    struct alignas(2 * VEC * sizeof(T)) In { T v[2 * VEC]; };
+    struct alignas(VEC * sizeof(T)) Out { T v[VEC]; };
+    const In a = *reinterpret_cast<const In*>(src), b = *reinterpret_cast<const In*>(src + Wo);
+    Out o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        o.v[e] = from_f32<T>(fmaxf(fmaxf(to_f32(a.v[2 * e]), to_f32(a.v[2 * e + 1])), fmaxf(to_f32(b.v[2 * e]), to_f32(b.v[2 * e + 1]))));
+    *reinterpret_cast<Out*>(y + (plane * Hp + ph) * (long)Wp + pw0) = o;
 }
 
 // ---- filter bank -> W9[tap][Cp/8][Kp][8] (zero padded) --------------------------------------------------

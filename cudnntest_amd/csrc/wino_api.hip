@@ -751,8 +751,8 @@ int tile_order_for(int src, int /*dst*/) {
 // the transformed tensors cost relative to the multiplies, and the more fusion pays.
 // Chosen from sweeps of the VGG-16 shapes over the three algorithms, per layout and element type.
 // ---- direct convolution of layers with C <= 4 ----------------------------------------
-// lanes along the contiguous axis of y (w for NCHW, n for CHWN, k for NHWC); pooled outputs stay on the
-// Winograd path
+// lanes along the contiguous axis of y (w for NCHW, n for CHWN, k for NHWC); the kernels do not pool: a pooled layer
+// runs unpooled into scratch and a pooling kernel follows (direct_pooled_ok)
 bool direct_ok(int dst, unsigned flags, const Geometry& g) {
     const size_t lds = direct_lds_bytes(g.C, g.K);
     return lds != 0 && lds <= 64 * 1024 && !(flags & WINO_FLAG_POOL2) && g.pad <= 1 &&
@@ -1212,23 +1212,47 @@ bool direct16_chwn_pool_ok(int src, int dst, int dtype, unsigned flags, const Ge
 size_t direct16_unpooled_bytes(int dtype, const Geometry& g) {
     return ((size_t)g.N * g.K * g.Ho * g.Wo * dtype_size(dtype) + 255) / 256 * 256;
 }
+// 2x2 pooling of an unpooled tensor in scratch (aligned) into y, [outer][Ho][Wo][inner] or, inner == 1, planes of rows
 template <typename T>
-int launch_pool2_chwn_t(const Geometry& g, const void* tmp, void* y, hipStream_t st) {
-    const int vec = g.N % 8 == 0 && !misaligned(y, 16) ? 8 : g.N % 2 == 0 && !misaligned(y, 4) ? 2 : 1;   // (tmp is scratch: aligned)
-    const long total = (long)g.K * (g.Ho / 2) * (g.Wo / 2) * (g.N / vec);
+int launch_pool2_t(int layout, const Geometry& g, const void* tmp, void* y, hipStream_t st) {
+    const int Hp = g.Ho / 2, Wp = g.Wo / 2;
+    if (layout == WINO_NCHW) {
+        constexpr int V = 8 / (int)sizeof(T);                                // 16-byte loads, 8-byte stores
+        const bool wide = g.Wo % (2 * V) == 0 && !misaligned(y, 8);
+        const long total = (long)g.N * g.K * Hp * (wide ? Wp / V : Wp);
+        const dim3 grid((unsigned)((total + 255) / 256));
+        if (wide) hipLaunchKernelGGL((pool2_rows_kernel<T, V>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, total);
+        else hipLaunchKernelGGL((pool2_rows_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, total);
+        LAUNCH_CHECK("pool2_rows");
+        return WINO_OK;
+    }
+    const int inner = layout == WINO_CHWN ? g.N : g.K, outer = layout == WINO_CHWN ? g.K : g.N;
+    constexpr int V = 16 / (int)sizeof(T);
+    const int vec = inner % V == 0 && !misaligned(y, 16) ? V : inner % 2 == 0 && !misaligned(y, 2 * sizeof(T)) ? 2 : 1;
+    const long total = (long)outer * Hp * Wp * (inner / vec);
     const dim3 grid((unsigned)((total + 255) / 256));
-    if (vec == 8) hipLaunchKernelGGL((pool2_chwn_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, g.N, total);
-    else if (vec == 2) hipLaunchKernelGGL((pool2_chwn_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, g.N, total);
-    else hipLaunchKernelGGL((pool2_chwn_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, g.N, total);
-    LAUNCH_CHECK("pool2_chwn");
+    if (vec == V) hipLaunchKernelGGL((pool2_inner_kernel<T, V>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, inner, total);
+    else if (vec == 2) hipLaunchKernelGGL((pool2_inner_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, inner, total);
+    else hipLaunchKernelGGL((pool2_inner_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)tmp, (T*)y, g.Ho, g.Wo, inner, total);
+    LAUNCH_CHECK("pool2_inner");
     return WINO_OK;
 }
 int launch_direct16_chwn_pooled(int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
                                 void* W9, void* tmp, void* y, hipStream_t st, int mode) {
     const int rc = launch_direct16(WINO_CHWN, WINO_CHWN, dtype, flags & ~(unsigned)WINO_FLAG_POOL2, bias, g, x, w, W9, tmp, st, mode);
     if (rc || mode == D16_PACK) return rc;
-    if (dtype == WINO_F16) return launch_pool2_chwn_t<f16_t>(g, tmp, y, st);
-    return launch_pool2_chwn_t<bf16_t>(g, tmp, y, st);
+    if (dtype == WINO_F16) return launch_pool2_t<f16_t>(WINO_CHWN, g, tmp, y, st);
+    return launch_pool2_t<bf16_t>(WINO_CHWN, g, tmp, y, st);
+}
+// pooled layers of at most four channels: the layer unpooled into `tmp` (room for direct16_unpooled_bytes), then pooling
+bool direct_pooled_ok(int dst, unsigned flags, const Geometry& g) {
+    return (flags & WINO_FLAG_POOL2) && direct_ok(dst, flags & ~(unsigned)WINO_FLAG_POOL2, g);
+}
+int launch_direct_pooled(int src, int dst, int dtype, unsigned flags, const void* bias, const Geometry& g, const void* x, const void* w,
+                         void* tmp, void* y, hipStream_t st) {
+    const int rc = launch_direct(src, dst, dtype, flags & ~(unsigned)WINO_FLAG_POOL2, bias, g, x, w, tmp, st);
+    if (rc) return rc;
+    DISPATCH_DTYPE(dtype, launch_pool2_t<T>(dst, g, tmp, y, st));
 }
 
 int pick_algo(int layout, int dtype, const Geometry& g) {
@@ -1330,7 +1354,9 @@ bool auto_f4(int dtype, const Geometry& g) {
     return tiles4 >= 512;
 }
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y, bool have_w) {
-    if (have_w && direct_ok(dst, flags, g)) return WINO_ALGO_DIRECT;
+    // (a pooled layer of at most four channels: direct into scratch, then pooling -- the network's first layer shape with
+    // pooling, N = 32: bf16 NCHW 59 + 31 us against 242 for the Winograd pipeline that pools in its output stage)
+    if (have_w && (direct_ok(dst, flags, g) || direct_pooled_ok(dst, flags, g))) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x, y)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct_few(src, dtype, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_f4(dtype, g)) return WINO_ALGO_STAGED_F4;
@@ -1385,12 +1411,36 @@ int conv_f4_impl(const ScratchSource& ss, int src, int dst, int dtype, int algo,
     DISPATCH_DTYPE(dtype, launch_f4_output<T>(dst, order, porder, flags, bias, N, K, g.Ho, g.Wo, g.Kp, g.P, g.Pp, Mo, y, st));
 }
 
-// What the automatic choice runs when its first choice does not fit a fixed scratch buffer: a pooled CHWN layer on the
-// direct path keeps the unpooled tensor in scratch; without room for it the Winograd pipelines take the layer.
+// Images per pass of a pooled layer of at most four channels (0: no room).  The unpooled tensor of a pass stays under
+// 224 MB, so that the last-level cache still holds it when the pooling kernel reads it (fp32, N = 32, 64 filters at
+// 224 x 224, 411 MB unpooled: 236 us in one pass, 179 in two; NHWC 256 and 204), and inside a fixed scratch buffer.
+// CHWN tensors are not cut: their images are the contiguous axis.
+int direct_pooled_images(const ScratchSource& ss, int src, int dst, int dtype, const Geometry& g) {
+    if (src == WINO_CHWN || dst == WINO_CHWN)
+        return !ss.fixed || kCounterBytes + direct16_unpooled_bytes(dtype, g) <= ss.fixed_bytes ? g.N : 0;
+    const size_t img = (size_t)g.K * g.Ho * g.Wo * dtype_size(dtype);
+    size_t lim = (size_t)224 << 20;
+    if (ss.fixed) lim = std::min(lim, ss.fixed_bytes > kCounterBytes + 256 ? ss.fixed_bytes - kCounterBytes - 256 : 0);
+    long fit = (long)(lim / img);
+    if (fit < 1 && !ss.fixed) fit = 1;
+    if (fit < 1) return 0;
+    const long passes = (g.N + fit - 1) / fit;
+    return (int)((g.N + passes - 1) / passes);
+}
+
+// What the automatic choice runs when its first choice does not fit a fixed scratch buffer: a pooled CHWN layer and a
+// pooled layer of at most four channels on the direct path keep the unpooled tensor in scratch; without room for it the
+// Winograd pipelines take the layer.
 int auto_within(const ScratchSource& ss, int algo, int src, int dst, int dtype, unsigned flags, const Geometry& g) {
-    if (algo == WINO_ALGO_DIRECT && ss.fixed && direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
-        kCounterBytes + (direct16_bank_bytes(g) + 255) / 256 * 256 + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) {
+    if (algo == WINO_ALGO_DIRECT && ss.fixed &&
+        ((direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
+          kCounterBytes + (direct16_bank_bytes(g) + 255) / 256 * 256 + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) ||
+         (direct_pooled_ok(dst, flags, g) && direct_pooled_images(ss, src, dst, dtype, g) == 0))) {
         algo = pick_algo(src, dtype, g);
+        // (the single kernel keeps only the transformed filters in scratch: it runs where the others' tensors do not fit)
+        if (algo != WINO_ALGO_FUSED && g.pad <= 1 && scratch_layout(g, dtype, algo).total > ss.fixed_bytes &&
+            (long)g.N * g.C * g.H * g.W * (long)dtype_size(dtype) < (1L << 32))
+            algo = WINO_ALGO_FUSED;
         if (algo == WINO_ALGO_FUSED && g.pad > 1) algo = WINO_ALGO_EPILOGUE;
     }
     return algo;
@@ -1422,6 +1472,24 @@ int conv_pass(const ScratchSource& ss, int src, int dst, int dtype, int algo, un
         if (direct_ok(dst, flags, g)) {
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
             return launch_direct(src, dst, dtype, flags, bias, g, x, w, y, (hipStream_t)stream);
+        }
+        if (direct_pooled_ok(dst, flags, g)) {
+            const int per = direct_pooled_images(ss, src, dst, dtype, g);
+            if (per == 0) return fail(WINO_ERR_WORKSPACE, "an image of this layer unpooled does not fit the scratch buffer");
+            Geometry gp;
+            make_geometry(dtype, per, C, K, H, W, pad, &gp);
+            void* base = nullptr;
+            const int rcb = ss.get(kCounterBytes + direct16_unpooled_bytes(dtype, gp), &base);
+            if (rcb) return rcb;
+            StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);
+            const size_t es = dtype_size(dtype), x_img = (size_t)C * H * W * es, y_img = (size_t)K * (g.Ho / 2) * (g.Wo / 2) * es;
+            for (int n0 = 0; n0 < g.N; n0 += per) {
+                make_geometry(dtype, std::min(per, g.N - n0), C, K, H, W, pad, &gp);
+                const int rc = launch_direct_pooled(src, dst, dtype, flags, bias, gp, (const char*)x + n0 * x_img, w, (char*)base + kCounterBytes,
+                                                    (char*)y + n0 * y_img, (hipStream_t)stream);
+                if (rc) return rc;
+            }
+            return WINO_OK;
         }
         if (direct_few_ok(dtype, flags, g)) {
             StageScope t(WINO_STAGE_GEMM, (hipStream_t)stream);

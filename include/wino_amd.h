@@ -77,7 +77,9 @@ typedef enum {
                                any layout pair, any padding, bias and ReLU but no pooling;
                                layers with C <= 4 (the network's first layer, which the reference runs through
                                the same wrappers: comparison/layoutCompare.cu:38-46): the 9*C <= 36 products of an
-                               output as one short MFMA reduction, any layout, fp32 or 2-byte;
+                               output as one short MFMA reduction, any layout, fp32 or 2-byte; with 2x2 pooling the
+                               layer runs unpooled into scratch, at most 224 MB of images at a time, and a pooling
+                               kernel follows;
                                2-byte NCHW -> NCHW layers with C a multiple of 8, an even width and a 4-byte aligned
                                x: an implicit GEMM on the 16-bit instruction with fp32 accumulation -- with 2-byte
                                operands the Winograd pipelines are bound by the transformed input in memory, the
@@ -94,8 +96,8 @@ typedef enum {
                                pooling in the kernel's stores for 32 images and an even width, otherwise the layer runs
                                unpooled into scratch (N*K*Ho*Wo elements) and a pooling kernel follows; other CHWN
                                layers, and layers with CHWN on one side only, are refused.
-                               Bias and ReLU; 2x2 pooling for the 2-byte layers that run on the 8-wave kernel (the
-                               shape just named), not for C <= 4; needs the filter bank itself (not
+                               Bias and ReLU; 2x2 pooling for C <= 4 and for the 2-byte layers that run on the
+                               8-wave kernel (the shape just named); needs the filter bank itself (not
                                wino_conv_prepared).
                                What WINO_ALGO_AUTO picks for C <= 4 and for large 2-byte NCHW, NHWC and CHWN layers. */
     WINO_ALGO_EPILOGUE_F4 = 6 /* F(4x4,3x3) with the output transform A^T (.) A in the epilogue of the 36-way GEMM: no

@@ -87,14 +87,39 @@ def test_floats_within_tolerance_and_auto_takes_the_path(oracle, layout, dtype):
     assert oracle.rel_l2(host(fused), host(got)) <= (1e-5 if dtype == ops.F32 else TOL[dtype])
 
 
+POOLED_SHAPES = [(2, 3, 64, 40, 70), (1, 4, 70, 18, 34), (3, 1, 33, 17, 32), (2, 2, 40, 33, 66), (32, 3, 64, 9, 6), (8, 3, 16, 2, 3)]
+
+
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
+@pytest.mark.parametrize("dtype", [ops.F32, ops.F16, ops.BF16])
+@pytest.mark.parametrize("shape", POOLED_SHAPES)
+def test_pooled_few_channel_layers_bit_exact(oracle, shape, dtype, layout):
+    """Bias, ReLU and 2x2 pooling on a layer of at most four channels: the direct kernel writes the unpooled tensor into
+    scratch and a pooling kernel follows (rows of planes for NCHW, 16-byte pieces where the width allows; vectors of the
+    contiguous axis for NHWC and CHWN).  Odd output heights and widths drop their last row and column; pad 0 and 1.
+    Integers: bit-exact against the pooled oracle; the automatic choice runs the same kernels."""
+    N, C, K, H, W = shape
+    x = synth.small_ints(N * C * H * W, sum(shape), -2, 2).reshape(N, C, H, W)
+    w = synth.small_ints(K * C * 9, 7 + sum(shape), -1, 1).reshape(K, C, 3, 3)
+    bias = synth.small_ints(K, 3, -2, 2).astype(np.float32)
+    xs, ws = synth.act_to_layout(x, layout), synth.flt_to_layout(w, layout)
+    for pad in (1, 0):
+        Ho, Wo = H + 2 * pad - 2, W + 2 * pad - 2
+        if Ho < 2 or Wo < 2:
+            continue
+        full = np.maximum(oracle.direct_conv(x, w, pad) + bias[None, :, None, None], 0).astype(np.float32)
+        Hp, Wp = Ho // 2, Wo // 2
+        want = full[:, :, :2 * Hp, :2 * Wp].reshape(N, K, Hp, 2, Wp, 2).max(axis=(3, 5))
+        want = synth.act_to_layout(np.ascontiguousarray(want), layout)
+        got = ops.conv(dev(xs, dtype), dev(ws, dtype), pad, layout, algo=ops.ALGO_DIRECT, relu=True, pool=True, bias=dev(bias, dtype))
+        assert np.array_equal(host(got), want), pad
+        auto = ops.conv(dev(xs, dtype), dev(ws, dtype), pad, layout, relu=True, pool=True, bias=dev(bias, dtype))
+        assert torch.equal(auto, got), pad
+
+
 def test_what_the_path_is_not_built_for():
     x = torch.zeros((1, 3, 8, 8), device="cuda")
     w = torch.zeros((4, 3, 3, 3), device="cuda")
-    for kwargs in (dict(pool=True),):
-        with pytest.raises(_lib.WinoError) as e:
-            ops.conv(x, w, algo=ops.ALGO_DIRECT, **kwargs)
-        assert e.value.code == -2
-        ops.conv(x, w, **kwargs)                     # AUTO falls back to the Winograd kernels
     with pytest.raises(_lib.WinoError) as e:         # five channels and more output pixels than the small-layer kernel takes
         ops.conv(torch.zeros((64, 5, 58, 58), device="cuda"), torch.zeros((64, 5, 3, 3), device="cuda"), algo=ops.ALGO_DIRECT)
     assert e.value.code == -2

@@ -98,3 +98,19 @@ def test_pooled_chwn_layers_with_and_without_room_for_the_unpooled_tensor(oracle
         got, want = both(dev(x, ops.BF16), dev(w, ops.BF16), bias, ops.CHWN, ops.ALGO_AUTO, relu=True, pool=True)
         assert (N * K * H * H * 2 > LIMIT) == (H == 160)
         assert torch.equal(got, want), H
+
+
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
+def test_pooled_first_layers_with_and_without_room_for_the_unpooled_tensor(oracle, layout):
+    """The same for a pooled layer of three channels (direct into scratch, then the pooling kernel): N = 32, K = 64 in
+    bf16 at 56 x 56 (12.8 MB unpooled) and at 160 x 160 (105 MB: NCHW and NHWC layers run in two passes of 16 images,
+    a CHWN layer, whose images cannot be cut, goes to the single Winograd kernel, which keeps only its filters in
+    scratch)."""
+    for H in (56, 160):
+        N, C, K = 32, 3, 64
+        x, w = synth.conv_inputs(N, C, K, H, H, seed=H, layout=layout, integer=True)
+        bias = dev(synth.small_ints(K, seed=4, lo=-2, hi=2).astype(np.float32), ops.BF16)
+        got, want = both(dev(x, ops.BF16), dev(w, ops.BF16), bias, layout, ops.ALGO_AUTO, relu=True, pool=True)
+        assert (N * K * H * H * 2 > LIMIT) == (H == 160)
+        assert torch.equal(got, want), H
+
