@@ -1269,7 +1269,9 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
         // With one filter tile (K <= 64) no tile is transformed twice, whatever C (C = 256, K = 64, H = 56:
         // 0.185 against 0.233 ms); with two, the single kernel needs many patches to win (C = K = 128: 196
         // patches 0.067 against 0.062 ms for EPILOGUE, 392 a tie, 12544 0.57 against 0.63)
-        if (fused_ok && g.K <= 64 && g.C <= 256) return WINO_ALGO_FUSED;
+        // (and past C = 256: C = 384, K = 64, N = 8, H = 112: 0.27 against 0.35 and 0.46 ms for the other two; C = 512,
+        // K = 32, N = 32, H = 56: 0.35 against 0.47 and 0.59)
+        if (fused_ok && g.K <= 64) return WINO_ALGO_FUSED;
         if (g.C <= 128 && g.K <= 128) return (fused_ok && patches >= 512) ? WINO_ALGO_FUSED : WINO_ALGO_EPILOGUE;
         if (patches < 256) return WINO_ALGO_STAGED;      // not even one 64x64 patch per CU
         if (g.C <= 256) return WINO_ALGO_EPILOGUE;
@@ -1283,13 +1285,20 @@ int pick_algo(int layout, int dtype, const Geometry& g) {
     // 16-bit operands: the fp32 product tensor is the largest HBM stream, so STAGED only for tiny problems;
     // the in-kernel input transform is VALU work repeated per filter tile and pays only with few filter
     // tiles and cheap loads (channel vectors for NHWC, which need C % 8 == 0)
-    if (patches < 64 || (g.C >= 256 && patches < 128) || (g.C >= 512 && patches < 256)) return WINO_ALGO_STAGED;
+    // (the last of these with more than one filter tile only: C = 512, K = 16 .. 64, N = 16, H = 56, 196 patches: EPILOGUE
+    // takes 92 to 107 us where STAGED takes 142 to 150)
+    if (patches < 64 || (g.C >= 256 && patches < 128) || (g.C >= 512 && g.K > 64 && patches < 256)) return WINO_ALGO_STAGED;
     if (!fused_ok) return WINO_ALGO_EPILOGUE;
     if (nhwc) {
         // (one filter tile: any C up to 256; two: only with many patches -- C = K = 128 at 196 patches is 6 % behind EPILOGUE)
-        if (g.C >= 16 && g.K <= 64 && g.C <= 256) return WINO_ALGO_FUSED;
+        // (a sweep of 720 bf16 NHWC layers: with one filter tile the single kernel wins at any C once there are some 400
+        // patches -- C = 512, K = 32, N = 16, H = 80: 125 against 233 us -- and from C = 8 on; with fewer patches and more
+        // than 64 channels it is 1.2 to 1.5 times behind -- C = 192, K = 16, N = 8, H = 48: 1.49)
+        if (g.C >= 8 && g.K <= 64 && (g.C <= 64 || patches >= 384)) return WINO_ALGO_FUSED;
         if (g.C >= 16 && g.C <= 128 && g.K <= 128 && patches >= 1024) return WINO_ALGO_FUSED;
     } else if (g.C <= 64 && g.K <= 64 && patches >= 1536) {   // (fewer patches: measured behind EPILOGUE)
+        return WINO_ALGO_FUSED;
+    } else if (g.C >= 384 && g.K <= 64 && patches >= 384) {   // (CHWN, C = 384, K = 64, N = 32, H = 56: 1.35 times faster than EPILOGUE)
         return WINO_ALGO_FUSED;
     }
     return WINO_ALGO_EPILOGUE;
@@ -1317,13 +1326,22 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
         // (measured at N = 32 in bf16, direct against the fastest Winograd pipeline: 177 against 532 us at C = K = 64,
         // H = 224; 140 against 307 at C = K = 128, H = 112; 73 against 91 and 130 against 183 at 56 x 56; at 28 x 28 the
         // 7 x 7 blocks of a filter tile leave a quarter of the chip idle: 121 against 72, 225 against 128 us)
-        return planc && g.Ho >= 48 && g.Wo >= 48 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus();
+        // (fewer than 64 channels, which the network does not have: C = 8 .. 32, K = 128 and 256, 56 x 56 to 112 x 112: 0.53
+        // to 0.81 of the fastest Winograd pipeline's time)
+        return planc && g.Ho >= 48 && g.Wo >= 48 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus();
     }
     const bool plan8 = direct16_rows_wf(g) == 2 ? direct16_rows_plan<2>(g, &d, src == WINO_NHWC) : direct16_rows_plan<1>(g, &d, src == WINO_NHWC);
-    if (plan8 && g.Ho >= 28 && g.Wo >= 28 && g.C >= 64 && 4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus()) return true;
-    if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 48 || g.Wo < 48) return false;
+    // (with an NHWC side and fewer than 64 channels, C = 8 .. 32: 0.45 to 0.83 of the fastest Winograd pipeline's time)
+    if (plan8 && g.Ho >= 28 && g.Wo >= 28 && (g.C >= 64 || src == WINO_NHWC || dst == WINO_NHWC) &&
+        4L * d.rowBlocks * d.colBlocks * d.kTiles >= 3L * device_cus())
+        return true;
+    // (the general kernel: a sweep of 780 bf16 NCHW layers, C = 8 .. 512, K = 16 .. 256, 28 x 28 to 224 x 224, N = 1 .. 32,
+    // against the fastest Winograd pipeline: it wins on 85 % of them, by 1.28 in the geometric mean; it loses where few
+    // tiles each carry a long reduction for two filter tiles one after the other -- N = 8, C = 512, K = 96, H = 48, 96
+    // tiles: 94 against 53 us -- so: a tile for every CU, or one filter tile, or a short reduction)
+    if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 28 || g.Wo < 28) return false;
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
-    return tiles >= 2L * device_cus();
+    return tiles >= device_cus() || g.K <= D16_KT || g.C <= 128;
 }
 // Small fp32 layers go to the one-launch direct kernel while its cost stays small: a round of the chip costs a fixed
 // part (the first group's trip to memory, the sum over the waves, the stores) and a part per group of 32 channels.
@@ -1338,7 +1356,10 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
 bool auto_direct_few(int src, int dtype, unsigned flags, const Geometry& g) {
     if (!direct_few_ok(dtype, flags, g)) return false;
     const long rounds = (direct_few_units(g) + device_cus() - 1) / device_cus(), groups = (g.C + 31) / 32;
-    return direct_few_filter_mode(src, g) ? rounds * (1 + groups) <= 10 : rounds * groups <= 2;
+    // (a sweep of 560 shapes, NCHW, against the fastest pipeline: at rounds x (1 + groups) = 12 the kernel takes 0.59 to
+    // 0.98 of its time, at 14 and 16 with at most 64 filters 0.60 to 0.99; at 17 and more, or 15 with 128 filters, it loses)
+    const long cost = rounds * (1 + groups);
+    return direct_few_filter_mode(src, g) ? cost <= 12 || (cost <= 16 && g.K <= 64) : rounds * groups <= 2;
 }
 // fp32 layers with a long reduction and enough 4x4 tiles run faster through the F(4x4,3x3) pipeline, product tensor
 // and all: 2.25 multiplies per output instead of 4, and a transformed input of 2.25x the tensor instead of 4x.
@@ -1348,15 +1369,32 @@ bool auto_direct_few(int src, int dtype, unsigned flags, const Geometry& g) {
 // (the single-kernel path); C = K = 128, H = 56: 0.14 against 0.18; C = 64, K = 128, H = 112: 0.36 against 0.31.
 // (NHWC: 0.40 against 0.53 on the first of these, CHWN 0.38 against 0.52.)  Its rounding error is about four times
 // that of F(2x2) (3e-6 to 5e-6 relative L2 on these layers).
+// Beyond those shapes (sweeps of 680 layers with C = 8 .. 512, K = 16 .. 512, 7 x 7 to 160 x 160, N = 1 .. 64, NCHW,
+// every pipeline by name; F(4x4) against the fastest F(2x2) pipeline):
+//   * more than one filter tile (K > 64) and C >= 96: F(4x4) takes 0.69 to 0.95 of the time at every size measured
+//     (C = 128, K = 96, N = 32, H = 112: 0.47 against 0.55 ms; C = 192, K = 96, N = 16, H = 80: 0.18 against 0.26);
+//   * K > 64 and 48 <= C < 96: it wins while V and the product together stay inside the 256 MB last-level cache
+//     (C = 64, K = 128, N = 32, H = 56, 177 MB: 0.085 against 0.107 ms) and loses beyond (N = 32, H = 112, 694 MB:
+//     0.36 against 0.31);
+//   * one filter tile (K <= 64): the single kernel transforms no tile twice and wins from about 400 patches on
+//     whatever C (C = 192, K = 64, N = 32, H = 80: 0.26 against 0.31 ms); with fewer patches it leaves the chip half
+//     empty and F(4x4) wins from C = 96 (C = 192, K = 64, N = 4, H = 80: 0.056 against 0.082).
 bool auto_f4(int dtype, const Geometry& g) {
-    if (dtype != WINO_F32 || g.C < 128 || g.K < 128) return false;
+    if (dtype != WINO_F32) return false;
     const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
-    return tiles4 >= 512;
+    if (tiles4 < 512) return false;
+    if (g.C >= 128 && g.K >= 128) return true;
+    if (g.K > 64) return g.C >= 96 || (g.C >= 48 && 36.0 * (double)tiles4 * (g.C + g.K) * 4 <= 256e6);
+    const long patches = (g.P + GO_T - 1) / GO_T;                            // (one filter tile)
+    return g.C >= 96 && patches <= 256;
 }
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y, bool have_w) {
     // (a pooled layer of at most four channels: direct into scratch, then pooling -- the network's first layer shape with
     // pooling, N = 32: bf16 NCHW 59 + 31 us against 242 for the Winograd pipeline that pools in its output stage)
-    if (have_w && (direct_ok(dst, flags, g) || direct_pooled_ok(dst, flags, g))) return WINO_ALGO_DIRECT;
+    // (its workgroups take 128 pixels and every filter tile in turn: with fewer workgroups than CUs and many filters the
+    // Winograd pipelines spread the work better -- N = 1, C = 3, K = 256, H = 112: 45 against 24 us; K = 96: a tie)
+    const bool few_wide = (long)g.N * g.Ho * g.Wo < 128L * device_cus() && g.K >= 192;
+    if (have_w && !few_wide && (direct_ok(dst, flags, g) || direct_pooled_ok(dst, flags, g))) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x, y)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct_few(src, dtype, flags, g)) return WINO_ALGO_DIRECT;
     if (have_w && auto_f4(dtype, g)) return WINO_ALGO_STAGED_F4;

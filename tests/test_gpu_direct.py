@@ -133,19 +133,22 @@ def test_what_the_path_is_not_built_for():
 @pytest.mark.parametrize("dtype", [ops.F32, ops.BF16])
 def test_direct_with_the_largest_filter_bank_that_fits_lds(oracle, dtype):
     """K = 544 at C = 3: 17 filter tiles, 63 KB of LDS in fp32 (the few-channel kernel is offered up to 64 KB); K = 576
-    no longer fits: a 2-byte layer goes back to the Winograd kernels, an fp32 one this small to the small-layer
-    kernel.  Integers: bit-exact either way."""
+    no longer fits: by name a 2-byte layer is refused, an fp32 one this small runs on the small-layer kernel.  The
+    automatic choice keeps a layer of 90 pixels and this many filters on the Winograd kernels (2-byte) or the
+    small-layer kernel (fp32).  Integers: bit-exact every way."""
     from gpu_util import dev, host
     N, C, H, W = 1, 3, 9, 10
-    for K, want_algo in ((544, ops.ALGO_DIRECT), (576, None)):
+    for K in (544, 576):
         x, w = synth.conv_inputs(N, C, K, H, W, seed=K, integer=True)
-        got_algo = ops.pick_algo(ops.NCHW, dtype, N, C, K, H, W)
-        if want_algo is None:
-            assert (got_algo != ops.ALGO_DIRECT) == (dtype != ops.F32)
+        want = oracle.direct_conv(x, w, 1)
+        assert (ops.pick_algo(ops.NCHW, dtype, N, C, K, H, W) == ops.ALGO_DIRECT) == (dtype == ops.F32)
+        assert np.array_equal(host(ops.conv(dev(x, dtype), dev(w, dtype), 1, ops.NCHW)), want)
+        if K == 544 or dtype == ops.F32:
+            assert np.array_equal(host(ops.conv(dev(x, dtype), dev(w, dtype), 1, ops.NCHW, algo=ops.ALGO_DIRECT)), want)
         else:
-            assert got_algo == want_algo
-        y = host(ops.conv(dev(x, dtype), dev(w, dtype), 1, ops.NCHW))
-        assert np.array_equal(y, oracle.direct_conv(x, w, 1))
+            with pytest.raises(_lib.WinoError) as e:
+                ops.conv(dev(x, dtype), dev(w, dtype), 1, ops.NCHW, algo=ops.ALGO_DIRECT)
+            assert e.value.code == -2
 
 
 FEW_SHAPES = [(1, 64, 64, 12, 16), (2, 7, 40, 6, 6), (1, 130, 70, 9, 11), (3, 36, 100, 13, 5), (1, 5, 33, 7, 20), (1, 8, 32, 3, 3), (2, 12, 30, 5, 9)]

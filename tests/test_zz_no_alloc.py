@@ -29,9 +29,10 @@ CASES = [(ops.F32, a) for a in ALGOS + [ops.ALGO_EPILOGUE_F4]] + [(ops.BF16, a) 
 @pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC, ops.CHWN])
 @pytest.mark.parametrize("dtype,algo", CASES)
 def test_two_calls_in_a_row_match_the_allocating_entry_point(oracle, dtype, algo, layout):
-    f4 = algo in (ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4)
     # first a layer that fills a good part of the buffer, then a smaller one with other channel and filter counts
     for (N, C, K, H) in [(4, 64, 96, 56), (1, 24, 40, 13)]:
+        resolved = ops.pick_algo(layout, dtype, N, C, K, H, H) if algo == ops.ALGO_AUTO else algo
+        f4 = resolved in (ops.ALGO_STAGED_F4, ops.ALGO_EPILOGUE_F4)      # (F(4x4) rounds where F(2x2) is exact)
         x, w = synth.conv_inputs(N, C, K, H, H, seed=900 + C, layout=layout, integer=True)
         bias = dev(synth.small_ints(K, seed=4, lo=-2, hi=2).astype(np.float32), dtype)
         got, want = both(dev(x, dtype), dev(w, dtype), bias, layout, algo, relu=True)
