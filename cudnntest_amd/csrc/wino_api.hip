@@ -1341,7 +1341,7 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     // tiles: 94 against 53 us -- so: a tile for every CU, or one filter tile, or a short reduction)
     if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 28 || g.Wo < 28) return false;
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
-    return tiles >= device_cus() || g.K <= D16_KT || g.C <= 128;
+    return tiles >= device_cus() || g.K <= D16_KT || g.C <= 64 || (g.C <= 128 && tiles >= 64);   // (N = 1, C = 128, K = 96, H = 56, 16 tiles: 30 against 21 us)
 }
 // Small fp32 layers go to the one-launch direct kernel while its cost stays small: a round of the chip costs a fixed
 // part (the first group's trip to memory, the sum over the waves, the stores) and a part per group of 32 channels.
@@ -1354,7 +1354,7 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
 // H = 56 (4, 1): 22.1 against 27.8.  With one element per load (C not a multiple of 4) the kernel takes about twice
 // as long per group: N = 2, C = K = 64, H = 56 (2, 2): 32 against 22; N = 1, C = K = 128, H = 22: 26 against 19.
 bool auto_direct_few(int src, int dtype, unsigned flags, const Geometry& g) {
-    if (!direct_few_ok(dtype, flags, g)) return false;
+    if (!direct_few_ok(dtype, flags, g) || g.C <= 4) return false;          // (at most four channels: the kernels above, or none)
     const long rounds = (direct_few_units(g) + device_cus() - 1) / device_cus(), groups = (g.C + 31) / 32;
     // (a sweep of 560 shapes, NCHW, against the fastest pipeline: at rounds x (1 + groups) = 12 the kernel takes 0.59 to
     // 0.98 of its time, at 14 and 16 with at most 64 filters 0.60 to 0.99; at 17 and more, or 15 with 128 filters, it loses)
@@ -1391,9 +1391,10 @@ bool auto_f4(int dtype, const Geometry& g) {
 int resolve_auto(int src, int dst, int dtype, unsigned flags, const Geometry& g, const void* x, const void* y, bool have_w) {
     // (a pooled layer of at most four channels: direct into scratch, then pooling -- the network's first layer shape with
     // pooling, N = 32: bf16 NCHW 59 + 31 us against 242 for the Winograd pipeline that pools in its output stage)
-    // (its workgroups take 128 pixels and every filter tile in turn: with fewer workgroups than CUs and many filters the
-    // Winograd pipelines spread the work better -- N = 1, C = 3, K = 256, H = 112: 45 against 24 us; K = 96: a tie)
-    const bool few_wide = (long)g.N * g.Ho * g.Wo < 128L * device_cus() && g.K >= 192;
+    // (its workgroups take 128 pixels and every filter tile in turn: with a workgroup for every other CU at most and many filters the
+    // Winograd pipelines spread the work better -- N = 1, C = 3, K = 256, H = 112: 45 against 24 us; N = 8, K = 128, H = 20: 28
+    // against 19; K = 96: a tie)
+    const bool few_wide = (long)g.N * g.Ho * g.Wo < 64L * device_cus() && g.K >= 128;
     if (have_w && !few_wide && (direct_ok(dst, flags, g) || direct_pooled_ok(dst, flags, g))) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct16(src, dst, dtype, flags, g, x, y)) return WINO_ALGO_DIRECT;
     if (have_w && auto_direct_few(src, dtype, flags, g)) return WINO_ALGO_DIRECT;
