@@ -1,9 +1,10 @@
 /*
  * wino_amd.h -- C ABI of the MI355X (gfx950) Winograd 3x3 convolution library: F(2x2,3x3) and F(4x4,3x3)
  * pipelines in fp32, F(2x2,3x3) with f16 / bf16 storage, and direct MFMA convolutions where those are faster.
- * What a caller of the whole-layer entry points gets under WINO_ALGO_AUTO: fp32 layers with C, K >= 128 run in
- * F(4x4,3x3), the reference's own tile size (relative L2 error against a direct convolution 3e-6 to 5e-6), other
- * fp32 layers in F(2x2,3x3) (about 1e-6), 2-byte layers in F(2x2,3x3) or directly (about 2e-3 bf16, 3e-4 f16).
+ * What a caller of the whole-layer entry points gets under WINO_ALGO_AUTO: fp32 layers with long reductions and
+ * more than one tile of 64 filters (C >= 96 or so, at least 512 tiles of 4x4 outputs) run in F(4x4,3x3), the
+ * reference's own tile size (relative L2 error against a direct convolution 3e-6 to 5e-6), other fp32 layers in
+ * F(2x2,3x3) or directly (about 1e-6), 2-byte layers in F(2x2,3x3) or directly (about 2e-3 bf16, 3e-4 f16).
  *
  * Every entry point takes plain device pointers and sizes; `stream` is a
  * hipStream_t passed as void* (NULL = the null stream).  Calls are asynchronous
@@ -67,9 +68,10 @@ typedef enum {
                                own tile size and matrices (wrapedConv_NCHW.cuh:836-855,879-899,1084-1101):
                                2.25 multiplies per output instead of 4, about four times the rounding error of
                                F(2x2) (3e-6 to 5e-6 relative L2 in fp32 on the VGG layers).  WINO_ALGO_AUTO takes it
-                               for fp32 layers with C, K >= 128 and at least 512 tiles when it is
-                               given the filter bank itself; transformed filters handed to this algorithm by
-                               name must come from wino_f4_filter_transform. */
+                               for fp32 layers with at least 512 tiles and either C, K >= 128, or K > 64 and
+                               C >= 96 (C >= 48 while its transformed tensors fit the 256 MB cache), or K <= 64,
+                               C >= 96 and few patches, when it is given the filter bank itself; transformed
+                               filters handed to this algorithm by name must come from wino_f4_filter_transform. */
     WINO_ALGO_DIRECT = 5,    /* no Winograd at all, the convolution itself on the matrix cores.  Three kinds of layer:
                                small fp32 layers -- at most four rounds of the chip in units of 4 x 8 pixels x 32
                                filters, e.g. the reference's sweep at batch 1 (comparison/layoutCompare.cu:38-46: N = 1,

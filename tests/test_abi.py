@@ -132,3 +132,10 @@ def test_bench_refuses_more_than_one_gpu_and_runs_nothing_without_one():
     if not torch.cuda.is_available():
         r = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True, text=True)
         assert r.returncode != 0 and "no GPU" in r.stderr
+
+
+def test_the_algorithm_sweep_tool_imports_without_a_gpu():
+    """python3 -m cudnntest_amd.algo_sweep needs a GPU to run; its grids and the algorithm table load without one."""
+    from cudnntest_amd import algo_sweep, ops
+    assert set(algo_sweep.GRIDS) == {"f32", "f16", "bf16"}
+    assert algo_sweep.ALGOS["f4"] == ops.ALGO_STAGED_F4 and algo_sweep.ALGOS["direct"] == ops.ALGO_DIRECT
