@@ -1341,7 +1341,8 @@ bool auto_direct16(int src, int dst, int dtype, unsigned flags, const Geometry& 
     // tiles: 94 against 53 us -- so: a tile for every CU, or one filter tile, or a short reduction)
     if (src == WINO_NHWC || dst == WINO_NHWC || g.Ho < 28 || g.Wo < 28) return false;
     const long tiles = ((long)g.N * g.Ho + 15) / 16 * ((g.Wo + 31) / 32) * ((g.K + D16_KT - 1) / D16_KT);
-    return tiles >= device_cus() || g.K <= D16_KT || g.C <= 64 || (g.C <= 128 && tiles >= 64);   // (N = 1, C = 128, K = 96, H = 56, 16 tiles: 30 against 21 us)
+    // (N = 1, C = 128, K = 96, H = 56, 16 tiles: 30 against 21 us; N = 1, C = 512, K = 64, 8 tiles: 44 against 29)
+    return tiles >= device_cus() || (g.K <= D16_KT && (tiles >= 32 || g.C <= 128)) || g.C <= 64 || (g.C <= 128 && tiles >= 64);
 }
 // Small fp32 layers go to the one-launch direct kernel while its cost stays small: a round of the chip costs a fixed
 // part (the first group's trip to memory, the sum over the waves, the stores) and a part per group of 32 channels.
