@@ -1360,7 +1360,12 @@ bool auto_direct_few(int src, int dtype, unsigned flags, const Geometry& g) {
     // (a sweep of 560 shapes, NCHW, against the fastest pipeline: at rounds x (1 + groups) = 12 the kernel takes 0.59 to
     // 0.98 of its time, at 14 and 16 with at most 64 filters 0.60 to 0.99; at 17 and more, or 15 with 128 filters, it loses)
     const long cost = rounds * (1 + groups);
-    return direct_few_filter_mode(src, g) ? cost <= 12 || (cost <= 16 && g.K <= 64) : rounds * groups <= 2;
+    // (one tile of 32 filters: up to 34 -- N = 64, C = 512, K = 16, H = 14: 66 against 94 us -- with 1.07 the worst ratio.
+    // The two wider offers hold for NCHW tensors only: from NHWC and CHWN the kernel is slower and F(4x4) wins there --
+    // NHWC, N = 4, C = 96, K = 64, H = 56, cost 16: 35 against 28 us; CHWN, N = 32, C = 192, K = 32, H = 28, cost 28: 72 against 51)
+    const int mode = direct_few_filter_mode(src, g);
+    if (mode == 0) return rounds * groups <= 2;
+    return cost <= 12 || (mode == 1 && ((cost <= 16 && g.K <= 64) || (cost <= 34 && g.K <= 32)));
 }
 // fp32 layers with a long reduction and enough 4x4 tiles run faster through the F(4x4,3x3) pipeline, product tensor
 // and all: 2.25 multiplies per output instead of 4, and a transformed input of 2.25x the tensor instead of 4x.
