@@ -1474,13 +1474,20 @@ int direct_pooled_images(const ScratchSource& ss, int src, int dst, int dtype, c
 }
 
 // What the automatic choice runs when its first choice does not fit a fixed scratch buffer: a pooled CHWN layer and a
-// pooled layer of at most four channels on the direct path keep the unpooled tensor in scratch; without room for it the
-// Winograd pipelines take the layer.
+// pooled layer of at most four channels on the direct path keep the unpooled tensor in scratch, the F(4x4) pipeline its
+// transformed input and product; without room for them the F(2x2) pipelines take the layer, the single kernel last.
 int auto_within(const ScratchSource& ss, int algo, int src, int dst, int dtype, unsigned flags, const Geometry& g) {
-    if (algo == WINO_ALGO_DIRECT && ss.fixed &&
-        ((direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
-          kCounterBytes + (direct16_bank_bytes(g) + 255) / 256 * 256 + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) ||
-         (direct_pooled_ok(dst, flags, g) && direct_pooled_images(ss, src, dst, dtype, g) == 0))) {
+    if (!ss.fixed) return algo;
+    bool refit = false;
+    if (algo == WINO_ALGO_DIRECT)
+        refit = (direct16_chwn_pool_ok(src, dst, dtype, flags, g) &&
+                 kCounterBytes + (direct16_bank_bytes(g) + 255) / 256 * 256 + direct16_unpooled_bytes(dtype, g) > ss.fixed_bytes) ||
+                (direct_pooled_ok(dst, flags, g) && direct_pooled_images(ss, src, dst, dtype, g) == 0);
+    if (algo == WINO_ALGO_STAGED_F4) {                                        // (V and the product of the 36 coordinates)
+        Geometry g4;
+        refit = !make_geometry(dtype, g.N, g.C, g.K, g.H, g.W, g.pad, &g4, 4) || scratch_layout(g4, dtype, algo).total > ss.fixed_bytes;
+    }
+    if (refit) {
         algo = pick_algo(src, dtype, g);
         // (the single kernel keeps only the transformed filters in scratch: it runs where the others' tensors do not fit)
         if (algo != WINO_ALGO_FUSED && g.pad <= 1 && scratch_layout(g, dtype, algo).total > ss.fixed_bytes &&

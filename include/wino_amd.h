@@ -179,7 +179,9 @@ int wino_conv_prepared_ex(int src, int dst, int dtype, int algo, unsigned flags,
  * process ends, instead of the arena.  The call makes no hipMalloc / hipFree and creates no events (stage timing
  * does not see it).  A problem whose pipeline needs more scratch than the buffer holds is refused with
  * WINO_ERR_WORKSPACE and a message giving both sizes: ask for WINO_ALGO_FUSED (keeps only the transformed
- * filters, 16*Cp*Kp elements) or WINO_ALGO_DIRECT, or use a smaller batch.  The first call on a device looks the
+ * filters, 16*Cp*Kp elements) or WINO_ALGO_DIRECT, or use a smaller batch.  Under WINO_ALGO_AUTO a first choice that
+ * keeps large tensors in scratch (F(4x4); a direct kernel that pools through scratch) gives way to one that fits: the
+ * pooled first layer in smaller passes, the F(2x2) pipelines, the single kernel last.  The first call on a device looks the
  * buffer's address up (wino_warmup() does the same ahead of time); nothing is cleared: the buffer is a
  * zero-initialised object of the device image, and the kernels that count arrivals in it leave their counters at zero.  Every call on a GPU shares that GPU's buffer: calls that overlap
  * on one GPU (two streams, two threads) race, exactly as whole-layer calls sharing the arena do.

@@ -115,3 +115,16 @@ def test_pooled_first_layers_with_and_without_room_for_the_unpooled_tensor(oracl
         assert (N * K * H * H * 2 > LIMIT) == (H == 160)
         assert torch.equal(got, want), H
 
+
+
+def test_the_automatic_choice_stays_inside_the_buffer(oracle):
+    """fp32, N = 8, C = 512, K = 64, 56 x 56: the automatic choice is F(4x4), whose transformed input and product take 130 MB;
+    inside the 64 MB buffer the call runs the single Winograd kernel instead (2 MB of transformed filters) -- the same bits
+    as that kernel by name."""
+    N, C, K, H = 8, 512, 64, 56
+    x, w = synth.conv_inputs(N, C, K, H, H, seed=5)
+    xd, wd = dev(x), dev(w)
+    assert ops.pick_algo(ops.NCHW, ops.F32, N, C, K, H, H) == ops.ALGO_STAGED_F4
+    out = torch.empty((N, K, H, H), device="cuda")
+    ops.conv_noalloc(xd, wd, out, 1, ops.NCHW, algo=ops.ALGO_AUTO)
+    assert torch.equal(out, ops.conv(xd, wd, 1, ops.NCHW, algo=ops.ALGO_FUSED))
