@@ -75,3 +75,27 @@ def test_first_layer_with_byte_offsets_past_2_31(oracle, Nl):
     assert all(torch.equal(y[i:i + 16], y2[i:i + 16]) for i in range(0, Nl, 16))
     del x, y, y2, shifted
     torch.cuda.empty_cache()
+
+
+def test_first_layer_from_nhwc_with_byte_offsets_past_2_31(oracle):
+    """The same for the NHWC tiles: 334 images, y of 4.29 GB; the last image against the oracle, the whole tensor
+    against the gathering kernel (an element-aligned view of x)."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * 2 ** 30:
+        pytest.skip("needs 16 GB of free device memory")
+    Nl = 334
+    g = torch.Generator(device="cuda").manual_seed(8)
+    xn = torch.rand((Nl, 3, 224, 224), device="cuda", generator=g) * 2 - 1
+    wn = torch.randn((64, 3, 3, 3), device="cuda", generator=g) * 0.2
+    x, w = xn.permute(0, 2, 3, 1).contiguous(), wn.permute(0, 2, 3, 1).contiguous()
+    y = ops.conv(x, w, 1, ops.NHWC, algo=ops.ALGO_DIRECT)
+    want = oracle.direct_conv_f32(host(xn[Nl - 1:]), host(wn), 1)
+    assert oracle.rel_l2(host(y[Nl - 1:].permute(0, 3, 1, 2).contiguous()), want) <= 1e-6
+    del xn
+    shifted = torch.empty(x.numel() + 1, dtype=x.dtype, device="cuda")[1:].view(x.shape)
+    shifted.copy_(x)
+    y2 = ops.conv(shifted, w, 1, ops.NHWC, algo=ops.ALGO_DIRECT)
+    assert all(torch.equal(y[i:i + 16], y2[i:i + 16]) for i in range(0, Nl, 16))
+    del x, y, y2, shifted
+    torch.cuda.empty_cache()
+
