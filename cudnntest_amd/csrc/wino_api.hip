@@ -1389,6 +1389,9 @@ bool auto_f4(int dtype, const Geometry& g) {
     if (dtype != WINO_F32) return false;
     const long tiles4 = (long)g.N * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4);
     if (tiles4 < 512) return false;
+    // (14 x 14 images fill 16 x 16 outputs of 4x4 tiles, 1.31 times the work: below C = 192 the F(2x2) pipelines keep such
+    // layers -- N = 64, C = K = 128, H = 14: 45 against 42 us; C = 64, K = 128: 39 against 34)
+    if (16L * ((g.Ho + 3) / 4) * ((g.Wo + 3) / 4) * 4 > 5L * g.Ho * g.Wo && g.C < 192) return false;
     if (g.C >= 128 && g.K >= 128) return true;
     if (g.K > 64) return g.C >= 96 || (g.C >= 48 && 36.0 * (double)tiles4 * (g.C + g.K) * 4 <= 256e6);
     const long patches = (g.P + GO_T - 1) / GO_T;                            // (one filter tile)
