@@ -1,6 +1,6 @@
 """Times every pipeline by name against the automatic choice over a grid of layer shapes, through the C ABI.
 
-    python3 -m cudnntest_amd.algo_sweep --dtype f32 --layout NCHW [--pool] [--quick]
+    python3 -m cudnntest_amd.algo_sweep --dtype f32 --layout NCHW [--dst NHWC] [--pool] [--quick]
 
 One line per shape (microseconds, median of event-timed calls issued one after the other) and a summary: the sum of
 the automatic choice's times, the sum of the fastest pipeline's, and the geometric mean of their ratio.  The rules
@@ -48,6 +48,7 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--dtype", choices=sorted(GRIDS), default="f32")
     ap.add_argument("--layout", choices=sorted(LAYOUTS), default="NCHW")
+    ap.add_argument("--dst", choices=sorted(LAYOUTS), default=None, help="layout of y (default: that of x)")
     ap.add_argument("--pool", action="store_true", help="bias, ReLU and 2x2 pooling in the output stage")
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="every third shape of the grid")
@@ -56,6 +57,7 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("algo_sweep needs a GPU")
     lay, tdt = LAYOUTS[args.layout], TORCH[args.dtype]
+    dst = LAYOUTS[args.dst or args.layout]
     Cs, Ks, NHs = GRIDS[args.dtype]
     shapes = [(N, C, K, H) for (N, H), C, K in itertools.product(NHs, Cs, Ks)
               if 2.0 * N * C * K * H * H * 9 <= args.max_gflop * 1e9 and N * max(C, K) * H * H * 4 <= 6e8]
@@ -71,17 +73,17 @@ def main():
         if lay == ops.CHWN:
             x, w = x.permute(1, 2, 3, 0).contiguous(), w.permute(1, 2, 3, 0).contiguous()
         kw = dict(relu=True, bias=b, pool=True) if args.pool else {}
-        y = ops.conv(x, w, 1, lay, **kw)
+        y = ops.conv(x, w, 1, lay, dst, **kw)
         times = {}
         for name, algo in ALGOS.items():
             if name == "f4" and args.dtype != "f32":
                 continue
             try:
-                ops.conv(x, w, 1, lay, out=y, algo=algo, **kw)
+                ops.conv(x, w, 1, lay, dst, out=y, algo=algo, **kw)
             except _lib.WinoError:          # the pipeline is not built for this shape
                 continue
-            times[name] = timed(lambda: ops.conv(x, w, 1, lay, out=y, algo=algo, **kw), args.steps)
-        auto = timed(lambda: ops.conv(x, w, 1, lay, out=y, **kw), args.steps)
+            times[name] = timed(lambda: ops.conv(x, w, 1, lay, dst, out=y, algo=algo, **kw), args.steps)
+        auto = timed(lambda: ops.conv(x, w, 1, lay, dst, out=y, **kw), args.steps)
         best = min(times, key=times.get)
         log_sum += math.log(auto / times[best])
         auto_sum += auto
@@ -89,7 +91,7 @@ def main():
         print(f"N{N} C{C} K{K} H{H}: auto {auto:.1f} best {best} {times[best]:.1f} x{auto / times[best]:.2f} | "
               + " ".join(f"{k}={v:.1f}" for k, v in times.items()), flush=True)
     n = max(len(shapes), 1)
-    print(f"{len(shapes)} shapes, {args.dtype} {args.layout}{' pooled' if args.pool else ''}: automatic choice {auto_sum / 1e3:.2f} ms in all, "
+    print(f"{len(shapes)} shapes, {args.dtype} {args.layout}{' -> ' + args.dst if args.dst else ''}{' pooled' if args.pool else ''}: automatic choice {auto_sum / 1e3:.2f} ms in all, "
           f"fastest by name {best_sum / 1e3:.2f} ms, geometric mean of the ratio {math.exp(log_sum / n):.3f}")
 
 
